@@ -1,0 +1,371 @@
+"""The cache manager: pages of keys and values with a block table per request, in groups of
+layers with the same needs, and slots for per-request state of fixed size.
+
+After simply/utils/ragged_paged_attention.py: `DecodeState` keeps a page pool, a free stack and
+`page_indices` per layer (:142-173); `allocate` (:475-518) pops pages from the front of the free
+stack, `release` (:521-541) and `release_for_window` (:437-472) push pages back at its end; layers
+with the same (pages, page size, window) share the bookkeeping (:865-917).  Differences: the
+bookkeeping lives on the host, a block table is indexed by the absolute block number of a key
+(position // page_size) so that a windowed group leaves holes instead of shifting its table, and
+running out of pages is reported to the caller instead of being excluded by construction.
+
+Bookkeeping is separate from storage: `CacheManager(device=None)` keeps no tensors and runs
+anywhere.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+from typing import Hashable, Sequence
+
+import numpy as np
+import torch
+
+from ..parts.base import PagedKVNeed, StateNeed
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+class OutOfPages(CacheError):
+    """Raised by `reserve` when a group cannot hold the tokens; nothing has been changed."""
+
+
+def ceil_div(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+class PagePool:
+    """Free pages of one group, handed out from the front and taken back at the end
+    (simply/utils/ragged_paged_attention.py:495-511, 530-535)."""
+
+    def __init__(self, num_pages: int):
+        self.num_pages = int(num_pages)
+        self._free = collections.deque(range(self.num_pages))
+        self._is_free = np.ones(self.num_pages, dtype=bool)
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def free_list(self) -> list[int]:
+        return list(self._free)
+
+    def take(self, n: int) -> list[int]:
+        if n > len(self._free):
+            raise OutOfPages(f"{n} pages wanted, {len(self._free)} free")
+        out = [self._free.popleft() for _ in range(n)]
+        self._is_free[out] = False
+        return out
+
+    def give_back(self, pages: Sequence[int]) -> None:
+        for p in pages:
+            if not 0 <= p < self.num_pages:
+                raise CacheError(f"page {p} does not exist")
+            if self._is_free[p]:
+                raise CacheError(f"page {p} freed twice")
+            self._is_free[p] = True
+            self._free.append(p)
+
+
+@dataclasses.dataclass
+class _Sequence:
+    slot: int
+    num_tokens: int = 0       # tokens whose keys have a place (prompt and generated)
+    first_block: int = 0      # blocks below this one have been given back (windowed groups)
+
+
+class CacheGroup:
+    """Pages and block tables of the layers that share one `PagedKVNeed`."""
+
+    def __init__(self, group_id: int, need: PagedKVNeed, page_size: int, num_pages: int, num_slots: int,
+                 max_blocks_per_seq: int):
+        self.group_id, self.need = group_id, need
+        self.page_size, self.num_slots, self.max_blocks = int(page_size), int(num_slots), int(max_blocks_per_seq)
+        self.pool = PagePool(num_pages)
+        #: table[slot, absolute block] = page, -1 where no page is held
+        self.table = np.full((self.num_slots, self.max_blocks), -1, dtype=np.int32)
+        self.seqs: dict[Hashable, _Sequence] = {}
+        self.dirty_slots: set[int] = set()
+
+    # -- what a step would need
+    def dead_blocks(self, num_computed: int) -> int:
+        """Blocks that no query at position >= num_computed can see (windowed groups only):
+        the first visible key is num_computed - window + 1
+        (simply/utils/ragged_paged_attention.py:441-445 with window_size = window - 1)."""
+        if self.need.window is None:
+            return 0
+        return max(num_computed - self.need.window + 1, 0) // self.page_size
+
+    def pages_needed(self, rid: Hashable, num_computed: int, q_len: int) -> int:
+        """New pages for tokens [num_computed, num_computed + q_len), net of those that become free first."""
+        s = self.seqs[rid]
+        have_to = ceil_div(s.num_tokens, self.page_size)
+        need_to = ceil_div(num_computed + q_len, self.page_size)
+        released = max(min(self.dead_blocks(num_computed), have_to) - s.first_block, 0)
+        return max(need_to - have_to, 0) - released
+
+    # -- changes
+    def add(self, rid: Hashable, slot: int) -> None:
+        if rid in self.seqs:
+            raise CacheError(f"request {rid!r} is already in group {self.group_id}")
+        self.seqs[rid] = _Sequence(slot)
+
+    def release_window(self, rid: Hashable, num_computed: int) -> list[int]:
+        s = self.seqs[rid]
+        dead = min(self.dead_blocks(num_computed), ceil_div(s.num_tokens, self.page_size))
+        if dead <= s.first_block:
+            return []
+        pages = [int(p) for p in self.table[s.slot, s.first_block:dead]]
+        self.table[s.slot, s.first_block:dead] = -1
+        s.first_block = dead
+        self.pool.give_back(pages)
+        self.dirty_slots.add(s.slot)
+        return pages
+
+    def extend(self, rid: Hashable, new_num_tokens: int) -> list[int]:
+        s = self.seqs[rid]
+        have_to = ceil_div(s.num_tokens, self.page_size)
+        need_to = ceil_div(new_num_tokens, self.page_size)
+        if need_to > self.max_blocks:
+            raise CacheError(f"request {rid!r}: {new_num_tokens} tokens need {need_to} blocks, the table has "
+                             f"{self.max_blocks}")
+        pages = self.pool.take(max(need_to - have_to, 0))
+        if pages:
+            self.table[s.slot, have_to:need_to] = pages
+            self.dirty_slots.add(s.slot)
+        s.num_tokens = max(s.num_tokens, new_num_tokens)
+        return pages
+
+    def remove(self, rid: Hashable) -> list[int]:
+        s = self.seqs.pop(rid)
+        row = self.table[s.slot]
+        pages = [int(p) for p in row[row >= 0]]
+        row[:] = -1
+        self.pool.give_back(pages)
+        self.dirty_slots.add(s.slot)
+        return pages
+
+    def pages_of(self, rid: Hashable) -> list[int]:
+        s = self.seqs[rid]
+        row = self.table[s.slot]
+        return [int(p) for p in row[row >= 0]]
+
+    def check(self) -> None:
+        """Invariants: every page is free or held by exactly one request, never both or twice."""
+        held = self.table[self.table >= 0]
+        if len(np.unique(held)) != len(held):
+            raise CacheError(f"group {self.group_id}: a page is held twice")
+        free = self.pool.free_list()
+        if len(set(free)) != len(free):
+            raise CacheError(f"group {self.group_id}: a page is in the free list twice")
+        if set(free) & set(int(p) for p in held):
+            raise CacheError(f"group {self.group_id}: a page is both free and held")
+        if len(free) + len(held) != self.pool.num_pages:
+            raise CacheError(f"group {self.group_id}: {self.pool.num_pages - len(free) - len(held)} pages lost")
+        live_slots = {s.slot for s in self.seqs.values()}
+        for slot in range(self.num_slots):
+            if slot not in live_slots and (self.table[slot] >= 0).any():
+                raise CacheError(f"group {self.group_id}: slot {slot} has pages but no request")
+
+
+class StateSlots:
+    """Slots for per-request state of fixed size; the slot also selects the request's block-table row
+    (the batch slot of simply/utils/ragged_paged_attention.py:1448-1462)."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = int(num_slots)
+        self._free = list(range(self.num_slots - 1, -1, -1))
+        self.owner: dict[int, Hashable] = {}
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def take(self, rid: Hashable) -> int:
+        if not self._free:
+            raise CacheError("no free state slot")
+        slot = self._free.pop()
+        self.owner[slot] = rid
+        return slot
+
+    def give_back(self, slot: int) -> None:
+        if slot not in self.owner:
+            raise CacheError(f"state slot {slot} freed twice")
+        del self.owner[slot]
+        self._free.append(slot)
+        self._free.sort(reverse=True)
+
+
+@dataclasses.dataclass
+class CacheView:
+    """What one schedule entry's mixer is handed: its own storage (or that of the entry it reads)."""
+
+    need: PagedKVNeed | StateNeed | None
+    group_id: int | None = None
+    k_pages: torch.Tensor | None = None   # [num_pages, kv heads, page_size, head_dim]
+    v_pages: torch.Tensor | None = None
+    state: torch.Tensor | None = None     # [num_slots, *need.shape]
+    write: bool = True                    # False: this entry reads the cache of another entry
+
+
+class CacheManager:
+    """All groups, the state slots and (if `device` is given) the storage.
+
+    needs: one `(need, cache_from)` per schedule entry, as `DecoderModel.cache_needs()` returns.
+    """
+
+    def __init__(self, needs, *, page_size: int, num_pages: int, num_slots: int, max_seq_len: int,
+                 dtype: torch.dtype = torch.float32, device=None, poison: bool = False):
+        self.page_size, self.num_pages, self.num_slots = int(page_size), int(num_pages), int(num_slots)
+        self.max_seq_len, self.dtype, self.device, self.poison = int(max_seq_len), dtype, device, bool(poison)
+        self.slots = StateSlots(num_slots)
+        self.groups: list[CacheGroup] = []
+        self.requests: dict[Hashable, int] = {}
+        self.views: list[CacheView] = []
+        self._group_entries: dict[int, list[int]] = {}
+        self._device_tables: dict[int, torch.Tensor] = {}
+        by_need: dict[PagedKVNeed, CacheGroup] = {}
+        max_blocks = ceil_div(self.max_seq_len, self.page_size)
+        for i, (need, cache_from) in enumerate(needs):
+            if cache_from is not None:
+                src = self.views[cache_from]
+                if type(src.need) is not type(need) or src.need != need:
+                    raise CacheError(f"schedule entry {i} reads the cache of entry {cache_from}, whose need differs: "
+                                     f"{need} vs {src.need}")
+                self.views.append(dataclasses.replace(src, write=False))
+                continue
+            if need is None:
+                self.views.append(CacheView(None))
+            elif isinstance(need, PagedKVNeed):
+                group = by_need.get(need)
+                if group is None:
+                    group = CacheGroup(len(self.groups), need, self.page_size, self.num_pages, self.num_slots, max_blocks)
+                    by_need[need] = group
+                    self.groups.append(group)
+                    self._group_entries[group.group_id] = []
+                view = CacheView(need, group.group_id)
+                if device is not None:
+                    shape = (self.num_pages, need.num_kv_heads, self.page_size, need.head_dim)
+                    fill = float("nan") if poison else 0.0
+                    view.k_pages = torch.full(shape, fill, dtype=dtype, device=device)
+                    view.v_pages = torch.full(shape, fill, dtype=dtype, device=device)
+                self._group_entries[group.group_id].append(i)
+                self.views.append(view)
+            elif isinstance(need, StateNeed):
+                view = CacheView(need)
+                if device is not None:
+                    view.state = torch.zeros((self.num_slots, *need.shape), dtype=need.dtype, device=device)
+                self.views.append(view)
+            else:
+                raise CacheError(f"schedule entry {i}: unknown cache need {need!r}")
+        if device is not None:
+            for g in self.groups:
+                self._device_tables[g.group_id] = torch.full((self.num_slots, g.max_blocks), -1, dtype=torch.int32,
+                                                             device=device)
+
+    # ------------------------------------------------------------------ requests
+    def has_slot(self) -> bool:
+        return self.slots.num_free > 0
+
+    def admit(self, rid: Hashable) -> int:
+        """Takes a state slot and an empty block-table row in every group; zeroes the request's state."""
+        if rid in self.requests:
+            raise CacheError(f"request {rid!r} is already admitted")
+        slot = self.slots.take(rid)
+        self.requests[rid] = slot
+        for g in self.groups:
+            g.add(rid, slot)
+        for v in self.views:
+            if v.state is not None and v.write:
+                v.state[slot].zero_()
+        return slot
+
+    def slot_of(self, rid: Hashable) -> int:
+        return self.requests[rid]
+
+    def pages_needed(self, rid: Hashable, num_computed: int, q_len: int) -> dict[int, int]:
+        return {g.group_id: g.pages_needed(rid, num_computed, q_len) for g in self.groups}
+
+    def can_reserve(self, wants: Sequence[tuple[Hashable, int, int]]) -> bool:
+        """Whether every group can hold all of `wants` = (request, num_computed, q_len) together."""
+        for g in self.groups:
+            if sum(g.pages_needed(rid, nc, q) for rid, nc, q in wants) > g.pool.num_free:
+                return False
+        return True
+
+    def reserve(self, rid: Hashable, num_computed: int, q_len: int) -> None:
+        """Makes room for tokens [num_computed, num_computed + q_len) in every group: first gives back
+        the pages that the window has passed, then takes new ones.  Raises OutOfPages, with nothing
+        changed, if any group is short."""
+        if num_computed + q_len > self.max_seq_len:
+            raise CacheError(f"request {rid!r}: {num_computed + q_len} tokens exceed max_seq_len {self.max_seq_len}")
+        for g in self.groups:
+            short = g.pages_needed(rid, num_computed, q_len) - g.pool.num_free
+            if short > 0:
+                raise OutOfPages(f"group {g.group_id} (window {g.need.window}): {short} pages short for request "
+                                 f"{rid!r}")
+        for g in self.groups:
+            self._poison(g, g.release_window(rid, num_computed))
+            g.extend(rid, num_computed + q_len)
+
+    def free(self, rid: Hashable) -> None:
+        """Gives back everything the request holds."""
+        slot = self.requests.pop(rid)
+        for g in self.groups:
+            self._poison(g, g.remove(rid))
+        self.slots.give_back(slot)
+
+    def _poison(self, g: CacheGroup, pages: Sequence[int]) -> None:
+        """Fills pages that were just given back with NaN (in stream order: after the steps that read
+        them, before the step that writes them again), so that a read of an unwritten key shows."""
+        if not (self.poison and self.device is not None and pages):
+            return
+        idx = torch.as_tensor(list(pages), dtype=torch.long, device=self.device)
+        for e in self._group_entries[g.group_id]:
+            self.views[e].k_pages[idx] = float("nan")
+            self.views[e].v_pages[idx] = float("nan")
+
+    def check(self) -> None:
+        for g in self.groups:
+            g.check()
+            if set(g.seqs) != set(self.requests):
+                raise CacheError(f"group {g.group_id} and the manager disagree on the live requests")
+        if set(self.slots.owner.values()) != set(self.requests):
+            raise CacheError("state slots and the manager disagree on the live requests")
+
+    # ------------------------------------------------------------------ what a step reads
+    def slot_mapping(self, group_id: int, rid: Hashable, start: int, q_len: int) -> np.ndarray:
+        """Storage slot (page * page_size + offset) of positions [start, start + q_len)."""
+        g = self.groups[group_id]
+        pos = np.arange(start, start + q_len, dtype=np.int64)
+        pages = g.table[g.seqs[rid].slot, pos // g.page_size].astype(np.int64)
+        if (pages < 0).any():
+            raise CacheError(f"request {rid!r}: a position in [{start}, {start + q_len}) has no page in group {group_id}")
+        return pages * g.page_size + pos % g.page_size
+
+    def check_readable(self, group_id: int, rid: Hashable, start: int, q_len: int) -> None:
+        """Every key that the queries at [start, start + q_len) may read has a page."""
+        g = self.groups[group_id]
+        lo = 0 if g.need.window is None else max(start - g.need.window + 1, 0)
+        blocks = g.table[g.seqs[rid].slot, lo // g.page_size: ceil_div(start + q_len, g.page_size)]
+        if (blocks < 0).any():
+            raise CacheError(f"request {rid!r}: keys [{lo}, {start + q_len}) are not all held in group {group_id}")
+
+    def sync_tables(self) -> dict[int, torch.Tensor]:
+        """Brings the device copies of the block tables up to date."""
+        for g in self.groups:
+            if self.device is not None and g.dirty_slots:
+                dev = self._device_tables[g.group_id]
+                rows = sorted(g.dirty_slots)
+                idx = torch.as_tensor(rows, dtype=torch.long)
+                dev.index_copy_(0, idx.to(self.device), torch.from_numpy(g.table[rows]).to(self.device))
+            g.dirty_slots.clear()
+        return self._device_tables
+
+    def bytes_per_token(self) -> int:
+        """Bytes of cache that one token takes over all schedule entries that keep their own."""
+        esize = torch.empty((), dtype=self.dtype).element_size()
+        return sum(2 * v.need.num_kv_heads * v.need.head_dim * esize for v in self.views
+                   if isinstance(v.need, PagedKVNeed) and v.write)

@@ -1,0 +1,75 @@
+// C interface of the gfx950 kernel library.  Every entry point returns 0 on
+// success; otherwise sa_last_error() describes the refusal (a size the kernels
+// do not take, an unknown element type, a failed launch).  Pointers are device
+// pointers unless a comment says otherwise; `stream` is the HIP stream to
+// launch on.  Element type codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+
+const char* sa_last_error();
+int sa_version();
+
+// out[t, :] = table[tokens[t], :] * scale (32-bit output: the residual stream).
+int sa_embed(const void* table, int table_dtype, const int* tokens, float* out, int T, int D, int V, float scale,
+             hipStream_t stream);
+
+// out = x * rsqrt(mean(x^2) + eps) * (w + plus_one), row by row.
+int sa_rmsnorm(const void* x, int x_dtype, int64_t x_stride, const void* w, int w_dtype, void* out, int out_dtype,
+               int64_t out_stride, int T, int D, float eps, int plus_one, hipStream_t stream);
+
+// residual += norm(y; w_post) (w_post null: residual += y); then, if w_next is not null,
+// out = norm(residual; w_next).
+int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, int w_post_dtype, float eps_post,
+                   int plus_one_post, float* residual, const void* w_next, int w_next_dtype, float eps_next,
+                   int plus_one_next, void* out, int out_dtype, int T, int D, hipStream_t stream);
+
+// Fused projection rows [T, (H + 2K) * hd]: rotate q and k (timescale null: no rotation), divide q by
+// q_div, write k and v into the pages at slot_mapping[t] = page * page_size + offset (k_pages null: no write).
+int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, const int* positions, const float* timescale,
+                        float scale_factor, float q_div, const int64_t* slot_mapping, void* k_pages, void* v_pages,
+                        int T, int H, int K, int hd, int page_size, hipStream_t stream);
+
+// Rotation alone, in place, then division by div.
+int sa_rope(void* x, int dtype, int64_t row_stride, const int* positions, const float* timescale, float scale_factor,
+            float div, int T, int n_heads, int hd, hipStream_t stream);
+
+int sa_gather_rows(const void* x, int x_dtype, const int* index, void* out, int out_dtype, int R, int D,
+                   hipStream_t stream);
+
+int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t stream);
+
+// C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1: gelu_tanh(A.W^T) * (A.W2^T);
+// 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel.
+int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C, int c_dtype,
+            int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, hipStream_t stream);
+
+// Attention of T query tokens over paged keys and values.
+//   q[t, h, :] at q + t * q_stride + h * hd; pages are [num_pages, Kh, page_size, hd];
+//   token_seq[t] is the row of block_table of the token's request, positions[t] its absolute position;
+//   window 0: all earlier keys, else the last `window` keys including the token's own; soft_cap 0: none.
+// algo 0: the library chooses; 1: the generic kernel.
+int sa_paged_attention(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
+                       const int* block_table, int table_stride, const int* token_seq, const int* positions, void* out,
+                       int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window, float soft_cap,
+                       int algo, hipStream_t stream);
+
+// One token per row of 32-bit logits.  temperature 0 or top_k 1: argmax.  top_k <= 0 and top_p >= 1: off.
+int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature, const int* top_k,
+              const float* top_p, const uint64_t* seed, const int* counter, int* tokens, float* logprobs,
+              hipStream_t stream);
+
+// Host function: one block of the Philox4x32-10 generator that sa_sample uses.
+void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* out4);
+}
+
+namespace sa {
+int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
+                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, hipStream_t stream);
+int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
+                            const int* block_table, int table_stride, const int* token_seq, const int* positions,
+                            void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
+                            float soft_cap, hipStream_t stream);
+}  // namespace sa

@@ -1,0 +1,90 @@
+// Shared helpers of the gfx950 kernels: element types, conversions, wave
+// reductions and the error channel of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sa {
+
+// Element type codes used across the C interface.
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+struct bf16 {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float to_float(bf16 x) {
+  union { uint32_t u; float f; } c;
+  c.u = static_cast<uint32_t>(x.bits) << 16;
+  return c.f;
+}
+__host__ __device__ inline float to_float(float x) { return x; }
+
+// Round to nearest even; NaN stays NaN.
+__host__ __device__ inline bf16 float_to_bf16(float f) {
+  union { uint32_t u; float f; } c;
+  c.f = f;
+  uint32_t u = c.u;
+  bf16 r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
+    return r;
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  r.bits = static_cast<uint16_t>(u >> 16);
+  return r;
+}
+
+template <typename T> __host__ __device__ inline T from_float(float f);
+template <> __host__ __device__ inline float from_float<float>(float f) { return f; }
+template <> __host__ __device__ inline bf16 from_float<bf16>(float f) { return float_to_bf16(f); }
+
+// Loads and stores through a runtime element type (uniform over a launch).
+__device__ inline float load_f(const void* p, int dtype, size_t i) {
+  return dtype == kF32 ? static_cast<const float*>(p)[i] : to_float(static_cast<const bf16*>(p)[i]);
+}
+__device__ inline void store_f(void* p, int dtype, size_t i, float v) {
+  if (dtype == kF32) static_cast<float*>(p)[i] = v;
+  else static_cast<bf16*>(p)[i] = float_to_bf16(v);
+}
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  The
+// order of additions depends only on the block size, never on the data.
+__device__ inline float block_sum(float v, float* scratch /* >= 16 floats */) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int nwaves = (blockDim.x + kWave - 1) / kWave;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+
+// Error channel: entry points return 0 on success, non-zero after set_error().
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+}  // namespace sa
+
+#define SA_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      sa::set_error(__VA_ARGS__);        \
+      return 1;                          \
+    }                                    \
+  } while (0)

@@ -1,0 +1,265 @@
+// Row-wise kernels: embedding lookup, RMSNorm (alone and fused with the residual
+// sum and the next norm), rotary encoding fused with the cache write, row gather.
+// All statistics, angles and the residual sum are in 32-bit whatever the
+// activation type is.
+#include "api.h"
+#include "common.h"
+
+namespace sa {
+
+// ------------------------------------------------------------------ embedding
+// out[t, :] = float(table[tokens[t], :]) * scale.   simply/utils/module.py:450-481
+__global__ void embed_kernel(const void* __restrict__ table, int table_dtype, const int* __restrict__ tokens,
+                             float* __restrict__ out, int D, int V, float scale) {
+  const int t = blockIdx.x;
+  int tok = tokens[t];
+  tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);  // the host has already refused ids outside the table
+  const size_t base = static_cast<size_t>(tok) * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x)
+    out[static_cast<size_t>(t) * D + d] = load_f(table, table_dtype, base + d) * scale;
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// y = x * rsqrt(mean(x^2) + eps) * (w + plus_one).   simply/model_lib.py:154-178
+__global__ void rmsnorm_kernel(const void* __restrict__ x, int x_dtype, int64_t x_stride,
+                               const void* __restrict__ w, int w_dtype, void* __restrict__ out, int out_dtype,
+                               int64_t out_stride, int D, float eps, float plus_one) {
+  __shared__ float scratch[16];
+  const size_t xb = static_cast<size_t>(blockIdx.x) * x_stride, ob = static_cast<size_t>(blockIdx.x) * out_stride;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float v = load_f(x, x_dtype, xb + d);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float r = rsqrtf(ss / static_cast<float>(D) + eps);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float v = load_f(x, x_dtype, xb + d) * r;
+    store_f(out, out_dtype, ob + d, v * (load_f(w, w_dtype, d) + plus_one));
+  }
+}
+
+// residual[t, :] += norm(y[t, :]; w_post);  then, if w_next: out[t, :] = norm(residual[t, :]; w_next).
+// The residual stream is 32-bit.  simply/model_lib.py:2681-2683 and :2690.
+__global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, const void* __restrict__ w_post,
+                                   int w_post_dtype, float eps_post, float plus_one_post, float* __restrict__ residual,
+                                   const void* __restrict__ w_next, int w_next_dtype, float eps_next,
+                                   float plus_one_next, void* __restrict__ out, int out_dtype, int D) {
+  __shared__ float scratch[16];
+  const size_t rb = static_cast<size_t>(blockIdx.x) * D;
+  float ss = 0.f;
+  if (w_post != nullptr) {
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+      const float v = load_f(y, y_dtype, rb + d);
+      ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+  }
+  const float r = w_post != nullptr ? rsqrtf(ss / static_cast<float>(D) + eps_post) : 1.f;
+  float ss2 = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float v = load_f(y, y_dtype, rb + d);
+    if (w_post != nullptr) v = v * r * (load_f(w_post, w_post_dtype, d) + plus_one_post);
+    const float h = residual[rb + d] + v;
+    residual[rb + d] = h;  // re-read below by the same thread only
+    ss2 += h * h;
+  }
+  if (w_next == nullptr) return;
+  ss2 = block_sum(ss2, scratch);
+  const float r2 = rsqrtf(ss2 / static_cast<float>(D) + eps_next);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float h = residual[rb + d] * r2;
+    store_f(out, out_dtype, rb + d, h * (load_f(w_next, w_next_dtype, d) + plus_one_next));
+  }
+}
+
+// ------------------------------------------------------------------ rotary + cache write
+// One block per (token, head) of a fused [T, (H + 2K) * hd] projection.
+//   q heads: rotate, divide by query_scale, write back in place.
+//   k heads: rotate, write into the key pages at slot_mapping[t].
+//   v heads: copy into the value pages.
+// Angles: pos / timescale[i] / scale_factor, pairs (i, i + hd/2).  simply/utils/position_encoding.py:83-110;
+// the query scale comes after the rotation (simply/model_lib.py:2010-2019).
+template <typename T>
+__global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions,
+                                        const float* __restrict__ timescale /* [hd/2] or null = no rotation */,
+                                        float inv_scale_factor, float q_div, const int64_t* __restrict__ slot_mapping,
+                                        T* __restrict__ k_pages, T* __restrict__ v_pages, int H, int K, int hd,
+                                        int page_size) {
+  const int t = blockIdx.x, head = blockIdx.y;
+  const int half = hd / 2;
+  T* src = qkv + static_cast<size_t>(t) * row_stride + static_cast<size_t>(head) * hd;
+  const float pos = static_cast<float>(positions[t]);
+  if (head < H + K) {
+    const bool is_q = head < H;
+    T* dst = src;
+    if (!is_q) {
+      if (k_pages == nullptr) return;
+      const int64_t slot = slot_mapping[t];
+      if (slot < 0) return;
+      const int64_t page = slot / page_size, off = slot % page_size;
+      dst = k_pages + ((page * K + (head - H)) * page_size + off) * hd;
+    }
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      const float x1 = to_float(src[i]), x2 = to_float(src[i + half]);
+      float o1 = x1, o2 = x2;
+      if (timescale != nullptr) {
+        const float angle = pos / timescale[i] * inv_scale_factor;
+        float s, c;
+        sincosf(angle, &s, &c);
+        o1 = x1 * c - x2 * s;
+        o2 = x2 * c + x1 * s;
+      }
+      if (is_q) {
+        o1 = o1 / q_div;
+        o2 = o2 / q_div;
+      }
+      dst[i] = from_float<T>(o1);
+      dst[i + half] = from_float<T>(o2);
+    }
+  } else {
+    if (v_pages == nullptr) return;
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) return;
+    const int64_t page = slot / page_size, off = slot % page_size;
+    T* dst = v_pages + ((page * K + (head - H - K)) * page_size + off) * hd;
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+  }
+}
+
+// Rotation alone, in place, on [T, n_heads, hd] rows of stride row_stride.
+template <typename T>
+__global__ void rope_kernel(T* __restrict__ x, int64_t row_stride, const int* __restrict__ positions,
+                            const float* __restrict__ timescale, float inv_scale_factor, float div, int hd) {
+  const int t = blockIdx.x, head = blockIdx.y, half = hd / 2;
+  T* p = x + static_cast<size_t>(t) * row_stride + static_cast<size_t>(head) * hd;
+  const float pos = static_cast<float>(positions[t]);
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float x1 = to_float(p[i]), x2 = to_float(p[i + half]);
+    const float angle = pos / timescale[i] * inv_scale_factor;
+    float s, c;
+    sincosf(angle, &s, &c);
+    p[i] = from_float<T>((x1 * c - x2 * s) / div);
+    p[i + half] = from_float<T>((x2 * c + x1 * s) / div);
+  }
+}
+
+// out[r, :] = x[index[r], :]
+__global__ void gather_rows_kernel(const void* __restrict__ x, int x_dtype, const int* __restrict__ index,
+                                   void* __restrict__ out, int out_dtype, int D) {
+  const size_t src = static_cast<size_t>(index[blockIdx.x]) * D, dst = static_cast<size_t>(blockIdx.x) * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) store_f(out, out_dtype, dst + d, load_f(x, x_dtype, src + d));
+}
+
+// p[i] = value for i < n (32-bit words); stands in for a memset inside captured graphs.
+__global__ void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t value, int64_t n) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    p[i] = value;
+}
+
+static int row_threads(int D) {
+  int t = 64;
+  while (t < 1024 && t * 4 < D) t *= 2;
+  return t;
+}
+
+}  // namespace sa
+
+using namespace sa;
+
+extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, float* out, int T, int D, int V,
+                        float scale, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(table_dtype == kF32 || table_dtype == kBF16, "embed: unknown table dtype %d", table_dtype);
+  SA_REQUIRE(T > 0 && D > 0 && V > 0, "embed: bad sizes T=%d D=%d V=%d", T, D, V);
+  embed_kernel<<<T, row_threads(D), 0, stream>>>(table, table_dtype, tokens, out, D, V, scale);
+  return check_launch("embed");
+}
+
+extern "C" int sa_rmsnorm(const void* x, int x_dtype, int64_t x_stride, const void* w, int w_dtype, void* out,
+                          int out_dtype, int64_t out_stride, int T, int D, float eps, int plus_one,
+                          hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && D > 0, "rmsnorm: bad sizes T=%d D=%d", T, D);
+  SA_REQUIRE(x_stride >= D && out_stride >= D, "rmsnorm: row strides %lld, %lld are below the width %d",
+             (long long)x_stride, (long long)out_stride, D);
+  rmsnorm_kernel<<<T, row_threads(D), 0, stream>>>(x, x_dtype, x_stride, w, w_dtype, out, out_dtype, out_stride, D,
+                                                   eps, plus_one ? 1.f : 0.f);
+  return check_launch("rmsnorm");
+}
+
+extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, int w_post_dtype, float eps_post,
+                              int plus_one_post, float* residual, const void* w_next, int w_next_dtype,
+                              float eps_next, int plus_one_next, void* out, int out_dtype, int T, int D,
+                              hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && D > 0, "add_rmsnorm: bad sizes T=%d D=%d", T, D);
+  SA_REQUIRE(w_next == nullptr || out != nullptr, "add_rmsnorm: a next norm needs an output");
+  add_rmsnorm_kernel<<<T, row_threads(D), 0, stream>>>(y, y_dtype, w_post, w_post_dtype, eps_post,
+                                                       plus_one_post ? 1.f : 0.f, residual, w_next, w_next_dtype,
+                                                       eps_next, plus_one_next ? 1.f : 0.f, out, out_dtype, D);
+  return check_launch("add_rmsnorm");
+}
+
+extern "C" int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, const int* positions,
+                                   const float* timescale, float scale_factor, float q_div,
+                                   const int64_t* slot_mapping, void* k_pages, void* v_pages, int T, int H, int K,
+                                   int hd, int page_size, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(hd > 0 && hd % 2 == 0, "rope_cache_write: head size %d must be even", hd);
+  SA_REQUIRE(H >= 0 && K >= 0 && H + 2 * K > 0, "rope_cache_write: bad head counts H=%d K=%d", H, K);
+  SA_REQUIRE(row_stride >= static_cast<int64_t>(H + 2 * K) * hd, "rope_cache_write: row stride %lld is too small",
+             (long long)row_stride);
+  SA_REQUIRE(page_size > 0 && scale_factor > 0.f && q_div > 0.f, "rope_cache_write: bad page size, scale factor or query scale");
+  SA_REQUIRE((k_pages == nullptr) == (v_pages == nullptr) && (k_pages == nullptr || slot_mapping != nullptr),
+             "rope_cache_write: key pages, value pages and slots come together");
+  const dim3 grid(T, H + 2 * K);
+  const int threads = hd / 2 >= 128 ? 128 : 64;
+  if (dtype == kF32)
+    rope_cache_write_kernel<float><<<grid, threads, 0, stream>>>(static_cast<float*>(qkv), row_stride, positions,
+                                                                 timescale, 1.f / scale_factor, q_div, slot_mapping,
+                                                                 static_cast<float*>(k_pages),
+                                                                 static_cast<float*>(v_pages), H, K, hd, page_size);
+  else if (dtype == kBF16)
+    rope_cache_write_kernel<bf16><<<grid, threads, 0, stream>>>(static_cast<bf16*>(qkv), row_stride, positions,
+                                                                timescale, 1.f / scale_factor, q_div, slot_mapping,
+                                                                static_cast<bf16*>(k_pages),
+                                                                static_cast<bf16*>(v_pages), H, K, hd, page_size);
+  else
+    SA_REQUIRE(false, "rope_cache_write: unknown dtype %d", dtype);
+  return check_launch("rope_cache_write");
+}
+
+extern "C" int sa_rope(void* x, int dtype, int64_t row_stride, const int* positions, const float* timescale,
+                       float scale_factor, float div, int T, int n_heads, int hd, hipStream_t stream) {
+  if (T == 0 || n_heads == 0) return 0;
+  SA_REQUIRE(hd > 0 && hd % 2 == 0, "rope: head size %d must be even", hd);
+  SA_REQUIRE(timescale != nullptr && scale_factor > 0.f && div > 0.f, "rope: no timescales, or a bad scale");
+  const dim3 grid(T, n_heads);
+  const int threads = hd / 2 >= 128 ? 128 : 64;
+  if (dtype == kF32)
+    rope_kernel<float><<<grid, threads, 0, stream>>>(static_cast<float*>(x), row_stride, positions, timescale,
+                                                     1.f / scale_factor, div, hd);
+  else if (dtype == kBF16)
+    rope_kernel<bf16><<<grid, threads, 0, stream>>>(static_cast<bf16*>(x), row_stride, positions, timescale,
+                                                    1.f / scale_factor, div, hd);
+  else
+    SA_REQUIRE(false, "rope: unknown dtype %d", dtype);
+  return check_launch("rope");
+}
+
+extern "C" int sa_gather_rows(const void* x, int x_dtype, const int* index, void* out, int out_dtype, int R, int D,
+                              hipStream_t stream) {
+  if (R == 0) return 0;
+  gather_rows_kernel<<<R, row_threads(D), 0, stream>>>(x, x_dtype, index, out, out_dtype, D);
+  return check_launch("gather_rows");
+}
+
+extern "C" int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  const int64_t blocks = (n + 255) / 256;
+  fill_u32_kernel<<<static_cast<int>(blocks > 4096 ? 4096 : blocks), 256, 0, stream>>>(static_cast<uint32_t*>(p),
+                                                                                      value, n);
+  return check_launch("fill_u32");
+}

@@ -1,0 +1,236 @@
+// Sampling from rows of 32-bit logits: greedy, temperature, top-k and top-p, one
+// workgroup per row.
+//
+// simply/utils/sampling_lib.py:472-537: temperature == 0 or top_k == 1 is argmax
+// with log-probability 0; otherwise the logits are divided by the temperature,
+// masked by top-k and/or top-p (kept entries: simply/utils/sampling_lib.py:427-469)
+// and a token is drawn from the categorical distribution, which
+// jax.random.categorical does with the Gumbel-max trick; the log-probability is
+// log_softmax(masked scaled logits)[token] (simply/utils/distributions.py:98-121).
+//
+// Random numbers are counter-based (Philox4x32-10) and keyed by the row's own
+// seed and draw counter, so a request's tokens do not depend on which other
+// requests share the batch.
+#include "api.h"
+#include "common.h"
+
+namespace sa {
+
+constexpr int kSampleThreads = 1024;
+
+struct Philox4 {
+  uint32_t v[4];
+};
+
+__host__ __device__ inline Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                                 uint32_t k1) {
+  const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = static_cast<uint64_t>(M0) * c0, p1 = static_cast<uint64_t>(M1) * c2;
+    const uint32_t hi0 = static_cast<uint32_t>(p0 >> 32), lo0 = static_cast<uint32_t>(p0);
+    const uint32_t hi1 = static_cast<uint32_t>(p1 >> 32), lo1 = static_cast<uint32_t>(p1);
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += W0; k1 += W1;
+  }
+  Philox4 o;
+  o.v[0] = c0; o.v[1] = c1; o.v[2] = c2; o.v[3] = c3;
+  return o;
+}
+
+// Standard Gumbel noise for vocabulary entry `index` of draw `counter` under `seed`.
+__device__ inline float gumbel_noise(uint64_t seed, uint32_t counter, uint32_t index) {
+  const Philox4 r = philox4x32_10(index >> 2, counter, 0u, 0u, static_cast<uint32_t>(seed),
+                                  static_cast<uint32_t>(seed >> 32));
+  const float u = (static_cast<float>(r.v[index & 3u] >> 8) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+  return -logf(-logf(u));
+}
+
+// Maps a float to an unsigned key with the same order.
+__device__ inline uint32_t ordered_key(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ inline float key_to_float(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+struct ArgMax {
+  float v;
+  int i;
+};
+__device__ inline ArgMax better(ArgMax a, ArgMax b) {
+  // larger value wins, the lower index on ties (jnp.argmax returns the first maximum)
+  return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+__device__ inline ArgMax block_argmax(ArgMax a, ArgMax* scratch) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    ArgMax b;
+    b.v = __shfl_xor(a.v, o, kWave);
+    b.i = __shfl_xor(a.i, o, kWave);
+    a = better(a, b);
+  }
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, nw = blockDim.x / kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = a;
+  __syncthreads();
+  ArgMax r = scratch[0];
+  for (int w = 1; w < nw; ++w) r = better(r, scratch[w]);
+  return r;
+}
+__device__ inline float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, nw = blockDim.x / kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float r = scratch[0];
+  for (int w = 1; w < nw; ++w) r = fmaxf(r, scratch[w]);
+  return r;
+}
+
+// Finds, among the entries x (scaled logits) of one row that are >= `floor_key`, the
+// key of the boundary entry, by radix selection from the most significant byte down:
+//   by_mass == 0: the `target_count`-th largest entry;
+//   by_mass == 1: the entry at which the mass exp(x - max) summed from the top first
+//                 reaches `target_mass` (so the mass strictly above it is below it).
+// Masses are accumulated as 64-bit fixed point so that the result does not depend on
+// the order in which threads add.  Returns the key; all threads get it.
+__device__ uint32_t radix_select(const float* __restrict__ row, int V, float inv_t, float max_scaled, int by_mass,
+                                 uint64_t target, uint32_t floor_key, unsigned long long* hist /* [256] LDS */,
+                                 uint32_t* shared_out /* [2] LDS */, unsigned long long* shared_above /* [1] LDS */) {
+  uint32_t prefix = 0, prefix_mask = 0;
+  unsigned long long above = 0;  // count or mass of entries whose key is above the current prefix range
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0ull;
+    __syncthreads();
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      const float x = row[i] * inv_t;
+      const uint32_t key = ordered_key(x);
+      if (key < floor_key || (key & prefix_mask) != prefix) continue;
+      unsigned long long w = 1ull;
+      if (by_mass) w = static_cast<unsigned long long>(expf(x - max_scaled) * 4294967296.0f);
+      atomicAdd(&hist[(key >> shift) & 0xffu], w);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      unsigned long long run = above;
+      int chosen = 0;
+      for (int b = 255; b >= 0; --b) {
+        if (run + hist[b] >= target) {
+          chosen = b;
+          break;
+        }
+        run += hist[b];
+        if (b == 0) chosen = 0;  // target beyond the total: take everything
+      }
+      shared_out[0] = static_cast<uint32_t>(chosen);
+      *shared_above = run;
+    }
+    __syncthreads();
+    prefix |= shared_out[0] << shift;
+    prefix_mask |= 0xffu << shift;
+    above = *shared_above;
+    __syncthreads();
+  }
+  return prefix;
+}
+
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(
+    const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const uint64_t* __restrict__ seed,
+    const int* __restrict__ counter, int* __restrict__ tokens, float* __restrict__ logprobs) {
+  __shared__ ArgMax am_scratch[kSampleThreads / kWave];
+  __shared__ float f_scratch[kSampleThreads / kWave];
+  __shared__ unsigned long long hist[256];
+  __shared__ uint32_t sel_out[2];
+  __shared__ unsigned long long sel_above;
+  const int r = blockIdx.x;
+  const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const float temp = temperature[r];
+  const int k = top_k[r];
+  const float p = top_p[r];
+
+  if (temp == 0.f || k == 1) {
+    ArgMax a{-INFINITY, 0x7fffffff};
+    for (int i = threadIdx.x; i < V; i += blockDim.x) a = better(a, ArgMax{row[i], i});
+    a = block_argmax(a, am_scratch);
+    if (threadIdx.x == 0) {
+      tokens[r] = a.i;
+      logprobs[r] = 0.f;
+    }
+    return;
+  }
+
+  const float inv_t = 1.f / temp;
+  float mx = -INFINITY;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
+  mx = block_max(mx, f_scratch);
+
+  // Entries whose key is >= floor_key stay (the mask of the reference, as a threshold).
+  uint32_t floor_key = 0u;
+  if (k > 0) {
+    const uint64_t kk = static_cast<uint64_t>(k < V ? k : V);
+    floor_key = radix_select(row, V, inv_t, mx, 0, kk, 0u, hist, sel_out, &sel_above);
+  }
+  if (p < 1.f) {
+    // total mass of the entries that are still in (after top-k, whose softmax is renormalised over them)
+    __syncthreads();
+    if (threadIdx.x == 0) hist[0] = 0ull;
+    __syncthreads();
+    unsigned long long local = 0ull;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      const float x = row[i] * inv_t;
+      if (ordered_key(x) >= floor_key) local += static_cast<unsigned long long>(expf(x - mx) * 4294967296.0f);
+    }
+    atomicAdd(&hist[0], local);
+    __syncthreads();
+    const unsigned long long total = hist[0];
+    __syncthreads();
+    // keep while the mass before an entry is < p * total: the boundary entry is the first at which the
+    // running mass reaches p * total (it is kept, simply/utils/sampling_lib.py:434-441)
+    unsigned long long target = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(total));
+    if (target < 1ull) target = 1ull;
+    const uint32_t p_key = radix_select(row, V, inv_t, mx, 1, target, floor_key, hist, sel_out, &sel_above);
+    floor_key = p_key > floor_key ? p_key : floor_key;
+  }
+
+  const uint64_t sd = seed[r];
+  const uint32_t ctr = static_cast<uint32_t>(counter[r]);
+  ArgMax a{-INFINITY, 0x7fffffff};
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+    const float x = row[i] * inv_t;
+    if (ordered_key(x) < floor_key) continue;
+    sum += expf(x - mx);
+    a = better(a, ArgMax{x + gumbel_noise(sd, ctr, static_cast<uint32_t>(i)), i});
+  }
+  a = block_argmax(a, am_scratch);
+  sum = block_sum(sum, f_scratch);
+  if (threadIdx.x == 0) {
+    tokens[r] = a.i;
+    logprobs[r] = row[a.i] * inv_t - mx - logf(sum);
+  }
+}
+
+}  // namespace sa
+
+using namespace sa;
+
+extern "C" int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature,
+                         const int* top_k, const float* top_p, const uint64_t* seed, const int* counter, int* tokens,
+                         float* logprobs, hipStream_t stream) {
+  if (R == 0) return 0;
+  SA_REQUIRE(R > 0 && V > 0 && row_stride >= V, "sample: bad sizes R=%d V=%d stride=%lld", R, V,
+             (long long)row_stride);
+  sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed, counter,
+                                                  tokens, logprobs);
+  return check_launch("sample");
+}
+
+// Host-side copy of the generator, for tests of the kernel's random stream.
+extern "C" void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* out4) {
+  const Philox4 r = philox4x32_10(counter4[0], counter4[1], counter4[2], counter4[3], key2[0], key2[1]);
+  for (int i = 0; i < 4; ++i) out4[i] = r.v[i];
+}

@@ -1,0 +1,43 @@
+"""What every part is told about the step it runs in.
+
+The batch is ragged: T tokens of S requests laid end to end, a portion of a prompt beside single
+decoded tokens (simply/utils/ragged_paged_attention.py:1992-2019 builds the same flat batch, with
+segment ids and absolute segment positions).  The description is independent of the kind of mixer.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Hashable
+
+import torch
+
+
+@dataclasses.dataclass
+class GroupStep:
+    """Per cache group: where this step's tokens are stored and where each request's pages are."""
+
+    block_table: torch.Tensor   # int32 [num_slots, max_blocks]: row = request's slot, column = position // page_size
+    slot_mapping: torch.Tensor  # int64 [T]: page * page_size + offset of each token of the step
+
+
+@dataclasses.dataclass
+class StepContext:
+    dtype: torch.dtype            # activation dtype
+    num_tokens: int
+    positions: torch.Tensor       # int32 [T] absolute position of each token in its request
+    token_seq: torch.Tensor       # int32 [T] slot of each token's request (block-table row, state row)
+    groups: dict[int, GroupStep]
+    # host-side description, in the order of the tokens
+    request_ids: list[Hashable]
+    seq_slots: list[int]          # slot of each request
+    seq_starts: list[int]         # tokens of the request that earlier steps have run
+    q_lens: list[int]             # tokens of the request in this step
+    cu_q_lens: list[int]          # [S + 1] offsets of the requests in the flat batch
+
+    @property
+    def num_seqs(self) -> int:
+        return len(self.q_lens)
+
+    @property
+    def max_q_len(self) -> int:
+        return max(self.q_lens) if self.q_lens else 0

@@ -1,0 +1,140 @@
+"""The step function: one ragged batch through the model, from the cache.
+
+`Executor.step` takes, for each request, its next tokens and the places among them whose logits
+are wanted; it runs only those tokens, as one batch, and returns float32 logits at the wanted
+places.  It corresponds to the forward half of `SamplingState.mixed_step`
+(simply/utils/ragged_paged_attention.py:1954-2019); choosing which tokens to run is the
+scheduler's job and sampling is the sampler's.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Hashable, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+from ..config import EngineConfig
+from ..models import DecoderModel
+from .context import GroupStep, StepContext
+
+
+@dataclasses.dataclass
+class StepEntry:
+    request_id: Hashable
+    tokens: Sequence[int]                 # the request's next tokens
+    want: Sequence[int] = ()              # places among `tokens` whose logits are wanted
+
+
+class Executor:
+    def __init__(self, model: DecoderModel, config: EngineConfig, *, num_pages: int | None = None):
+        config.validate()
+        if not model.loaded:
+            raise RuntimeError("the model has no weights yet")
+        self.model, self.config = model, config
+        self.device = torch.device(config.device)
+        self.dtype = config.dtype
+        pages = num_pages if num_pages is not None else config.total_num_pages
+        if pages is None:
+            pages = config.batch_size * -(-config.max_seq_len // config.page_size)
+        self.cache = CacheManager(model.cache_needs(), page_size=config.page_size, num_pages=pages,
+                                  num_slots=config.batch_size, max_seq_len=config.max_seq_len, dtype=self.dtype,
+                                  device=self.device, poison=config.poison_freed_pages)
+        self.num_computed: dict[Hashable, int] = {}
+        self.vocab_size = model.spec.vocab_size
+        # one pinned staging buffer and one device buffer for all of a step's integers
+        cap = max(config.issue_budget, config.batch_size)
+        self._cap = cap
+        ngroups = len(self.cache.groups)
+        self._words = cap * (4 + 2 * ngroups)
+        self._on_gpu = self.device.type == "cuda"
+        self._host = torch.empty(self._words, dtype=torch.int32, pin_memory=self._on_gpu)
+        self._dev = torch.empty(self._words, dtype=torch.int32, device=self.device)
+        self._copied = torch.cuda.Event() if self._on_gpu else None
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, rid: Hashable) -> int:
+        slot = self.cache.admit(rid)
+        self.num_computed[rid] = 0
+        return slot
+
+    def finish_request(self, rid: Hashable) -> None:
+        self.cache.free(rid)
+        del self.num_computed[rid]
+
+    def has_request(self, rid: Hashable) -> bool:
+        return rid in self.num_computed
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+        """Runs the entries as one batch.  Returns float32 logits [wanted, vocab] in the order of the
+        entries and of their `want`, or None if nothing is wanted."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        T = sum(len(e.tokens) for e in entries)
+        if T == 0:
+            return None
+        if T > self._cap:
+            raise ValueError(f"a step of {T} tokens exceeds max_num_issue_tokens {self._cap}")
+        seen = set()
+        for e in entries:
+            if e.request_id in seen:
+                raise ValueError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            if e.request_id not in self.num_computed:
+                raise KeyError(f"request {e.request_id!r} has not been added")
+        cache, cap = self.cache, self._cap
+        # make room for every entry first: a failure leaves earlier steps' state untouched only if nothing
+        # has been reserved, so check all of them together before changing anything
+        wants = [(e.request_id, self.num_computed[e.request_id], len(e.tokens)) for e in entries]
+        if not cache.can_reserve(wants):
+            from ..cache import OutOfPages
+
+            raise OutOfPages("the cache cannot hold this step's tokens: " + ", ".join(
+                f"{rid!r}+{q}" for rid, _, q in wants))
+        for rid, start, q in wants:
+            cache.reserve(rid, start, q)
+
+        if self._copied is not None:
+            self._copied.synchronize()  # the last step's copy out of the staging buffer has finished
+        host = self._host.numpy()
+        tok, pos, seq, rows = (host[i * cap:(i + 1) * cap] for i in range(4))
+        slot_maps = [host[(4 + 2 * g) * cap:(6 + 2 * g) * cap].view(np.int64) for g in range(len(cache.groups))]
+        ctx_ids, ctx_slots, ctx_starts, ctx_q, cu = [], [], [], [], [0]
+        R = 0
+        t0 = 0
+        for e, (rid, start, q) in zip(entries, wants):
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if ids.min() < 0 or ids.max() >= self.vocab_size:
+                raise ValueError(f"request {rid!r}: token id outside [0, {self.vocab_size})")
+            slot = cache.slot_of(rid)
+            tok[t0:t0 + q] = ids
+            pos[t0:t0 + q] = np.arange(start, start + q)
+            seq[t0:t0 + q] = slot
+            for g in cache.groups:
+                slot_maps[g.group_id][t0:t0 + q] = cache.slot_mapping(g.group_id, rid, start, q)
+                cache.check_readable(g.group_id, rid, start, q)
+            for w in e.want:
+                if not 0 <= w < q:
+                    raise ValueError(f"request {rid!r}: wanted place {w} is outside its {q} tokens")
+                rows[R] = t0 + w
+                R += 1
+            ctx_ids.append(rid); ctx_slots.append(slot); ctx_starts.append(start); ctx_q.append(q)
+            t0 += q
+            cu.append(t0)
+        tables = cache.sync_tables()
+        self._dev.copy_(self._host, non_blocking=True)
+        if self._copied is not None:
+            self._copied.record()
+        dev = self._dev
+        groups = {g.group_id: GroupStep(tables[g.group_id],
+                                        dev[(4 + 2 * g.group_id) * cap:(6 + 2 * g.group_id) * cap].view(torch.int64)[:T])
+                  for g in cache.groups}
+        ctx = StepContext(dtype=self.dtype, num_tokens=T, positions=dev[cap:cap + T], token_seq=dev[2 * cap:2 * cap + T],
+                          groups=groups, request_ids=ctx_ids, seq_slots=ctx_slots, seq_starts=ctx_starts, q_lens=ctx_q,
+                          cu_q_lens=cu)
+        logit_rows = dev[3 * cap:3 * cap + R] if R else None
+        logits = self.model.forward(dev[:T], ctx, cache.views, logit_rows)
+        for rid, start, q in wants:
+            self.num_computed[rid] = start + q
+        return logits

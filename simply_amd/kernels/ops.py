@@ -1,0 +1,298 @@
+"""Tensor-level calls of the gfx950 kernels.
+
+Each function checks on the host that shapes, element types, strides and devices
+are what the kernel assumes, then launches on torch's current stream.  Nothing
+here computes on the CPU and nothing falls back to a library routine.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import lib as _lib
+from .lib import KernelError
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+ALGO_AUTO, ALGO_GENERIC = 0, 1
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"element type {t.dtype} is not supported by the kernels (float32, bfloat16)") from None
+
+
+def _dev(*tensors) -> None:
+    first = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError("the kernels run on the GPU only: a tensor lies on " + str(t.device))
+        if first is None:
+            first = t.device
+        elif t.device != first:
+            raise KernelError(f"tensors lie on different devices: {first} and {t.device}")
+
+
+def _ptr(t: torch.Tensor | None):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _rows(t: torch.Tensor, what: str) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{what}: expected a 2-D tensor with contiguous rows, got shape {tuple(t.shape)} "
+                          f"strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _i32(t: torch.Tensor, what: str, n: int | None = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{what}: expected a contiguous int32 tensor, got {t.dtype}")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{what}: {t.numel()} entries, {n} needed")
+
+
+# --------------------------------------------------------------------------- row-wise
+
+
+def embed(table: torch.Tensor, tokens: torch.Tensor, scale: float, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = float32(table[tokens[t]]) * scale."""
+    _dev(table, tokens, out)
+    V, D = table.shape
+    T = tokens.numel()
+    _i32(tokens, "embed: tokens")
+    if not table.is_contiguous():
+        raise KernelError("embed: the table must be contiguous")
+    if out is None:
+        out = torch.empty((T, D), dtype=torch.float32, device=table.device)
+    if out.dtype != torch.float32 or not out.is_contiguous() or tuple(out.shape) != (T, D):
+        raise KernelError("embed: the output must be a contiguous float32 [T, D] tensor")
+    _lib.call("sa_embed", _ptr(table), _code(table), _ptr(tokens), _ptr(out), T, D, V, float(scale), _stream())
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, plus_one: bool, out_dtype: torch.dtype,
+            out: torch.Tensor | None = None) -> torch.Tensor:
+    _dev(x, weight, out)
+    xs = _rows(x, "rmsnorm: x")
+    T, D = x.shape
+    if weight.numel() != D or not weight.is_contiguous():
+        raise KernelError(f"rmsnorm: weight has {weight.numel()} entries for width {D}")
+    if out is None:
+        out = torch.empty((T, D), dtype=out_dtype, device=x.device)
+    if tuple(out.shape) != (T, D):
+        raise KernelError("rmsnorm: output shape differs from the input's")
+    os_ = _rows(out, "rmsnorm: out")
+    _lib.call("sa_rmsnorm", _ptr(x), _code(x), xs, _ptr(weight), _code(weight), _ptr(out), _code(out), os_, T, D,
+              float(eps), int(plus_one), _stream())
+    return out
+
+
+def add_rmsnorm(y: torch.Tensor, residual: torch.Tensor, *, post_weight: torch.Tensor | None = None,
+                post_eps: float = 0.0, post_plus_one: bool = True, next_weight: torch.Tensor | None = None,
+                next_eps: float = 0.0, next_plus_one: bool = True, out_dtype: torch.dtype | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor | None:
+    """residual += norm(y; post_weight) (or += y); returns norm(residual; next_weight) if asked."""
+    _dev(y, residual, post_weight, next_weight, out)
+    T, D = residual.shape
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("add_rmsnorm: the residual stream must be contiguous float32")
+    if tuple(y.shape) != (T, D) or not y.is_contiguous():
+        raise KernelError(f"add_rmsnorm: y {tuple(y.shape)} does not match the residual {T, D}")
+    for w in (post_weight, next_weight):
+        if w is not None and (w.numel() != D or not w.is_contiguous()):
+            raise KernelError("add_rmsnorm: a norm weight does not match the width")
+    if next_weight is not None:
+        if out is None:
+            out = torch.empty((T, D), dtype=out_dtype or y.dtype, device=y.device)
+        if tuple(out.shape) != (T, D) or not out.is_contiguous():
+            raise KernelError("add_rmsnorm: bad output")
+    else:
+        out = None
+    _lib.call("sa_add_rmsnorm", _ptr(y), _code(y), _ptr(post_weight),
+              _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one),
+              _ptr(residual), _ptr(next_weight), _code(next_weight) if next_weight is not None else 0,
+              float(next_eps), int(next_plus_one), _ptr(out), _code(out) if out is not None else 0, T, D, _stream())
+    return out
+
+
+def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, timescale: torch.Tensor | None, scale_factor: float,
+                     q_div: float, num_heads: int, num_kv_heads: int, head_dim: int,
+                     slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
+                     v_pages: torch.Tensor | None = None) -> None:
+    """In place on the fused projection rows; writes keys and values into their pages."""
+    _dev(qkv, positions, timescale, slot_mapping, k_pages, v_pages)
+    stride = _rows(qkv, "rope_cache_write: qkv")
+    T = qkv.shape[0]
+    if qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
+        raise KernelError(f"rope_cache_write: row width {qkv.shape[1]} is not (H + 2K) * hd = "
+                          f"{(num_heads + 2 * num_kv_heads) * head_dim}")
+    _i32(positions, "rope_cache_write: positions", T)
+    if timescale is not None and (timescale.dtype != torch.float32 or timescale.numel() != head_dim // 2
+                                  or not timescale.is_contiguous()):
+        raise KernelError("rope_cache_write: timescale must be float32 [head_dim / 2]")
+    page_size = 1
+    if k_pages is not None:
+        if v_pages is None or slot_mapping is None:
+            raise KernelError("rope_cache_write: key pages, value pages and slots come together")
+        for p in (k_pages, v_pages):
+            if p.dim() != 4 or p.shape[1] != num_kv_heads or p.shape[3] != head_dim or not p.is_contiguous() \
+                    or p.dtype != qkv.dtype or p.shape != k_pages.shape:
+                raise KernelError(f"rope_cache_write: pages must be contiguous [pages, {num_kv_heads}, page_size, "
+                                  f"{head_dim}] of {qkv.dtype}, got {tuple(p.shape)} {p.dtype}")
+        page_size = k_pages.shape[2]
+        if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
+            raise KernelError("rope_cache_write: slot_mapping must be int64 [T]")
+    _lib.call("sa_rope_cache_write", _ptr(qkv), _code(qkv), stride, _ptr(positions), _ptr(timescale),
+              float(scale_factor), float(q_div), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), T, num_heads,
+              num_kv_heads, head_dim, page_size, _stream())
+
+
+def rope(x: torch.Tensor, positions: torch.Tensor, timescale: torch.Tensor, scale_factor: float, div: float,
+         num_heads: int, head_dim: int) -> None:
+    """In place: x[t, h, :] rotated by positions[t], then divided by div.  x: [T, >= num_heads * head_dim]."""
+    _dev(x, positions, timescale)
+    stride = _rows(x, "rope: x")
+    T = x.shape[0]
+    if x.shape[1] < num_heads * head_dim:
+        raise KernelError("rope: rows are shorter than heads * head size")
+    _i32(positions, "rope: positions", T)
+    if timescale.dtype != torch.float32 or timescale.numel() != head_dim // 2 or not timescale.is_contiguous():
+        raise KernelError("rope: timescale must be float32 [head_dim / 2]")
+    _lib.call("sa_rope", _ptr(x), _code(x), stride, _ptr(positions), _ptr(timescale), float(scale_factor), float(div),
+              T, num_heads, head_dim, _stream())
+
+
+def gather_rows(x: torch.Tensor, index: torch.Tensor, out_dtype: torch.dtype | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    _dev(x, index, out)
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("gather_rows: x must be contiguous 2-D")
+    _i32(index, "gather_rows: index")
+    R, D = index.numel(), x.shape[1]
+    if out is None:
+        out = torch.empty((R, D), dtype=out_dtype or x.dtype, device=x.device)
+    if tuple(out.shape) != (R, D) or not out.is_contiguous():
+        raise KernelError("gather_rows: bad output")
+    _lib.call("sa_gather_rows", _ptr(x), _code(x), _ptr(index), _ptr(out), _code(out), R, D, _stream())
+    return out
+
+
+def fill_(t: torch.Tensor, value_bits: int = 0) -> None:
+    """Sets every 32-bit word of `t` to `value_bits` with a kernel (safe inside a captured graph)."""
+    _dev(t)
+    nbytes = t.numel() * t.element_size()
+    if not t.is_contiguous() or nbytes % 4:
+        raise KernelError("fill_: needs a contiguous tensor of a multiple of 4 bytes")
+    _lib.call("sa_fill_u32", _ptr(t), value_bits & 0xFFFFFFFF, nbytes // 4, _stream())
+
+
+# --------------------------------------------------------------------------- matrix products
+
+EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: torch.Tensor | None = None, soft_cap: float | None = None,
+         out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None, algo: int = ALGO_AUTO) -> torch.Tensor:
+    """a[M, K] . w[N, K]^T.  With w2: gelu_tanh(a.w^T) * (a.w2^T).  With soft_cap: cap * tanh(. / cap)."""
+    _dev(a, w, w2, out)
+    lda = _rows(a, "gemm: a")
+    M, K = a.shape
+    if w.dim() != 2 or not w.is_contiguous() or w.shape[1] != K:
+        raise KernelError(f"gemm: weight {tuple(w.shape)} does not match a {tuple(a.shape)} (expects [N, K] contiguous)")
+    N = w.shape[0]
+    if w.dtype != a.dtype:
+        raise KernelError(f"gemm: a is {a.dtype} but the weight is {w.dtype}")
+    epi, cap = EPILOGUE_NONE, 0.0
+    if w2 is not None:
+        if soft_cap:
+            raise KernelError("gemm: the gated and the soft-cap epilogue do not combine")
+        if w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous():
+            raise KernelError("gemm: the second weight must match the first")
+        epi = EPILOGUE_GATED_GELU
+    elif soft_cap:
+        epi, cap = EPILOGUE_SOFT_CAP, float(soft_cap)
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+    if tuple(out.shape) != (M, N):
+        raise KernelError("gemm: bad output shape")
+    ldc = _rows(out, "gemm: out")
+    _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(w), _ptr(w2), _code(w), _ptr(out), _code(out), ldc, M, N, K, epi,
+              cap, algo, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------- attention
+
+
+def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                    token_seq: torch.Tensor, positions: torch.Tensor, num_heads: int, *, window: int | None,
+                    soft_cap: float | None, out: torch.Tensor | None = None, algo: int = ALGO_AUTO) -> torch.Tensor:
+    """q: [T, >= H * hd] rows (a view into the fused projection is fine).  Returns [T, H * hd]."""
+    _dev(q, k_pages, v_pages, block_table, token_seq, positions, out)
+    q_stride = _rows(q, "paged_attention: q")
+    T = q.shape[0]
+    if k_pages.dim() != 4 or k_pages.shape != v_pages.shape or not k_pages.is_contiguous() \
+            or not v_pages.is_contiguous() or k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+        raise KernelError("paged_attention: pages must be contiguous [pages, K, page_size, hd] of the query's type")
+    num_pages, Kh, page_size, hd = k_pages.shape
+    if q.shape[1] < num_heads * hd:
+        raise KernelError("paged_attention: query rows are shorter than heads * head size")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("paged_attention: block_table must be int32 [sequences, blocks]")
+    _i32(token_seq, "paged_attention: token_seq", T)
+    _i32(positions, "paged_attention: positions", T)
+    if out is None:
+        out = torch.empty((T, num_heads * hd), dtype=q.dtype, device=q.device)
+    if tuple(out.shape) != (T, num_heads * hd) or out.dtype != q.dtype:
+        raise KernelError("paged_attention: bad output")
+    out_stride = _rows(out, "paged_attention: out")
+    _lib.call("sa_paged_attention", _ptr(q), _code(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+              block_table.stride(0), _ptr(token_seq), _ptr(positions), _ptr(out), out_stride, T, num_heads, Kh, hd,
+              page_size, int(window or 0), float(soft_cap or 0.0), algo, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------- sampling
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           seed: torch.Tensor, counter: torch.Tensor, tokens: torch.Tensor | None = None,
+           logprobs: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """One token per row.  All per-row parameter tensors are on the device, [R]."""
+    _dev(logits, temperature, top_k, top_p, seed, counter, tokens, logprobs)
+    if logits.dtype != torch.float32:
+        raise KernelError("sample: logits must be float32")
+    stride = _rows(logits, "sample: logits")
+    R, V = logits.shape
+    for t, dt, name in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                        (top_p, torch.float32, "top_p"), (seed, torch.int64, "seed"), (counter, torch.int32, "counter")):
+        if t.dtype != dt or t.numel() < R or not t.is_contiguous():
+            raise KernelError(f"sample: {name} must be a contiguous {dt} tensor with one entry per row")
+    if tokens is None:
+        tokens = torch.empty(R, dtype=torch.int32, device=logits.device)
+    if logprobs is None:
+        logprobs = torch.empty(R, dtype=torch.float32, device=logits.device)
+    _i32(tokens, "sample: tokens", R)
+    _lib.call("sa_sample", _ptr(logits), stride, R, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seed),
+              _ptr(counter), _ptr(tokens), _ptr(logprobs), _stream())
+    return tokens, logprobs
+
+
+def philox4x32_10(counter: tuple[int, int, int, int], key: tuple[int, int]) -> tuple[int, int, int, int]:
+    """Host function: one block of the generator that `sample` uses."""
+    c = (ctypes.c_uint32 * 4)(*counter)
+    k = (ctypes.c_uint32 * 2)(*key)
+    o = (ctypes.c_uint32 * 4)()
+    _lib.load().sa_philox4x32_10(c, k, o)
+    return tuple(int(v) for v in o)

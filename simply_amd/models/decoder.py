@@ -1,0 +1,93 @@
+"""A decoder put together from a `ModelSpec`: embedding, the layers run in the order of the
+schedule, final norm, head (simply/model_lib.py:2750 TransformerLM, apply :2935-3189).
+
+The model knows nothing of any one architecture: every part is built from its registry by
+the kind that the spec names.
+"""
+from __future__ import annotations
+
+from typing import Callable, Mapping
+
+import torch
+
+from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
+from ..config.spec import LayerSpec, ModelSpec, PartSpec
+from ..kernels import ops
+from ..parts.base import Block, ParamSpec, Part
+from ..parts.embedding import EMBEDDINGS, HEADS
+from ..registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+
+
+def _build_layer(spec: LayerSpec) -> Block:
+    mixer = MIXERS.build(spec.mixer.kind, **spec.mixer.params)
+    ffn = FEED_FORWARDS.build(spec.feed_forward.kind, **spec.feed_forward.params)
+    norms = {name: NORMS.build(ns.kind, **ns.params) for name, ns in spec.norms.items()}
+    return BLOCKS.build(spec.block.kind, mixer, ffn, norms, **spec.block.params)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        if spec.embedding.kind not in EMBEDDINGS:
+            raise ValueError(f"unknown embedding {spec.embedding.kind!r}; known: {sorted(EMBEDDINGS)}")
+        if spec.head.kind not in HEADS:
+            raise ValueError(f"unknown head {spec.head.kind!r}; known: {sorted(HEADS)}")
+        self.embedding = EMBEDDINGS[spec.embedding.kind](**spec.embedding.params)
+        self.head = HEADS[spec.head.kind](**spec.head.params)
+        self.final_norm = NORMS.build(spec.final_norm.kind, **spec.final_norm.params)
+        self.layers: list[Block] = [_build_layer(ls) for ls in spec.layers]
+        self.loaded = False
+
+    # ------------------------------------------------------------------ tensors
+    def _bindings(self) -> list[tuple[Part, PartSpec]]:
+        out: list[tuple[Part, PartSpec]] = [(self.embedding, self.spec.embedding)]
+        for block, ls in zip(self.layers, self.spec.layers):
+            out.append((block.mixer, ls.mixer))
+            out.append((block.feed_forward, ls.feed_forward))
+            for name, ns in ls.norms.items():
+                out.append((block.norms[name], ns))
+        out.append((self.final_norm, self.spec.final_norm))
+        out.append((self.head, self.spec.head))
+        return out
+
+    def expected_tensors(self) -> dict[str, ParamSpec]:
+        """Tensor name in the model folder -> what is expected of it, in a fixed order."""
+        expected: dict[str, ParamSpec] = {}
+        for part, ps in self._bindings():
+            for local, pspec in part.param_specs().items():
+                if local not in ps.tensors:
+                    raise ValueError(f"part {ps.kind!r} needs a tensor {local!r} that its spec does not name")
+                name = ps.tensors[local]
+                if name in expected and expected[name].shape != pspec.shape:
+                    raise ValueError(f"tensor {name!r} is used with shapes {expected[name].shape} and {pspec.shape}")
+                expected.setdefault(name, pspec)
+        return expected
+
+    def load_tensors(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """`tensors`: name in the model folder -> device tensor in its final dtype."""
+        for part, ps in self._bindings():
+            part.load({local: tensors[ps.tensors[local]] for local in part.param_specs()})
+        self.loaded = True
+
+    # ------------------------------------------------------------------ cache
+    def cache_needs(self):
+        """For each schedule entry: (need of its mixer or None, cache_from)."""
+        return [(self.layers[e.layer].mixer.cache_need(), e.cache_from) for e in self.spec.schedule]
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, tokens: torch.Tensor, ctx, cache_views, logit_rows: torch.Tensor | None) -> torch.Tensor | None:
+        """Runs this step's tokens through the schedule.  Returns float32 logits [R, V] at the rows of
+        the step that `logit_rows` (int32 [R]) names, or None if it is None or empty."""
+        h = self.embedding.forward(tokens)
+        schedule = self.spec.schedule
+        normed = None
+        for i, entry in enumerate(schedule):
+            block = self.layers[entry.layer]
+            nxt = self.layers[schedule[i + 1].layer].first_norm() if i + 1 < len(schedule) else None
+            h, normed = block.forward(h, ctx, cache_views[i], normed, nxt)
+        if logit_rows is None or logit_rows.numel() == 0:
+            return None
+        rows = ops.gather_rows(h, logit_rows)
+        x = self.final_norm.forward(rows, ctx.dtype)
+        return self.head.forward(x)

@@ -1,0 +1,71 @@
+"""Grouped-query attention over a paged cache.
+
+simply/model_lib.py:1605 (Attention): q/k/v projections, position encoding on q and k,
+q / query_scale (:1987-2020), attention over the cache with soft-cap and window
+(simply/utils/ragged_paged_attention.py:870-949), output projection (:2362).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.spec import PartSpec
+from ..kernels import ops
+from ..registry import MIXERS, POSITION_ENCODINGS
+from .base import Mixer, PagedKVNeed, ParamSpec
+
+
+@MIXERS.register("paged_attention")
+class PagedAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, query_scale: float,
+                 soft_cap: float | None = None, window: int | None = None,
+                 position_encoding: PartSpec | None = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"paged_attention: {num_heads} heads do not split over {num_kv_heads} kv heads")
+        if head_dim % 16:
+            raise ValueError(f"paged_attention: head_dim {head_dim} must be a multiple of 16")
+        self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.query_scale = float(query_scale)
+        self.soft_cap = float(soft_cap) if soft_cap else None
+        self.window = int(window) if window else None
+        self.position_encoding = (POSITION_ENCODINGS.build(position_encoding.kind, **position_encoding.params)
+                                  if position_encoding is not None else None)
+        self.qkv_proj: torch.Tensor | None = None
+        self.o_proj: torch.Tensor | None = None
+
+    def param_specs(self):
+        D, H, K, hd = self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim
+        return {"q_proj": ParamSpec((H * hd, D)), "k_proj": ParamSpec((K * hd, D)),
+                "v_proj": ParamSpec((K * hd, D)), "o_proj": ParamSpec((D, H * hd))}
+
+    def load(self, tensors):
+        # one product for q, k and v: rows [q heads | k heads | v heads]
+        self.qkv_proj = torch.cat([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]], dim=0).contiguous()
+        self.o_proj = tensors["o_proj"]
+        if self.position_encoding is not None and hasattr(self.position_encoding, "to_device"):
+            self.position_encoding.to_device(self.o_proj.device)
+
+    def cache_need(self):
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, ctx, cache):
+        H, K, hd = self.num_heads, self.num_kv_heads, self.head_dim
+        group = ctx.groups[cache.group_id]
+        qkv = ops.gemm(x, self.qkv_proj)
+        pe = self.position_encoding
+        rotary = pe.rotary_table() if pe is not None else None
+        write = cache.write
+        if pe is None or rotary is not None:
+            table, sf = rotary if rotary is not None else (None, 1.0)
+            ops.rope_cache_write(qkv, ctx.positions, table, sf, self.query_scale, H, K, hd,
+                                 slot_mapping=group.slot_mapping if write else None,
+                                 k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+        else:
+            # another position encoding: applied by the part itself, then the plain scale-and-write kernel
+            pe.apply(qkv, ctx.positions, H, hd, 1.0)
+            pe.apply(qkv[:, H * hd:], ctx.positions, K, hd, 1.0)
+            ops.rope_cache_write(qkv, ctx.positions, None, 1.0, self.query_scale, H, K, hd,
+                                 slot_mapping=group.slot_mapping if write else None,
+                                 k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+        o = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions,
+                                H, window=self.window, soft_cap=self.soft_cap)
+        return ops.gemm(o, self.o_proj)

@@ -1,0 +1,30 @@
+"""Dense gated feed-forward: down(act(gate(x)) * up(x))  (simply/model_lib.py:643-730 with
+use_gated_activation_in_ffn=True, ffn_use_bias=False)."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..registry import ACTIVATIONS, FEED_FORWARDS
+from .base import FeedForward, ParamSpec
+
+# activation name -> epilogue of the fused gate/up product
+ACTIVATIONS.register("gelu_tanh", ops.EPILOGUE_GATED_GELU)
+
+
+@FEED_FORWARDS.register("gated_dense")
+class GatedDense(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh"):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        if ACTIVATIONS.get(activation) != ops.EPILOGUE_GATED_GELU:
+            raise ValueError(f"gated_dense: activation {activation!r} has no fused kernel")
+        self.activation = activation
+        self.gate_proj = self.up_proj = self.down_proj = None
+
+    def param_specs(self):
+        D, F = self.hidden_size, self.intermediate_size
+        return {"gate_proj": ParamSpec((F, D)), "up_proj": ParamSpec((F, D)), "down_proj": ParamSpec((D, F))}
+
+    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+        z = ops.gemm(x, self.gate_proj, w2=self.up_proj)   # gelu(x.Wg^T) * (x.Wu^T), one kernel
+        return ops.gemm(z, self.down_proj)

@@ -1,0 +1,66 @@
+"""The engine on the GPU against the plain implementation, in float32 and in bfloat16, under every
+way of cutting the work."""
+import numpy as np
+import pytest
+import torch
+
+import plain_gemma2 as plain
+import tiny
+from simply_amd.config import EngineConfig
+from simply_amd.engine import Executor, StepEntry
+from simply_amd.engine.loading import load_model
+
+pytestmark = pytest.mark.gpu
+
+# largest difference of logits, as a fraction of the largest logit of the plain implementation
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+@pytest.fixture(autouse=True)
+def _lib(gpu_lib):
+    return gpu_lib
+
+
+def make_executor(model_dir, dtype, page_size=4, num_pages=64, batch=4, max_len=256, poison=True):
+    cfg = EngineConfig(activation_dtype=dtype, page_size=page_size, batch_size=batch, max_seq_len=max_len,
+                       max_num_issue_tokens=max_len, total_num_pages=num_pages, device="cuda:0", use_graphs=False,
+                       poison_freed_pages=poison)
+    model, _ = load_model(model_dir, cfg.dtype, "cuda:0")
+    return Executor(model, cfg)
+
+
+def run_cut(ex, rid, tokens, cuts):
+    out, i = [], 0
+    ex.add_request(rid)
+    for c in cuts:
+        part = tokens[i:i + c]
+        out.append(ex.step([StepEntry(rid, part, list(range(len(part))))]).cpu())
+        i += len(part)
+    assert i == len(tokens)
+    ex.finish_request(rid)
+    ex.cache.check()
+    return torch.cat(out)
+
+
+def plain_logits(model_dir, tokens, dtype):
+    """The plain implementation in float64 on the weights as the engine holds them."""
+    w, cfg = plain.load(model_dir)
+    if dtype == "bfloat16":
+        w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    return plain.forward(w, cfg, tokens, torch.float64), cfg
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_cuts_match_plain(tmp_path, name, dtype):
+    d = tiny.write_model(name, str(tmp_path / name), std=0.3)
+    vocab = plain.load(d)[1]["vocab_size"]
+    tokens = tiny.random_tokens(77, vocab, 7)
+    want, cfg = plain_logits(d, tokens, dtype)
+    scale = want.abs().max().item()
+    ex = make_executor(d, dtype)
+    for cuts in ([77], [45] + [1] * 32, [7, 5, 3, 2, 11, 2, 2, 13, 17, 2, 13], [1] * 77):
+        got = run_cut(ex, "r", tokens, cuts).double()
+        assert torch.isfinite(got).all()
+        err = (got - want).abs().max().item() / scale
+        assert err <= TOL[dtype], (cuts, err)

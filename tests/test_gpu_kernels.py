@@ -1,0 +1,226 @@
+"""Each HIP kernel alone against its plain torch reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+import torch_ops as ref
+
+pytestmark = pytest.mark.gpu
+
+DT = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.fixture(autouse=True)
+def _lib(gpu_lib):
+    return gpu_lib
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("V,D,T", [(50, 24, 7), (333, 1000, 33)])
+def test_embed(dtype, V, D, T):
+    from simply_amd.kernels import ops
+    table = rand((V, D), dtype, 0)
+    tokens = torch.randint(0, V, (T,), dtype=torch.int32).cuda()
+    got = ops.embed(table, tokens, 3.25)
+    torch.testing.assert_close(got, ref.embed(table, tokens, 3.25), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,D", [(1, 16), (5, 100), (3, 2304), (2, 5000)])
+def test_rmsnorm(dtype, T, D):
+    from simply_amd.kernels import ops
+    x = rand((T, D), torch.float32, 1, 3.0)
+    w = rand((D,), dtype, 2, 0.3)
+    for plus_one in (True, False):
+        got = ops.rmsnorm(x, w, 1e-5, plus_one, dtype)
+        torch.testing.assert_close(got.float(), ref.rmsnorm(x, w, 1e-5, plus_one, dtype).float(), **tol(dtype))
+    xa = x.to(dtype)
+    got = ops.rmsnorm(xa, w, 1e-6, True, dtype)
+    torch.testing.assert_close(got.float(), ref.rmsnorm(xa, w, 1e-6, True, dtype).float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304)])
+def test_add_rmsnorm(dtype, T, D):
+    from simply_amd.kernels import ops
+    y = rand((T, D), dtype, 3, 2.0)
+    h0 = rand((T, D), torch.float32, 4, 5.0)
+    w1, w2 = rand((D,), dtype, 5, 0.3), rand((D,), torch.float32, 6, 0.3)
+    for with_post in (True, False):
+        for with_next in (True, False):
+            h_got, h_ref = h0.clone(), h0.clone()
+            kw = dict(post_weight=w1 if with_post else None, post_eps=1e-6, next_weight=w2 if with_next else None,
+                      next_eps=1e-5, out_dtype=dtype)
+            o_got = ops.add_rmsnorm(y, h_got, **kw)
+            o_ref = ref.add_rmsnorm(y, h_ref, **kw)
+            torch.testing.assert_close(h_got, h_ref, rtol=1e-5, atol=1e-5)
+            assert (o_got is None) == (o_ref is None)
+            if o_got is not None:
+                torch.testing.assert_close(o_got.float(), o_ref.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("H,K,hd,P", [(4, 2, 16, 4), (6, 1, 32, 3), (8, 4, 256, 16), (3, 3, 48, 5)])
+def test_rope_cache_write(dtype, H, K, hd, P):
+    from simply_amd.kernels import ops
+    T, pages = 11, 9
+    qkv = rand((T, (H + 2 * K) * hd), dtype, 7)
+    positions = torch.tensor([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7], dtype=torch.int32).cuda()
+    ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda()
+    slots = torch.randperm(pages * P)[:T].to(torch.int64).cuda()
+    kp, vp = (torch.zeros((pages, K, P, hd), dtype=dtype).cuda() for _ in range(2))
+    kp2, vp2, qkv2 = kp.clone(), vp.clone(), qkv.clone()
+    ops.rope_cache_write(qkv, positions, ts, 1.0, 12.0, H, K, hd, slots, kp, vp)
+    ref.rope_cache_write(qkv2, positions, ts, 1.0, 12.0, H, K, hd, slots, kp2, vp2)
+    t = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else tol(dtype)  # sin/cos of angles up to 8000 rad
+    torch.testing.assert_close(qkv[:, :H * hd].float(), qkv2[:, :H * hd].float(), **t)
+    torch.testing.assert_close(kp.float(), kp2.float(), **t)
+    torch.testing.assert_close(vp, vp2, rtol=0, atol=0)
+    # without rotation and without a cache: only the query scale
+    q3 = rand((T, (H + 2 * K) * hd), dtype, 8)
+    q4 = q3.clone()
+    ops.rope_cache_write(q3, positions, None, 1.0, 3.0, H, K, hd)
+    torch.testing.assert_close(q3[:, :H * hd].float(), (q4[:, :H * hd].float() / 3.0).to(dtype).float(), **tol(dtype))
+    torch.testing.assert_close(q3[:, H * hd:], q4[:, H * hd:], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("M,N,K", [(1, 7, 5), (3, 64, 64), (65, 130, 100), (17, 333, 72), (128, 96, 2304)])
+def test_gemm_generic(dtype, M, N, K):
+    from simply_amd.kernels import ops
+    a, w, w2 = rand((M, K), dtype, 9), rand((N, K), dtype, 10, 0.1), rand((N, K), dtype, 11, 0.1)
+    t = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else tol(dtype)
+    for algo in (ops.ALGO_AUTO, ops.ALGO_GENERIC):
+        torch.testing.assert_close(ops.gemm(a, w, algo=algo).float(), ref.gemm(a, w).float(), **t)
+        torch.testing.assert_close(ops.gemm(a, w, w2=w2, algo=algo).float(), ref.gemm(a, w, w2=w2).float(), **t)
+        got = ops.gemm(a, w, soft_cap=2.0, out_dtype=torch.float32, algo=algo)
+        assert got.dtype == torch.float32
+        torch.testing.assert_close(got, ref.gemm(a, w, soft_cap=2.0, out_dtype=torch.float32), **t)
+    # rows of a wider buffer as input (a view), as the attention output is
+    wide = rand((M, K + 24), dtype, 12)
+    torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], w).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
+
+
+def test_gemm_rows_do_not_depend_on_the_batch():
+    """float32: a row's product is bit-identical whatever other rows are in the batch."""
+    from simply_amd.kernels import ops
+    a, w = rand((70, 200), torch.float32, 13), rand((150, 200), torch.float32, 14)
+    full = ops.gemm(a, w)
+    for rows in ([0], [69], [3, 4, 5], list(range(64, 70))):
+        part = ops.gemm(a[rows].contiguous(), w)
+        assert torch.equal(part, full[rows])
+
+
+def paged_setup(dtype, S, H, Kh, hd, P, lens, seed):
+    """Random cache contents for S requests of the given lengths, pages handed out in a shuffled order."""
+    max_blocks = max(-(-l // P) for l in lens) + 1
+    num_pages = S * max_blocks + 3
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    table = torch.full((S, max_blocks), -1, dtype=torch.int32)
+    kp = torch.full((num_pages, Kh, P, hd), float("nan"), dtype=dtype)
+    vp = torch.full((num_pages, Kh, P, hd), float("nan"), dtype=dtype)
+    for s, l in enumerate(lens):
+        for b in range(-(-l // P)):
+            page = perm.pop()
+            table[s, b] = page
+            n = min(P, l - b * P)
+            kp[page, :, :n] = torch.randn((Kh, n, hd), generator=g).to(dtype)
+            vp[page, :, :n] = torch.randn((Kh, n, hd), generator=g).to(dtype)
+    return kp.cuda(), vp.cuda(), table.cuda()
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("H,Kh,hd,P,window,cap", [
+    (4, 2, 16, 4, None, 50.0), (4, 2, 16, 4, 8, 50.0), (6, 1, 32, 3, 16, None), (8, 4, 256, 16, None, 50.0),
+    (6, 3, 48, 5, 5, 20.0), (16, 1, 64, 16, 70, None), (2, 2, 128, 64, 100, 30.0)])
+def test_paged_attention_generic(dtype, H, Kh, hd, P, window, cap):
+    from simply_amd.kernels import ops
+    lens = [1, 37, 150, 64]
+    kp, vp, table = paged_setup(dtype, len(lens), H, Kh, hd, P, lens, 21)
+    # queries: the last tokens of each request, several per request (a portion), unfilled page tails are NaN
+    token_seq, positions = [], []
+    for s, l in enumerate(lens):
+        for p in range(max(0, l - 5), l):
+            token_seq.append(s)
+            positions.append(p)
+    T = len(positions)
+    q = rand((T, H * hd + 32), dtype, 22, 0.5)[:, :H * hd]
+    ts = torch.tensor(token_seq, dtype=torch.int32).cuda()
+    ps = torch.tensor(positions, dtype=torch.int32).cuda()
+    got = ops.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap, algo=ops.ALGO_GENERIC)
+    want = ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap)
+    assert torch.isfinite(got.float()).all()
+    t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else tol(dtype)
+    torch.testing.assert_close(got.float(), want.float(), **t)
+
+
+def test_paged_attention_far_key_and_window_edge():
+    """One key far back gets a score that stands out: a global layer must find it, a windowed layer
+    must see it exactly while it is inside the window."""
+    from simply_amd.kernels import ops
+    H = Kh = 1
+    hd, P, L = 32, 16, 300
+    kp, vp, table = paged_setup(torch.float32, 1, H, Kh, hd, P, [L], 31)
+    kp.mul_(0.01)
+    far = 37
+    page, off = int(table[0, far // P]), far % P
+    kp[page, 0, off] = 0.0
+    kp[page, 0, off, 3] = 50.0
+    vp[page, 0, off] = 7.0
+    q = torch.zeros((1, hd)).cuda()
+    q[0, 3] = 1.0
+    ts = torch.zeros(1, dtype=torch.int32).cuda()
+    for window, pos, sees in [(None, L - 1, True), (100, far + 99, True), (100, far + 100, False), (1, far, True)]:
+        ps = torch.tensor([pos], dtype=torch.int32).cuda()
+        out = ops.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=None)
+        assert (abs(out.mean().item() - 7.0) < 1e-3) == sees, (window, pos, out.mean().item())
+        torch.testing.assert_close(out, ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=None),
+                                   rtol=1e-4, atol=1e-5)
+
+
+def test_sampling_kernel():
+    from simply_amd.kernels import ops
+    V, R = 1000, 6
+    logits = rand((R, V), torch.float32, 41, 3.0)
+    temperature = torch.tensor([0.0, 1.0, 0.7, 1.0, 1.3, 1.0]).cuda()
+    top_k = torch.tensor([-1, -1, -1, 1, 20, 50], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 1.0, 1.0, 1.0, 1.0, 0.6]).cuda()
+    seed = torch.tensor([1, 2, 3, 4, 5, 2**40 + 17], dtype=torch.int64).cuda()
+    counter = torch.tensor([0, 5, 9, 0, 3, 77], dtype=torch.int32).cuda()
+    tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
+    rtok, rlp = ref.sample(logits, temperature, top_k, top_p, seed, counter)
+    assert tok.tolist() == rtok.tolist()
+    torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+    assert tok[0].item() == int(logits[0].argmax()) and tok[3].item() == int(logits[3].argmax())
+    # same seed and counter: same token; another counter: (almost surely) another stream
+    tok2, _ = ops.sample(logits, temperature, top_k, top_p, seed, counter)
+    assert tok.tolist() == tok2.tolist()
+    # host copy of the generator agrees with the reference implementation
+    assert ops.philox4x32_10((1, 2, 3, 4), (5, 6)) == ref.philox4x32_10((1, 2, 3, 4), (5, 6))
+
+
+def test_sampling_frequencies():
+    """10^4 draws from a 4-way distribution lie within 4 sigma of softmax(logits / T)
+    (after simply/utils/sampling_lib_test.py:138-152)."""
+    from simply_amd.kernels import ops
+    n, T = 10000, 0.7
+    base = torch.tensor([1.0, 0.0, -1.0, 2.0])
+    logits = base.repeat(n, 1).cuda()
+    tok, _ = ops.sample(logits, torch.full((n,), T).cuda(), torch.full((n,), -1, dtype=torch.int32).cuda(),
+                        torch.ones(n).cuda(), torch.full((n,), 1234, dtype=torch.int64).cuda(),
+                        torch.arange(n, dtype=torch.int32).cuda())
+    freq = torch.bincount(tok.long().cpu(), minlength=4).double() / n
+    p = torch.softmax(base.double() / T, -1)
+    sigma = torch.sqrt(p * (1 - p) / n)
+    assert ((freq - p).abs() < 4 * sigma).all(), (freq, p)

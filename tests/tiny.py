@@ -1,0 +1,48 @@
+"""Two tiny Gemma 2 configurations that differ in every size and option, and helpers that write them
+as model folders with random weights (in a temporary folder, never committed)."""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+
+TINY_A = dict(
+    architectures=["Gemma2ForCausalLM"], hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
+    num_key_value_heads=2, head_dim=16, intermediate_size=128, vocab_size=256, rms_norm_eps=1e-6,
+    rope_theta=10000.0, sliding_window=8, query_pre_attn_scalar=16, attn_logit_softcapping=50.0,
+    final_logit_softcapping=30.0, tie_word_embeddings=True, max_position_embeddings=512,
+    hidden_activation="gelu_pytorch_tanh", initializer_range=0.02,
+)
+TINY_B = dict(
+    architectures=["Gemma2ForCausalLM"], hidden_size=96, num_hidden_layers=3, num_attention_heads=6,
+    num_key_value_heads=1, head_dim=32, intermediate_size=320, vocab_size=512, rms_norm_eps=1e-5,
+    rope_theta=1000000.0, sliding_window=16, query_pre_attn_scalar=24, attn_logit_softcapping=None,
+    final_logit_softcapping=15.0, tie_word_embeddings=True, max_position_embeddings=512,
+    hidden_activation="gelu_pytorch_tanh", initializer_range=0.05,
+)
+# a third one with sizes that are no power of two anywhere and a vocabulary that is no multiple of 64
+TINY_C = dict(
+    architectures=["Gemma2ForCausalLM"], hidden_size=120, num_hidden_layers=4, num_attention_heads=6,
+    num_key_value_heads=3, head_dim=48, intermediate_size=200, vocab_size=333, rms_norm_eps=1e-6,
+    rope_theta=5000.0, sliding_window=5, query_pre_attn_scalar=30, attn_logit_softcapping=20.0,
+    final_logit_softcapping=None, tie_word_embeddings=True, max_position_embeddings=512,
+    layer_types=["full_attention", "sliding_attention", "sliding_attention", "full_attention"],
+    hidden_activation="gelu_pytorch_tanh", initializer_range=0.08,
+)
+CONFIGS = {"A": (TINY_A, 0, 0.1), "B": (TINY_B, 1, 0.2), "C": (TINY_C, 2, 0.3)}
+
+
+def write_model(name: str, out_dir: str, dtype=torch.float32, std: float | None = None) -> str:
+    """Writes configuration `name` with random weights through the framework's random-weights mode."""
+    from simply_amd.config import config_from_dict
+    from simply_amd.weights import write_random_model
+
+    d, seed, norm_std = CONFIGS[name]
+    cfg = config_from_dict(d)
+    return write_random_model(cfg, out_dir, seed, dtype, std=std, norm_std=norm_std)
+
+
+def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
