@@ -223,6 +223,9 @@ class CacheManager:
         self.slots = StateSlots(num_slots)
         self.groups: list[CacheGroup] = []
         self.requests: dict[Hashable, int] = {}
+        #: a number that is new for every admission (a request that comes back after giving up its pages gets another)
+        self.admission: dict[Hashable, int] = {}
+        self._admissions = 0
         self.views: list[CacheView] = []
         self._group_entries: dict[int, list[int]] = {}
         self._device_tables: dict[int, torch.Tensor] = {}
@@ -275,6 +278,8 @@ class CacheManager:
             raise CacheError(f"request {rid!r} is already admitted")
         slot = self.slots.take(rid)
         self.requests[rid] = slot
+        self._admissions += 1
+        self.admission[rid] = self._admissions
         for g in self.groups:
             g.add(rid, slot)
         for v in self.views:
@@ -313,6 +318,7 @@ class CacheManager:
     def free(self, rid: Hashable) -> None:
         """Gives back everything the request holds."""
         slot = self.requests.pop(rid)
+        del self.admission[rid]
         for g in self.groups:
             self._poison(g, g.remove(rid))
         self.slots.give_back(slot)

@@ -25,6 +25,7 @@ class StepEntry:
     request_id: Hashable
     tokens: Sequence[int]                 # the request's next tokens
     want: Sequence[int] = ()              # places among `tokens` whose logits are wanted
+    start: int | None = None              # position of tokens[0]; None: right after the tokens run so far
 
 
 class Executor:
@@ -41,7 +42,7 @@ class Executor:
         self.cache = CacheManager(model.cache_needs(), page_size=config.page_size, num_pages=pages,
                                   num_slots=config.batch_size, max_seq_len=config.max_seq_len, dtype=self.dtype,
                                   device=self.device, poison=config.poison_freed_pages)
-        self.num_computed: dict[Hashable, int] = {}
+        self.num_computed: dict[Hashable, tuple[int, int]] = {}  # request -> (admission, tokens run)
         self.vocab_size = model.spec.vocab_size
         # one pinned staging buffer and one device buffer for all of a step's integers
         cap = max(config.issue_budget, config.batch_size)
@@ -55,16 +56,25 @@ class Executor:
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid: Hashable) -> int:
-        slot = self.cache.admit(rid)
-        self.num_computed[rid] = 0
-        return slot
+        """Admits a request to the cache (a scheduler may do that itself on `self.cache`)."""
+        return self.cache.admit(rid)
 
     def finish_request(self, rid: Hashable) -> None:
         self.cache.free(rid)
-        del self.num_computed[rid]
 
     def has_request(self, rid: Hashable) -> bool:
-        return rid in self.num_computed
+        return rid in self.cache.requests
+
+    def _start_of(self, e: "StepEntry") -> int:
+        admission, done = self.num_computed.get(e.request_id, (0, 0))
+        if admission != self.cache.admission[e.request_id]:
+            done = 0  # the request has given up its pages and come back since
+        if e.start is None:
+            return done
+        if e.start > done:
+            raise ValueError(f"request {e.request_id!r}: a portion starting at {e.start} would leave positions "
+                             f"{done}..{e.start - 1} without keys")
+        return e.start
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
@@ -81,12 +91,15 @@ class Executor:
             if e.request_id in seen:
                 raise ValueError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            if e.request_id not in self.num_computed:
-                raise KeyError(f"request {e.request_id!r} has not been added")
+            if e.request_id not in self.cache.requests:
+                raise KeyError(f"request {e.request_id!r} has not been admitted to the cache")
         cache, cap = self.cache, self._cap
         # make room for every entry first: a failure leaves earlier steps' state untouched only if nothing
         # has been reserved, so check all of them together before changing anything
-        wants = [(e.request_id, self.num_computed[e.request_id], len(e.tokens)) for e in entries]
+        # forget what is known of requests that have left the cache since (finished or preempted elsewhere)
+        for rid in [r for r in self.num_computed if r not in self.cache.requests]:
+            del self.num_computed[rid]
+        wants = [(e.request_id, self._start_of(e), len(e.tokens)) for e in entries]
         if not cache.can_reserve(wants):
             from ..cache import OutOfPages
 
@@ -136,5 +149,5 @@ class Executor:
         logit_rows = dev[3 * cap:3 * cap + R] if R else None
         logits = self.model.forward(dev[:T], ctx, cache.views, logit_rows)
         for rid, start, q in wants:
-            self.num_computed[rid] = start + q
+            self.num_computed[rid] = (cache.admission[rid], start + q)
         return logits

@@ -1,0 +1,186 @@
+"""The Python entry point: token ids in, generated token ids out.
+
+Shaped after `LMInterface.generate` (simply/model_lib.py:4579-4942) and its `SamplingOutput`
+(simply/model_lib.py:4461-4480), but over the paged cache and continuous batching of
+simply/serving/page_batcher.py.  The engine takes and returns token ids; text is out of its scope.
+"""
+from __future__ import annotations
+
+import dataclasses
+import time
+from typing import Sequence
+
+import torch
+
+from ..config import EngineConfig, load_config
+from ..sampling import Sampler, SamplingParams, request_seed
+from .executor import Executor, StepEntry
+from .loading import load_model, random_model
+from .scheduler import Request, Scheduler
+
+
+@dataclasses.dataclass(frozen=True)
+class SamplingOutput:
+    """simply/model_lib.py:4461-4480, the fields that exist without a tokenizer."""
+
+    input_token_ids: list[int]
+    output_token_ids: list[int]
+    output_token_logprobs: list[float]
+    is_truncated: bool
+    finish_reason: str
+    num_preemptions: int = 0
+
+    @property
+    def sum_output_logprob(self) -> float:
+        return float(sum(self.output_token_logprobs))
+
+    @property
+    def avg_output_logprob(self) -> float:
+        return self.sum_output_logprob / max(len(self.output_token_logprobs), 1)
+
+
+RequestOutput = SamplingOutput
+
+
+class LMInterface:
+    """A model with weights, a cache, a scheduler and a sampler on one GPU.
+
+    model: a model folder (config.json, model.safetensors); or `config` (a typed architecture
+    configuration) together with `random_weights` (a seed) for weights drawn on the device.
+    The other arguments are the serving knobs of simply/serving/common_flags.py by their names there.
+    """
+
+    def __init__(self, model: str | None = None, *, config=None, random_weights: int | None = None,
+                 activation_dtype: str = "bfloat16", batch_size: int = 8, max_seq_len: int | None = None,
+                 page_size: int = 16, max_num_issue_tokens: int = 2048, total_num_pages: int | None = None,
+                 seed: int = 0, device: str = "cuda:0", poison_freed_pages: bool = False, use_graphs: bool = True,
+                 _model=None):
+        from ..kernels import lib
+
+        lib.load()  # fails here, loudly, if the kernel library is missing and cannot be built
+        dtype = EngineConfig(activation_dtype=activation_dtype).dtype
+        if _model is not None:       # a model that is already on the device (several engines over one set of weights)
+            self.model, self.model_config = _model, config
+        elif model is not None:
+            self.model, self.model_config = load_model(model, dtype, torch.device(device))
+        elif config is not None and random_weights is not None:
+            self.model_config = config
+            self.model = random_model(config, random_weights, dtype, torch.device(device))
+        else:
+            raise ValueError("give a model folder, or a configuration and a seed for random weights")
+        if max_seq_len is None:
+            max_seq_len = self.model.spec.max_position
+        self.engine_config = EngineConfig(
+            activation_dtype=activation_dtype, page_size=page_size, batch_size=batch_size, max_seq_len=max_seq_len,
+            max_num_issue_tokens=max_num_issue_tokens, total_num_pages=total_num_pages, device=device,
+            poison_freed_pages=poison_freed_pages, use_graphs=use_graphs)
+        self.executor = Executor(self.model, self.engine_config)
+        self.scheduler = Scheduler(self.executor.cache, max_num_issue_tokens=self.engine_config.issue_budget,
+                                   max_seq_len=max_seq_len)
+        self.sampler = Sampler(device, max(batch_size, 1))
+        self.seed = int(seed)
+        self._num_requests = 0
+        self.stats = {"steps": 0, "tokens": 0, "preemptions": 0, "seconds": 0.0}
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, request_id, prompt_token_ids: Sequence[int], params: SamplingParams | None = None) -> Request:
+        params = params or SamplingParams()
+        seed = params.seed if params.seed is not None else request_seed(self.seed, self._num_requests)
+        self._num_requests += 1
+        vocab = self.model.spec.vocab_size
+        ids = [int(t) for t in prompt_token_ids]
+        if any(t < 0 or t >= vocab for t in ids):
+            raise ValueError(f"request {request_id!r}: token id outside [0, {vocab})")
+        r = Request(request_id, ids, params, seed=seed, eos_ids=tuple(self.model.spec.eos_token_ids))
+        self.scheduler.add(r)
+        return r
+
+    def step(self) -> list[Request]:
+        """One scheduling decision and one run of the step function.  Returns the requests that finished."""
+        out = self.scheduler.schedule()
+        self.stats["preemptions"] += len(out.preempted)
+        finished = list(out.finished)
+        if not out.scheduled:
+            return finished
+        entries = []
+        for s in out.scheduled:
+            toks = s.request.all_token_ids[s.start:s.start + s.num_tokens]
+            entries.append(StepEntry(s.request.request_id, toks, [s.num_tokens - 1] if s.samples else [], s.start))
+        logits = self.executor.step(entries)
+        tokens: list = [None] * len(entries)
+        logprobs: list = [None] * len(entries)
+        rows = [i for i, s in enumerate(out.scheduled) if s.samples]
+        if rows:
+            reqs = [out.scheduled[i].request for i in rows]
+            toks, lps = self.sampler.sample(logits, [r.params for r in reqs], [r.seed for r in reqs],
+                                            [len(r.output_token_ids) for r in reqs])
+            for i, t, lp in zip(rows, toks, lps):
+                tokens[i], logprobs[i] = t, lp
+        finished += self.scheduler.update(out.scheduled, tokens, logprobs)
+        self.stats["steps"] += 1
+        self.stats["tokens"] += out.num_tokens
+        return finished
+
+    # ------------------------------------------------------------------ generate
+    def generate(self, input_token_ids: Sequence[int] | Sequence[Sequence[int]], prng_key: int | None = None,
+                 sampling_params: SamplingParams | Sequence[SamplingParams] | None = None) -> list[SamplingOutput]:
+        """Generates a continuation for each input (a list of token ids, or a list of such lists).
+        `prng_key`, if given, replaces the engine's seed for requests whose params carry none."""
+        single = len(input_token_ids) > 0 and isinstance(input_token_ids[0], int)
+        inputs = [input_token_ids] if single else list(input_token_ids)
+        if isinstance(sampling_params, SamplingParams) or sampling_params is None:
+            plist = [sampling_params or SamplingParams()] * len(inputs)
+        else:
+            plist = list(sampling_params)
+            if len(plist) != len(inputs):
+                raise ValueError("one SamplingParams per input, or one for all")
+        if prng_key is not None:
+            self.seed, self._num_requests = int(prng_key), 0
+        t0 = time.perf_counter()
+        requests = [self.add_request(("gen", id(inputs), i), ids, p) for i, (ids, p) in enumerate(zip(inputs, plist))]
+        while self.scheduler.has_work():
+            self.step()
+        self.stats["seconds"] += time.perf_counter() - t0
+        return [SamplingOutput(list(r.prompt_token_ids), list(r.output_token_ids), list(r.output_token_logprobs),
+                               r.is_truncated, r.finish_reason or "", r.num_preemptions) for r in requests]
+
+
+LLM = LMInterface
+
+
+def preload(lm: LMInterface, request_id, prompt_token_ids: Sequence[int], params: SamplingParams, *,
+            seed: int = 0) -> Request:
+    """For measurements: admits a request as if all of its prompt but the last token had been run.  Its
+    pages are reserved as a run would have reserved them and hold what `fill_cache_random` put there, so
+    the next steps are decode steps at the prompt's length without the cost of a real prefill."""
+    from .scheduler import Status
+
+    r = lm.add_request(request_id, prompt_token_ids, params)
+    sched, cache = lm.scheduler, lm.executor.cache
+    sched.waiting.remove(r)
+    cache.admit(r.request_id)
+    n = r.num_tokens - 1
+    if n > 0:
+        cache.reserve(r.request_id, 0, n)
+        # what a windowed group would have given back on the way
+        cache.reserve(r.request_id, n, 0)
+        lm.executor.num_computed[r.request_id] = (cache.admission[r.request_id], n)
+    r.num_computed = n
+    r.status = Status.RUNNING
+    sched.running.append(r)
+    return r
+
+
+def fill_cache_random(lm: LMInterface, std: float = 0.5, seed: int = 0) -> None:
+    """For measurements: fills every page of keys and values with N(0, std)."""
+    gen = torch.Generator(device=lm.executor.device)
+    gen.manual_seed(seed)
+    for v in lm.executor.cache.views:
+        if v.k_pages is not None and v.write:
+            for t in (v.k_pages, v.v_pages):
+                # in slices, so that no float32 copy of a whole pool is made
+                flat = t.view(-1)
+                step = 1 << 26
+                for i in range(0, flat.numel(), step):
+                    n = min(step, flat.numel() - i)
+                    flat[i:i + n] = (torch.randn(n, generator=gen, device=t.device, dtype=torch.float32) * std).to(t.dtype)

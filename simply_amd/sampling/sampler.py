@@ -1,0 +1,61 @@
+"""Draws one token per row of logits with the HIP sampling kernel.
+
+Every request has its own random stream, keyed by its seed and advanced by its own count of drawn
+tokens, so its tokens do not depend on which other requests are in the batch (the reference splits
+one key per step for the whole batch: simply/utils/ragged_paged_attention.py:2031).
+"""
+from __future__ import annotations
+
+from typing import Sequence
+
+import torch
+
+from ..kernels import ops
+from .params import SamplingParams
+
+
+def request_seed(engine_seed: int, request_index: int) -> int:
+    """A 63-bit seed for a request that brought none (splitmix64 of the engine seed and the index)."""
+    z = (engine_seed * 0x9E3779B97F4A7C15 + request_index + 1) & (2**64 - 1)
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & (2**64 - 1)
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & (2**64 - 1)
+    return (z ^ (z >> 31)) & (2**63 - 1)
+
+
+class Sampler:
+    def __init__(self, device, max_rows: int):
+        self.device = torch.device(device)
+        self.max_rows = max_rows
+        pin = self.device.type == "cuda"
+        # [temperature | top_p] as float32 and [top_k | counter] as int32, seeds as int64: one staging buffer each
+        self._f_host = torch.empty(2 * max_rows, dtype=torch.float32, pin_memory=pin)
+        self._i_host = torch.empty(2 * max_rows, dtype=torch.int32, pin_memory=pin)
+        self._s_host = torch.empty(max_rows, dtype=torch.int64, pin_memory=pin)
+        self._f_dev = torch.empty(2 * max_rows, dtype=torch.float32, device=self.device)
+        self._i_dev = torch.empty(2 * max_rows, dtype=torch.int32, device=self.device)
+        self._s_dev = torch.empty(max_rows, dtype=torch.int64, device=self.device)
+        self._tokens = torch.empty(max_rows, dtype=torch.int32, device=self.device)
+        self._logprobs = torch.empty(max_rows, dtype=torch.float32, device=self.device)
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+               counters: Sequence[int]) -> tuple[list[int], list[float]]:
+        """logits float32 [R, V]; one SamplingParams, seed and draw counter per row."""
+        R = logits.shape[0]
+        if not (len(params) == len(seeds) == len(counters) == R):
+            raise ValueError("sample: one params, seed and counter per row of logits")
+        if R > self.max_rows:
+            raise ValueError(f"sample: {R} rows, room for {self.max_rows}")
+        n = self.max_rows
+        for r, (p, s, c) in enumerate(zip(params, seeds, counters)):
+            self._f_host[r] = p.temperature
+            self._f_host[n + r] = p.top_p
+            self._i_host[r] = p.top_k
+            self._i_host[n + r] = c
+            self._s_host[r] = s
+        self._f_dev.copy_(self._f_host, non_blocking=True)
+        self._i_dev.copy_(self._i_host, non_blocking=True)
+        self._s_dev.copy_(self._s_host, non_blocking=True)
+        tokens, logprobs = ops.sample(logits, self._f_dev[:n], self._i_dev[:n], self._f_dev[n:], self._s_dev,
+                                      self._i_dev[n:], self._tokens, self._logprobs)
+        # one synchronising copy back: the scheduler needs the tokens to go on
+        return tokens[:R].tolist(), logprobs[:R].tolist()

@@ -1,0 +1,64 @@
+"""The entry point's loop (scheduler, step function, sampler) with the kernels replaced by their plain
+references: greedy generation equals the plain implementation's, also when pages run out."""
+import torch
+
+import plain_gemma2 as plain
+import tiny
+from simply_amd.engine.llm import LMInterface
+from simply_amd.sampling import SamplingParams
+
+
+def lm(d, **kw):
+    args = dict(activation_dtype="float32", batch_size=3, max_seq_len=64, page_size=4, max_num_issue_tokens=16,
+                device="cpu", use_graphs=False)
+    args.update(kw)
+    return LMInterface(d, **args)
+
+
+def test_greedy_generation_matches_plain(tmp_path, cpu_ops):
+    d = tiny.write_model("A", str(tmp_path / "A"), std=0.5)
+    w, cfg = plain.load(d)
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 50 + n) for n in (5, 11, 17)]
+    want = [plain.greedy(w, cfg, p, 8) for p in prompts]
+    params = SamplingParams(temperature=0.0, max_decode_steps=8)
+    outs = lm(d).generate(prompts, sampling_params=params)
+    assert [o.output_token_ids for o in outs] == want
+    assert all(o.finish_reason == "length" and o.is_truncated for o in outs)
+    assert all(lp == 0.0 for o in outs for lp in o.output_token_logprobs)
+    # so few pages that requests give way and are recomputed: the tokens stay the same
+    small = lm(d, total_num_pages=11)
+    outs2 = small.generate(prompts, sampling_params=params)
+    assert [o.output_token_ids for o in outs2] == want
+    assert small.stats["preemptions"] > 0
+    small.executor.cache.check()
+    assert all(g.pool.num_free == 11 for g in small.executor.cache.groups)
+
+
+def test_sampled_tokens_do_not_depend_on_the_batch(tmp_path, cpu_ops):
+    d = tiny.write_model("B", str(tmp_path / "B"), std=0.1)
+    _, cfg = plain.load(d)
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 70 + n) for n in (1, 9, 23, 40)]
+    plist = [SamplingParams(temperature=0.7, max_decode_steps=6, seed=1000 + i) for i in range(4)]
+    together = lm(d, batch_size=4).generate(prompts, sampling_params=plist)
+    alone = [lm(d, batch_size=1).generate([p], sampling_params=[sp])[0] for p, sp in zip(prompts, plist)]
+    assert [o.output_token_ids for o in together] == [o.output_token_ids for o in alone]
+    for a, b in zip(together, alone):
+        torch.testing.assert_close(torch.tensor(a.output_token_logprobs), torch.tensor(b.output_token_logprobs),
+                                   rtol=1e-4, atol=1e-4)
+    # another seed gives another continuation
+    other = lm(d, batch_size=1).generate([prompts[3]], sampling_params=[SamplingParams(temperature=0.7, max_decode_steps=6, seed=5)])
+    assert other[0].output_token_ids != together[3].output_token_ids
+
+
+def test_eos_stops(tmp_path, cpu_ops):
+    d = tiny.write_model("A", str(tmp_path / "A"), std=0.5)
+    w, cfg = plain.load(d)
+    prompt = tiny.random_tokens(6, cfg["vocab_size"], 3)
+    free_run = plain.greedy(w, cfg, prompt, 6)
+    import json, os
+    cfg["eos_token_id"] = free_run[2]
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    out = lm(d).generate(prompt, sampling_params=SamplingParams(temperature=0.0, max_decode_steps=6))[0]
+    stop = free_run.index(free_run[2]) + 1
+    assert out.output_token_ids == free_run[:stop] and out.finish_reason == "eos" and not out.is_truncated
