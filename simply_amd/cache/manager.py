@@ -205,7 +205,7 @@ class CacheView:
     need: PagedKVNeed | StateNeed | None
     group_id: int | None = None
     k_pages: torch.Tensor | None = None   # [num_pages, kv heads, page_size, head_dim]
-    v_pages: torch.Tensor | None = None
+    v_pages: torch.Tensor | None = None   # [num_pages, kv heads, head_dim, page_size]
     state: torch.Tensor | None = None     # [num_slots, *need.shape]
     write: bool = True                    # False: this entry reads the cache of another entry
 
@@ -250,10 +250,12 @@ class CacheManager:
                     self._group_entries[group.group_id] = []
                 view = CacheView(need, group.group_id)
                 if device is not None:
-                    shape = (self.num_pages, need.num_kv_heads, self.page_size, need.head_dim)
                     fill = float("nan") if poison else 0.0
-                    view.k_pages = torch.full(shape, fill, dtype=dtype, device=device)
-                    view.v_pages = torch.full(shape, fill, dtype=dtype, device=device)
+                    view.k_pages = torch.full((self.num_pages, need.num_kv_heads, self.page_size, need.head_dim), fill,
+                                              dtype=dtype, device=device)
+                    # values are stored transposed, so that the keys of a page are contiguous for each dimension
+                    view.v_pages = torch.full((self.num_pages, need.num_kv_heads, need.head_dim, self.page_size), fill,
+                                              dtype=dtype, device=device)
                 self._group_entries[group.group_id].append(i)
                 self.views.append(view)
             elif isinstance(need, StateNeed):

@@ -1,0 +1,321 @@
+// Paged attention in bfloat16 for requests that bring few query tokens (decode: one token): bound
+// by reading each request's keys and values once.
+//
+// One workgroup of four waves takes one (request, key/value head, range of keys).  All G query
+// heads of the key/value head and all of the request's q_len query tokens are the G * q_len <= 16
+// columns of one MFMA tile, so keys and values are read once for all of them.  Per tile of 32 keys a
+// wave computes
+//     S^T[key, row] = K[key, :] . Q[row, :]     v_mfma_f32_16x16x32_bf16, K rows as the A operand,
+//                                               loaded straight from the page (16 keys = 8 KiB)
+//     soft-cap, mask, running maximum and sum per row (float32)
+//     O^T[d, row]  += V^T[d, key] . P^T[key, row]
+// The second product needs no data movement: S^T comes out of the first MFMA in the register
+// layout that the second MFMA wants for its B operand, and value pages are stored transposed
+// ([hd, page_size]) so that the A operand is a plain load as well.  The four waves take tiles in
+// turn and merge their (maximum, sum, output) through LDS; key ranges are merged through a
+// workspace by the workgroup that finishes last, in a fixed order.
+#include "api.h"
+#include "common.h"
+
+namespace sa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+constexpr int kTile = 32;  // keys per MFMA tile
+
+__device__ inline float fast_tanh(float x) {
+  // tanh(x) = 1 - 2 / (exp(2x) + 1); exact at both ends, relative error ~1e-6 in between
+  const float e = __expf(2.f * x);
+  return 1.f - 2.f / (e + 1.f);
+}
+
+__device__ inline __bf16 to_bf16_raw(float f) {
+  const bf16 b = float_to_bf16(f);
+  return __builtin_bit_cast(__bf16, b.bits);
+}
+
+struct SeqMeta {
+  int slot, q_start, q_len, pos0;
+};
+
+// NDC = head size / 32
+template <int NDC>
+__global__ __launch_bounds__(256) void paged_attention_decode_kernel(
+    const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ seq_meta, int seq_begin,
+    bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
+    float* __restrict__ workspace, unsigned* __restrict__ counters) {
+  constexpr int HD = NDC * 32;
+  constexpr int NDB = HD / 16;  // output blocks of 16 dimensions
+  __shared__ float o_s[2][16][HD + 1];   // a wave's output [row][d], while two waves are merged
+  __shared__ float m_s[2][16], l_s[2][16];
+  __shared__ int is_last_s;
+
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int r = lane % 16, grp = lane / 16;
+  const int split = blockIdx.x, num_splits = gridDim.x, kh = blockIdx.y, seq = seq_begin + blockIdx.z;
+  const SeqMeta sm = seq_meta[seq];
+  const int rows = G * sm.q_len;  // <= 16
+  const int* table = block_table + static_cast<size_t>(sm.slot) * table_stride;
+
+  // this lane's row of the tile: query token qi, query head g of the group
+  const int qi = r / G, g = r % G;
+  const bool row_ok = r < rows;
+  const int pos_r = sm.pos0 + qi;
+  const int hi = sm.pos0 + sm.q_len;  // keys [lo, hi) are visible to some row
+  const int lo = (window > 0 && sm.pos0 - window + 1 > 0) ? sm.pos0 - window + 1 : 0;
+  const int lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
+
+  // tiles of 32 keys aligned to absolute positions; this workgroup's share, then this wave's
+  const int tile0 = lo / kTile, tile1 = (hi + kTile - 1) / kTile;
+  const int ntiles = tile1 - tile0;
+  const int tb = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * split / num_splits);
+  const int te = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * (split + 1) / num_splits);
+
+  // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
+  bf16x8 qf[NDC];
+  {
+    const bf16* qp = q + static_cast<size_t>(sm.q_start + (row_ok ? qi : 0)) * q_stride +
+                     static_cast<size_t>(kh * G + (row_ok ? g : 0)) * HD + grp * 8;
+#pragma unroll
+    for (int dc = 0; dc < NDC; ++dc)
+      qf[dc] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + dc * 32) : bf16x8{};
+  }
+
+  floatx4 acc[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;  // per row (lane % 16); l_run is this lane group's share
+
+  for (int tile = tb + wave; tile < te; tile += 4) {
+    const int key0 = tile * kTile;
+    // ---- scores of two sub-tiles of 16 keys
+    floatx4 s[2];
+    bool sub_ok[2];
+    const bf16* vbase[2];
+    int voff[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int sk0 = key0 + t * 16;                    // first key of the sub-tile
+      sub_ok[t] = sk0 < hi && sk0 + 16 > lo;            // wave-uniform
+      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+      vbase[t] = nullptr;
+      voff[t] = 0;
+      if (sub_ok[t]) {
+        const int page = table[sk0 / page_size];
+        const int off = sk0 % page_size;                // multiple of 16
+        const bf16* kp = k_pages + ((static_cast<size_t>(page) * Kh + kh) * page_size + off + r) * HD + grp * 8;
+        bf16x8 kf[NDC];
+#pragma unroll
+        for (int dc = 0; dc < NDC; ++dc) kf[dc] = *reinterpret_cast<const bf16x8*>(kp + dc * 32);
+#pragma unroll
+        for (int dc = 0; dc < NDC; ++dc) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[dc], qf[dc], s[t], 0, 0, 0);
+        vbase[t] = v_pages + (static_cast<size_t>(page) * Kh + kh) * HD * page_size;
+        voff[t] = off + grp * 4;
+      }
+    }
+    // ---- cap, mask, online softmax.  Lane (row r, grp) holds keys sk0 + 4 * grp + v of each sub-tile.
+    float p[2][4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int key = key0 + t * 16 + grp * 4 + v;
+        float x = s[t][v];
+        if (soft_cap > 0.f) x = soft_cap * fast_tanh(x / soft_cap);
+        const bool vis = sub_ok[t] && row_ok && key <= pos_r && key >= lo_r;
+        x = vis ? x : -INFINITY;
+        p[t][v] = x;
+        mx = fmaxf(mx, x);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m_run, mx);
+    // a row that has seen no visible key yet keeps m = -inf; exp(-inf - -inf) must not appear
+    const float alpha = m_new == -INFINITY ? 1.f : __expf(m_run - m_new);
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float e = p[t][v] == -INFINITY ? 0.f : __expf(p[t][v] - m_new);
+        psum += e;
+        pf[t * 4 + v] = to_bf16_raw(e);
+      }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    // ---- output: O^T[d][row] = alpha * O^T + V^T[d][keys] . P^T[keys][row]
+    // lane (d = r, grp) of the A operand holds V^T[db * 16 + r][the same 8 keys as pf]
+    const bool tail = key0 + kTile > hi;  // keys at or beyond hi may be unwritten: their values count as 0
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+      bf16x8 vf = {};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        if (sub_ok[t]) {
+          const bf16x4 x = *reinterpret_cast<const bf16x4*>(vbase[t] + static_cast<size_t>(db * 16 + r) * page_size +
+                                                           voff[t]);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) vf[t * 4 + v] = x[v];
+        }
+      }
+      if (tail) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int key = key0 + (e / 4) * 16 + grp * 4 + (e % 4);
+          if (key >= hi) vf[e] = to_bf16_raw(0.f);
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[db][v] *= alpha;
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[db], 0, 0, 0);
+    }
+  }
+
+  // ---- merge the four waves in two rounds through LDS (waves 2, 3 into 0, 1; then 1 into 0).
+  // acc[db][v] is O^T[d = db * 16 + 4 * grp + v][row r].
+  l_run += __shfl_xor(l_run, 16, kWave);
+  l_run += __shfl_xor(l_run, 32, kWave);
+  auto put = [&](int slot) {
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) o_s[slot][r][db * 16 + 4 * grp + v] = acc[db][v];
+    if (grp == 0) {
+      m_s[slot][r] = m_run;
+      l_s[slot][r] = l_run;
+    }
+  };
+  auto take = [&](int slot) {
+    const float m_o = m_s[slot][r], l_o = l_s[slot][r];
+    const float M = fmaxf(m_run, m_o);
+    const float a = m_run == -INFINITY ? 0.f : __expf(m_run - M);
+    const float b = m_o == -INFINITY ? 0.f : __expf(m_o - M);
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[db][v] = acc[db][v] * a + o_s[slot][r][db * 16 + 4 * grp + v] * b;
+    l_run = l_run * a + l_o * b;
+    m_run = M;
+  };
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave == 0) take(0);
+
+  const int KS = num_splits;
+  const size_t row_words = HD + 2;  // output, maximum, sum
+  const size_t unit = (static_cast<size_t>(blockIdx.z) * Kh + kh);
+  if (wave == 0 && row_ok) {
+    if (KS == 1) {
+      bf16* op = out + static_cast<size_t>(sm.q_start + qi) * out_stride + static_cast<size_t>(kh * G + g) * HD;
+      const float inv = 1.f / l_run;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) op[db * 16 + 4 * grp + v] = float_to_bf16(acc[db][v] * inv);
+    } else {
+      float* wp = workspace + ((unit * KS + split) * 16 + r) * row_words;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) wp[db * 16 + 4 * grp + v] = acc[db][v];
+      if (grp == 0) {
+        wp[HD] = m_run;
+        wp[HD + 1] = l_run;
+      }
+    }
+  }
+  if (KS == 1) return;
+  // ---- the workgroup that finishes last for this (request, head) adds the key ranges up, in their order
+  __threadfence();
+  __syncthreads();
+  if (tid == 0) is_last_s = atomicAdd(&counters[unit], 1u) == static_cast<unsigned>(KS - 1);
+  __syncthreads();
+  if (!is_last_s) return;
+  __threadfence();
+  if (tid == 0) counters[unit] = 0u;
+  const int orow = tid / 16, oc = tid % 16;  // thread -> (row, 16 threads over d)
+  if (orow >= rows) return;
+  const float* base = workspace + (unit * KS * 16 + orow) * row_words;
+  const size_t stride = 16 * row_words;
+  float Mg = -INFINITY;
+  for (int y = 0; y < KS; ++y) Mg = fmaxf(Mg, __builtin_nontemporal_load(base + y * stride + HD));
+  float Lg = 0.f;
+  for (int y = 0; y < KS; ++y) {
+    const float my = __builtin_nontemporal_load(base + y * stride + HD);
+    Lg += __builtin_nontemporal_load(base + y * stride + HD + 1) * (my == -INFINITY ? 0.f : __expf(my - Mg));
+  }
+  const int oq = orow / G, og = orow % G;
+  bf16* op = out + static_cast<size_t>(sm.q_start + oq) * out_stride + static_cast<size_t>(kh * G + og) * HD;
+  const float inv = 1.f / Lg;
+  for (int d = oc; d < HD; d += 16) {
+    float o = 0.f;
+    for (int y = 0; y < KS; ++y) {
+      const float my = __builtin_nontemporal_load(base + y * stride + HD);
+      o += __builtin_nontemporal_load(base + y * stride + d) * (my == -INFINITY ? 0.f : __expf(my - Mg));
+    }
+    op[d] = float_to_bf16(o * inv);
+  }
+}
+
+bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q) {
+  const int G = H / Kh;
+  return (hd == 64 || hd == 128 || hd == 256) && page_size % 16 == 0 && G * max_q_len <= 16 && q_stride % 8 == 0 &&
+         (reinterpret_cast<uintptr_t>(q) & 15u) == 0;
+}
+
+int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                           const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
+                           void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
+                           float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
+                           void* counters, int num_counters, hipStream_t stream) {
+  if (seq_count == 0) return 0;
+  const int G = H / Kh;
+  const int units = seq_count * Kh;
+  int span = window > 0 && window < max_kv_len ? window + 16 : max_kv_len;  // keys a request reads at most
+  if (span < 1) span = 1;
+  const int max_tiles = (span + kTile - 1) / kTile + 1;
+  int KS = num_splits;
+  if (KS <= 0) {
+    KS = (256 * 4 + units - 1) / units;      // about four workgroups per CU
+    const int cap_by_work = (max_tiles + 7) / 8;  // at least 8 tiles (256 keys) per workgroup
+    if (KS > cap_by_work) KS = cap_by_work;
+  }
+  if (KS > max_tiles) KS = max_tiles;
+  if (KS < 1) KS = 1;
+  const size_t per_split = static_cast<size_t>(units) * 16 * (hd + 2) * sizeof(float);
+  while (KS > 1 && (workspace == nullptr || counters == nullptr || units > num_counters ||
+                    per_split * KS > workspace_bytes))
+    --KS;
+  const dim3 grid(KS, Kh, seq_count);
+  const bf16* qp = static_cast<const bf16*>(q);
+  const bf16* kp = static_cast<const bf16*>(k_pages);
+  const bf16* vp = static_cast<const bf16*>(v_pages);
+  const SeqMeta* sm = reinterpret_cast<const SeqMeta*>(seq_meta);
+  bf16* op = static_cast<bf16*>(out);
+  float* ws = static_cast<float*>(workspace);
+  unsigned* cn = static_cast<unsigned*>(counters);
+#define SA_LAUNCH(NDC)                                                                                              \
+  paged_attention_decode_kernel<NDC><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, sm, \
+                                                               seq_begin, op, out_stride, Kh, G, page_size, window,  \
+                                                               soft_cap, ws, cn)
+  if (hd == 64) SA_LAUNCH(2);
+  else if (hd == 128) SA_LAUNCH(4);
+  else if (hd == 256) SA_LAUNCH(8);
+  else {
+    set_error("paged_attention_decode: head size %d is not 64, 128 or 256", hd);
+    return 1;
+  }
+#undef SA_LAUNCH
+  return check_launch("paged_attention_decode");
+}
+
+}  // namespace sa

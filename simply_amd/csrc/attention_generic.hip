@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
           for (int j = jlo; j < jhi; ++j) {
             const int key = c0 + j;
             const float v = to_float(
-                v_pages[((static_cast<size_t>(page_s[j]) * Kh + kh) * page_size + key % page_size) * hd + d]);
+                v_pages[((static_cast<size_t>(page_s[j]) * Kh + kh) * hd + d) * page_size + key % page_size]);
 #pragma unroll
             for (int g = 0; g < 8; ++g)
               if (g < gn) acc[s][g] = fmaf(s_s[(g0 + g) * kChunk + j], v, acc[s][g]);

@@ -77,7 +77,7 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
 // One block per (token, head) of a fused [T, (H + 2K) * hd] projection.
 //   q heads: rotate, divide by query_scale, write back in place.
 //   k heads: rotate, write into the key pages at slot_mapping[t].
-//   v heads: copy into the value pages.
+//   v heads: copy into the value pages (stored transposed: [page, head, hd, page_size]).
 // Angles: pos / timescale[i] / scale_factor, pairs (i, i + hd/2).  simply/utils/position_encoding.py:83-110;
 // the query scale comes after the rotation (simply/model_lib.py:2010-2019).
 template <typename T>
@@ -122,8 +122,9 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
     const int64_t slot = slot_mapping[t];
     if (slot < 0) return;
     const int64_t page = slot / page_size, off = slot % page_size;
-    T* dst = v_pages + ((page * K + (head - H - K)) * page_size + off) * hd;
-    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+    // value pages are [page, head, hd, page_size]: the keys of a page are contiguous for each dimension
+    T* dst = v_pages + (page * K + (head - H - K)) * page_size * hd + off;
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[static_cast<size_t>(i) * page_size] = src[i];
   }
 }
 

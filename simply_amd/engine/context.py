@@ -26,8 +26,9 @@ class StepContext:
     num_tokens: int
     positions: torch.Tensor       # int32 [T] absolute position of each token in its request
     token_seq: torch.Tensor       # int32 [T] slot of each token's request (block-table row, state row)
+    seq_meta: torch.Tensor        # int32 [S, 4] per request: slot, index of its first token, its tokens, position of the first
     groups: dict[int, GroupStep]
-    # host-side description, in the order of the tokens
+    # host-side description, in the order of the tokens: requests with fewer tokens come first
     request_ids: list[Hashable]
     seq_slots: list[int]          # slot of each request
     seq_starts: list[int]         # tokens of the request that earlier steps have run
@@ -40,4 +41,16 @@ class StepContext:
 
     @property
     def max_q_len(self) -> int:
-        return max(self.q_lens) if self.q_lens else 0
+        return self.q_lens[-1] if self.q_lens else 0
+
+    @property
+    def max_kv_len(self) -> int:
+        """The most keys that any request of the step may attend to."""
+        return max(s + q for s, q in zip(self.seq_starts, self.q_lens))
+
+    def short_requests(self, max_tokens: int) -> tuple[int, int]:
+        """(number of leading requests with at most max_tokens tokens, number of their tokens)."""
+        n = 0
+        while n < len(self.q_lens) and self.q_lens[n] <= max_tokens:
+            n += 1
+        return n, self.cu_q_lens[n]

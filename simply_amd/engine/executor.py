@@ -48,7 +48,8 @@ class Executor:
         cap = max(config.issue_budget, config.batch_size)
         self._cap = cap
         ngroups = len(self.cache.groups)
-        self._words = cap * (4 + 2 * ngroups)
+        self._meta_at = cap * (4 + 2 * ngroups)          # [batch_size, 4] request descriptors after the token arrays
+        self._words = self._meta_at + 4 * config.batch_size
         self._on_gpu = self.device.type == "cuda"
         self._host = torch.empty(self._words, dtype=torch.int32, pin_memory=self._on_gpu)
         self._dev = torch.empty(self._words, dtype=torch.int32, device=self.device)
@@ -99,6 +100,11 @@ class Executor:
         # forget what is known of requests that have left the cache since (finished or preempted elsewhere)
         for rid in [r for r in self.num_computed if r not in self.cache.requests]:
             del self.num_computed[rid]
+        # requests with few tokens first (the attention kernels take them as one range); `order` remembers
+        # where each entry went so that the logits come back in the callers' order
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens))
+        if len(entries) > self.config.batch_size:
+            raise ValueError(f"{len(entries)} requests in one step, batch_size is {self.config.batch_size}")
         wants = [(e.request_id, self._start_of(e), len(e.tokens)) for e in entries]
         if not cache.can_reserve(wants):
             from ..cache import OutOfPages
@@ -113,10 +119,12 @@ class Executor:
         host = self._host.numpy()
         tok, pos, seq, rows = (host[i * cap:(i + 1) * cap] for i in range(4))
         slot_maps = [host[(4 + 2 * g) * cap:(6 + 2 * g) * cap].view(np.int64) for g in range(len(cache.groups))]
+        meta = host[self._meta_at:self._meta_at + 4 * len(entries)].reshape(len(entries), 4)
         ctx_ids, ctx_slots, ctx_starts, ctx_q, cu = [], [], [], [], [0]
-        R = 0
+        first_token = [0] * len(entries)
         t0 = 0
-        for e, (rid, start, q) in zip(entries, wants):
+        for j, i in enumerate(order):
+            e, (rid, start, q) = entries[i], wants[i]
             ids = np.asarray(e.tokens, dtype=np.int64)
             if ids.min() < 0 or ids.max() >= self.vocab_size:
                 raise ValueError(f"request {rid!r}: token id outside [0, {self.vocab_size})")
@@ -124,17 +132,22 @@ class Executor:
             tok[t0:t0 + q] = ids
             pos[t0:t0 + q] = np.arange(start, start + q)
             seq[t0:t0 + q] = slot
+            meta[j] = (slot, t0, q, start)
             for g in cache.groups:
                 slot_maps[g.group_id][t0:t0 + q] = cache.slot_mapping(g.group_id, rid, start, q)
                 cache.check_readable(g.group_id, rid, start, q)
-            for w in e.want:
-                if not 0 <= w < q:
-                    raise ValueError(f"request {rid!r}: wanted place {w} is outside its {q} tokens")
-                rows[R] = t0 + w
-                R += 1
+            first_token[i] = t0
             ctx_ids.append(rid); ctx_slots.append(slot); ctx_starts.append(start); ctx_q.append(q)
             t0 += q
             cu.append(t0)
+        R = 0
+        for i, e in enumerate(entries):
+            q = len(e.tokens)
+            for w in e.want:
+                if not 0 <= w < q:
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is outside its {q} tokens")
+                rows[R] = first_token[i] + w
+                R += 1
         tables = cache.sync_tables()
         self._dev.copy_(self._host, non_blocking=True)
         if self._copied is not None:
@@ -144,6 +157,7 @@ class Executor:
                                         dev[(4 + 2 * g.group_id) * cap:(6 + 2 * g.group_id) * cap].view(torch.int64)[:T])
                   for g in cache.groups}
         ctx = StepContext(dtype=self.dtype, num_tokens=T, positions=dev[cap:cap + T], token_seq=dev[2 * cap:2 * cap + T],
+                          seq_meta=dev[self._meta_at:self._meta_at + 4 * len(entries)].view(len(entries), 4),
                           groups=groups, request_ids=ctx_ids, seq_slots=ctx_slots, seq_starts=ctx_starts, q_lens=ctx_q,
                           cu_q_lens=cu)
         logit_rows = dev[3 * cap:3 * cap + R] if R else None

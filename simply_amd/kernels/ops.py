@@ -16,7 +16,7 @@ from .lib import KernelError
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
-ALGO_AUTO, ALGO_GENERIC = 0, 1
+ALGO_AUTO, ALGO_GENERIC, ALGO_SKINNY, ALGO_TILED = 0, 1, 2, 3
 
 
 def _code(t: torch.Tensor) -> int:
@@ -126,6 +126,18 @@ def add_rmsnorm(y: torch.Tensor, residual: torch.Tensor, *, post_weight: torch.T
     return out
 
 
+def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtype, what: str) -> int:
+    """Key pages [pages, K, page_size, hd], value pages [pages, K, hd, page_size]; returns page_size."""
+    if k_pages.dim() != 4 or v_pages.dim() != 4 or not k_pages.is_contiguous() or not v_pages.is_contiguous() \
+            or k_pages.dtype != dtype or v_pages.dtype != dtype:
+        raise KernelError(f"{what}: pages must be contiguous 4-D tensors of {dtype}")
+    n, K, P, hd = k_pages.shape
+    if tuple(v_pages.shape) != (n, K, hd, P):
+        raise KernelError(f"{what}: key pages {tuple(k_pages.shape)} want value pages {(n, K, hd, P)}, "
+                          f"got {tuple(v_pages.shape)}")
+    return P
+
+
 def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, timescale: torch.Tensor | None, scale_factor: float,
                      q_div: float, num_heads: int, num_kv_heads: int, head_dim: int,
                      slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
@@ -145,12 +157,10 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, timescale: torc
     if k_pages is not None:
         if v_pages is None or slot_mapping is None:
             raise KernelError("rope_cache_write: key pages, value pages and slots come together")
-        for p in (k_pages, v_pages):
-            if p.dim() != 4 or p.shape[1] != num_kv_heads or p.shape[3] != head_dim or not p.is_contiguous() \
-                    or p.dtype != qkv.dtype or p.shape != k_pages.shape:
-                raise KernelError(f"rope_cache_write: pages must be contiguous [pages, {num_kv_heads}, page_size, "
-                                  f"{head_dim}] of {qkv.dtype}, got {tuple(p.shape)} {p.dtype}")
-        page_size = k_pages.shape[2]
+        page_size = _check_pages(k_pages, v_pages, qkv.dtype, "rope_cache_write")
+        if k_pages.shape[1] != num_kv_heads or k_pages.shape[3] != head_dim:
+            raise KernelError(f"rope_cache_write: pages {tuple(k_pages.shape)} do not match {num_kv_heads} heads of "
+                              f"size {head_dim}")
         if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
             raise KernelError("rope_cache_write: slot_mapping must be int64 [T]")
     _lib.call("sa_rope_cache_write", _ptr(qkv), _code(qkv), stride, _ptr(positions), _ptr(timescale),
@@ -201,9 +211,23 @@ def fill_(t: torch.Tensor, value_bits: int = 0) -> None:
 
 EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
 
+#: scratch memory of kernels that cut K over workgroups, one per device, allocated at the first product
+WORKSPACE_BYTES = 64 << 20
+NUM_COUNTERS = 1 << 16
+_scratch: dict = {}
+
+
+def _workspace(device):
+    key = (device.type, device.index)
+    if key not in _scratch:
+        _scratch[key] = (torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device),
+                         torch.zeros(NUM_COUNTERS, dtype=torch.int32, device=device))
+    return _scratch[key]
+
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: torch.Tensor | None = None, soft_cap: float | None = None,
-         out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None, algo: int = ALGO_AUTO) -> torch.Tensor:
+         out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None, algo: int = ALGO_AUTO,
+         splits: int = 0) -> torch.Tensor:
     """a[M, K] . w[N, K]^T.  With w2: gelu_tanh(a.w^T) * (a.w2^T).  With soft_cap: cap * tanh(. / cap)."""
     _dev(a, w, w2, out)
     lda = _rows(a, "gemm: a")
@@ -227,8 +251,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: torch.Tensor | None = None, so
     if tuple(out.shape) != (M, N):
         raise KernelError("gemm: bad output shape")
     ldc = _rows(out, "gemm: out")
+    ws, counters = _workspace(a.device)
     _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(w), _ptr(w2), _code(w), _ptr(out), _code(out), ldc, M, N, K, epi,
-              cap, algo, _stream())
+              cap, algo, _ptr(ws), ws.numel(), _ptr(counters), counters.numel(), int(splits), _stream())
     return out
 
 
@@ -242,9 +267,7 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
     _dev(q, k_pages, v_pages, block_table, token_seq, positions, out)
     q_stride = _rows(q, "paged_attention: q")
     T = q.shape[0]
-    if k_pages.dim() != 4 or k_pages.shape != v_pages.shape or not k_pages.is_contiguous() \
-            or not v_pages.is_contiguous() or k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
-        raise KernelError("paged_attention: pages must be contiguous [pages, K, page_size, hd] of the query's type")
+    _check_pages(k_pages, v_pages, q.dtype, "paged_attention")
     num_pages, Kh, page_size, hd = k_pages.shape
     if q.shape[1] < num_heads * hd:
         raise KernelError("paged_attention: query rows are shorter than heads * head size")
@@ -260,6 +283,42 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
     _lib.call("sa_paged_attention", _ptr(q), _code(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
               block_table.stride(0), _ptr(token_seq), _ptr(positions), _ptr(out), out_stride, T, num_heads, Kh, hd,
               page_size, int(window or 0), float(soft_cap or 0.0), algo, _stream())
+    return out
+
+
+def decode_attention_takes(q: torch.Tensor, k_pages: torch.Tensor, num_heads: int, max_q_len: int) -> bool:
+    """Whether `paged_attention_decode` takes requests of up to max_q_len tokens at these sizes."""
+    _, Kh, page_size, hd = k_pages.shape
+    G = num_heads // Kh
+    return (q.dtype == torch.bfloat16 and hd in (64, 128, 256) and page_size % 16 == 0 and G * max_q_len <= 16
+            and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
+
+
+def paged_attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                           seq_meta: torch.Tensor, seq_begin: int, seq_count: int, num_heads: int, *,
+                           window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
+                           out: torch.Tensor, num_splits: int = 0) -> torch.Tensor:
+    """Attention of requests seq_begin .. seq_begin + seq_count - 1 of seq_meta, each with few tokens
+    ((heads per key head) * tokens <= 16).  q and out are the whole step's rows."""
+    _dev(q, k_pages, v_pages, block_table, seq_meta, out)
+    if q.dtype != torch.bfloat16:
+        raise KernelError("paged_attention_decode: bfloat16 only")
+    q_stride = _rows(q, "paged_attention_decode: q")
+    _check_pages(k_pages, v_pages, q.dtype, "paged_attention_decode")
+    _, Kh, page_size, hd = k_pages.shape
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("paged_attention_decode: block_table must be int32 [sequences, blocks]")
+    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
+            or seq_begin < 0 or seq_begin + seq_count > seq_meta.shape[0]:
+        raise KernelError("paged_attention_decode: seq_meta must be int32 [S, 4] covering the requested range")
+    if out.dtype != q.dtype or out.shape[0] != q.shape[0] or out.shape[1] != num_heads * hd:
+        raise KernelError("paged_attention_decode: bad output")
+    out_stride = _rows(out, "paged_attention_decode: out")
+    ws, counters = _workspace(q.device)
+    _lib.call("sa_paged_attention_decode", _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+              block_table.stride(0), _ptr(seq_meta), seq_begin, seq_count, _ptr(out), out_stride, num_heads, Kh, hd,
+              page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
+              _ptr(ws), ws.numel(), _ptr(counters), counters.numel(), _stream())
     return out
 
 

@@ -66,6 +66,17 @@ class PagedAttention(Mixer):
             ops.rope_cache_write(qkv, ctx.positions, None, 1.0, self.query_scale, H, K, hd,
                                  slot_mapping=group.slot_mapping if write else None,
                                  k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
-        o = ops.paged_attention(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions,
-                                H, window=self.window, soft_cap=self.soft_cap)
+        o = torch.empty((qkv.shape[0], H * hd), dtype=qkv.dtype, device=qkv.device)
+        # requests with few tokens (decode) go to the kernel that reads each request's keys once for all of its
+        # query heads; the others to the kernel for portions of prompts
+        n_short = t_short = 0
+        if ops.decode_attention_takes(qkv, cache.k_pages, H, 1):
+            n_short, t_short = ctx.short_requests(16 // (H // K))
+        if n_short:
+            ops.paged_attention_decode(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.seq_meta, 0, n_short, H,
+                                       window=self.window, soft_cap=self.soft_cap, max_kv_len=ctx.max_kv_len,
+                                       max_q_len=ctx.q_lens[n_short - 1], out=o)
+        if t_short < ctx.num_tokens:
+            ops.paged_attention(qkv[t_short:], cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq[t_short:],
+                                ctx.positions[t_short:], H, window=self.window, soft_cap=self.soft_cap, out=o[t_short:])
         return ops.gemm(o, self.o_proj)

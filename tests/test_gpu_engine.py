@@ -64,3 +64,19 @@ def test_cuts_match_plain(tmp_path, name, dtype):
         assert torch.isfinite(got).all()
         err = (got - want).abs().max().item() / scale
         assert err <= TOL[dtype], (cuts, err)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_match_plain_at_kernel_sizes(tmp_path, dtype):
+    """Head size 64 and pages of 16: the sizes at which the bfloat16 path runs its MFMA kernels."""
+    d = tiny.write_model("D", str(tmp_path / "D"), std=0.15)
+    vocab = plain.load(d)[1]["vocab_size"]
+    tokens = tiny.random_tokens(150, vocab, 8)
+    want, cfg = plain_logits(d, tokens, dtype)
+    scale = want.abs().max().item()
+    ex = make_executor(d, dtype, page_size=16, num_pages=24, max_len=320)
+    for cuts in ([150], [118] + [1] * 32, [40, 7, 5, 3, 2, 30, 2, 2, 13, 17, 2, 27], [1] * 150, [3, 4, 2] * 16 + [6]):
+        got = run_cut(ex, "r", tokens, cuts).double()
+        assert torch.isfinite(got).all()
+        err = (got - want).abs().max().item() / scale
+        assert err <= TOL[dtype], (cuts, err)

@@ -78,7 +78,7 @@ def test_rope_cache_write(dtype, H, K, hd, P):
     positions = torch.tensor([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7], dtype=torch.int32).cuda()
     ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda()
     slots = torch.randperm(pages * P)[:T].to(torch.int64).cuda()
-    kp, vp = (torch.zeros((pages, K, P, hd), dtype=dtype).cuda() for _ in range(2))
+    kp, vp = torch.zeros((pages, K, P, hd), dtype=dtype).cuda(), torch.zeros((pages, K, hd, P), dtype=dtype).cuda()
     kp2, vp2, qkv2 = kp.clone(), vp.clone(), qkv.clone()
     ops.rope_cache_write(qkv, positions, ts, 1.0, 12.0, H, K, hd, slots, kp, vp)
     ref.rope_cache_write(qkv2, positions, ts, 1.0, 12.0, H, K, hd, slots, kp2, vp2)
@@ -129,14 +129,14 @@ def paged_setup(dtype, S, H, Kh, hd, P, lens, seed):
     perm = torch.randperm(num_pages, generator=g).tolist()
     table = torch.full((S, max_blocks), -1, dtype=torch.int32)
     kp = torch.full((num_pages, Kh, P, hd), float("nan"), dtype=dtype)
-    vp = torch.full((num_pages, Kh, P, hd), float("nan"), dtype=dtype)
+    vp = torch.full((num_pages, Kh, hd, P), float("nan"), dtype=dtype)
     for s, l in enumerate(lens):
         for b in range(-(-l // P)):
             page = perm.pop()
             table[s, b] = page
             n = min(P, l - b * P)
             kp[page, :, :n] = torch.randn((Kh, n, hd), generator=g).to(dtype)
-            vp[page, :, :n] = torch.randn((Kh, n, hd), generator=g).to(dtype)
+            vp[page, :, :, :n] = torch.randn((Kh, hd, n), generator=g).to(dtype)
     return kp.cuda(), vp.cuda(), table.cuda()
 
 
@@ -177,7 +177,7 @@ def test_paged_attention_far_key_and_window_edge():
     page, off = int(table[0, far // P]), far % P
     kp[page, 0, off] = 0.0
     kp[page, 0, off, 3] = 50.0
-    vp[page, 0, off] = 7.0
+    vp[page, 0, :, off] = 7.0
     q = torch.zeros((1, hd)).cuda()
     q[0, 3] = 1.0
     ts = torch.zeros(1, dtype=torch.int32).cuda()
@@ -224,3 +224,101 @@ def test_sampling_frequencies():
     p = torch.softmax(base.double() / T, -1)
     sigma = torch.sqrt(p * (1 - p) / n)
     assert ((freq - p).abs() < 4 * sigma).all(), (freq, p)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(48, 64), (100, 72), (2304, 2048), (333, 1000), (4096, 2304)])
+def test_gemm_skinny(M, N, K):
+    """The few-rows bfloat16 kernel, also with K cut over several workgroups (partials through the workspace)."""
+    from simply_amd.kernels import ops
+    a, w, w2 = rand((M, K), torch.bfloat16, 50), rand((N, K), torch.bfloat16, 51, 0.05), rand((N, K), torch.bfloat16, 52, 0.05)
+    for splits in (0, 4, 16):
+        kw = dict(algo=ops.ALGO_SKINNY, splits=splits)
+        torch.testing.assert_close(ops.gemm(a, w, **kw).float(), ref.gemm(a, w).float(), rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(ops.gemm(a, w, w2=w2, **kw).float(), ref.gemm(a, w, w2=w2).float(), rtol=2e-2, atol=2e-2)
+        got = ops.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32, **kw)
+        torch.testing.assert_close(got, ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+    # the same call twice gives the same bits (the order of the partial sums is fixed)
+    assert torch.equal(ops.gemm(a, w, algo=ops.ALGO_SKINNY, splits=16), ops.gemm(a, w, algo=ops.ALGO_SKINNY, splits=16))
+    # a view with a row stride, as the attention output is
+    wide = rand((M, K + 16), torch.bfloat16, 53)
+    torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], w, algo=ops.ALGO_SKINNY).float(), ref.gemm(wide[:, 8:8 + K], w).float(),
+                               rtol=2e-2, atol=2e-2)
+
+
+def test_gemm_skinny_refuses_what_it_does_not_take():
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.lib import KernelError
+    a, w = rand((4, 100), torch.bfloat16, 54), rand((8, 100), torch.bfloat16, 55)   # K is no multiple of 8
+    with pytest.raises(KernelError, match="few-rows"):
+        ops.gemm(a, w, algo=ops.ALGO_SKINNY)
+    torch.testing.assert_close(ops.gemm(a, w).float(), ref.gemm(a, w).float(), rtol=2e-2, atol=2e-2)   # auto falls back
+    with pytest.raises(KernelError):
+        ops.gemm(rand((65, 64), torch.bfloat16, 56), rand((8, 64), torch.bfloat16, 57), algo=ops.ALGO_SKINNY)
+
+
+def seq_meta_for(lens, q_lens):
+    """Requests whose last q tokens are this step's; returns (meta [S, 4], token_seq, positions)."""
+    meta, token_seq, positions, t0 = [], [], [], 0
+    for s, (l, q) in enumerate(zip(lens, q_lens)):
+        meta.append((s, t0, q, l - q))
+        token_seq += [s] * q
+        positions += list(range(l - q, l))
+        t0 += q
+    return (torch.tensor(meta, dtype=torch.int32).cuda(), torch.tensor(token_seq, dtype=torch.int32).cuda(),
+            torch.tensor(positions, dtype=torch.int32).cuda())
+
+
+@pytest.mark.parametrize("H,Kh,hd,P,window,cap", [
+    (8, 4, 256, 16, None, 50.0), (8, 4, 256, 16, 100, 50.0), (4, 2, 64, 16, 33, None), (16, 1, 128, 32, None, 30.0),
+    (2, 2, 128, 64, 200, None), (6, 3, 64, 16, 1, 20.0), (32, 16, 128, 16, 500, 50.0)])
+@pytest.mark.parametrize("splits", [0, 1, 5])
+def test_paged_attention_decode(H, Kh, hd, P, window, cap, splits):
+    """The few-tokens bfloat16 kernel against the plain reference: lengths around page and tile edges, one
+    to several tokens per request, unwritten page tails holding NaN, keys cut over workgroups."""
+    from simply_amd.kernels import ops
+    G = H // Kh
+    lens = [1, 16, 17, 33, 250, 700, 64, 1000]
+    max_q = max(1, 16 // G)
+    q_lens = [min(l, 1 + (i * 3) % max_q) for i, l in enumerate(lens)]
+    order = sorted(range(len(lens)), key=lambda i: q_lens[i])
+    lens, q_lens = [lens[i] for i in order], [q_lens[i] for i in order]
+    kp, vp, table = paged_setup(torch.bfloat16, len(lens), H, Kh, hd, P, lens, 61)
+    meta, ts, ps = seq_meta_for(lens, q_lens)
+    T = ts.numel()
+    q = rand((T, (H + 2 * Kh) * hd), torch.bfloat16, 62, 0.3)
+    out = torch.zeros((T, H * hd), dtype=torch.bfloat16).cuda()
+    assert ops.decode_attention_takes(q, kp, H, max(q_lens))
+    ops.paged_attention_decode(q, kp, vp, table, meta, 0, len(lens), H, window=window, soft_cap=cap,
+                               max_kv_len=max(lens), max_q_len=max(q_lens), out=out, num_splits=splits)
+    want = ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap)
+    assert torch.isfinite(out.float()).all()
+    torch.testing.assert_close(out.float(), want.float(), rtol=2e-2, atol=2e-2)
+    # a sub-range of the requests: the others' rows stay untouched
+    out2 = torch.full_like(out, 7.0)
+    ops.paged_attention_decode(q, kp, vp, table, meta, 2, 3, H, window=window, soft_cap=cap, max_kv_len=max(lens),
+                               max_q_len=max(q_lens), out=out2, num_splits=splits)
+    a, b = int(meta[2, 1]), int(meta[4, 1] + meta[4, 2])
+    assert torch.equal(out2[a:b], out[a:b]) and (out2[:a] == 7).all() and (out2[b:] == 7).all()
+
+
+def test_paged_attention_decode_far_key():
+    """A key 3000 positions back with a score that stands out, among keys cut over many workgroups."""
+    from simply_amd.kernels import ops
+    H, Kh, hd, P, L = 2, 1, 128, 16, 3100
+    kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 63)
+    kp.mul_(0.01)
+    far = 71
+    page, off = int(table[0, far // P]), far % P
+    kp[page, 0, off] = 0.0
+    kp[page, 0, off, 5] = 60.0
+    vp[page, 0, :, off] = 3.0
+    meta, ts, ps = seq_meta_for([L], [1])
+    q = torch.zeros((1, 4 * hd), dtype=torch.bfloat16).cuda()
+    q[0, 5] = 1.0
+    q[0, hd + 5] = 1.0
+    for window, sees in ((None, True), (L - far, True), (L - far - 1, False)):
+        out = torch.zeros((1, H * hd), dtype=torch.bfloat16).cuda()
+        ops.paged_attention_decode(q, kp, vp, table, meta, 0, 1, H, window=window, soft_cap=None, max_kv_len=L,
+                                   max_q_len=1, out=out)
+        assert (abs(out.float().mean().item() - 3.0) < 0.05) == sees, (window, out.float().mean().item())

@@ -30,7 +30,15 @@ TINY_C = dict(
     layer_types=["full_attention", "sliding_attention", "sliding_attention", "full_attention"],
     hidden_activation="gelu_pytorch_tanh", initializer_range=0.08,
 )
-CONFIGS = {"A": (TINY_A, 0, 0.1), "B": (TINY_B, 1, 0.2), "C": (TINY_C, 2, 0.3)}
+# sizes that the bfloat16 MFMA kernels take (head size 64, pages of 16), still tiny
+TINY_D = dict(
+    architectures=["Gemma2ForCausalLM"], hidden_size=128, num_hidden_layers=3, num_attention_heads=4,
+    num_key_value_heads=2, head_dim=64, intermediate_size=256, vocab_size=1000, rms_norm_eps=1e-6,
+    rope_theta=10000.0, sliding_window=40, query_pre_attn_scalar=64, attn_logit_softcapping=50.0,
+    final_logit_softcapping=30.0, tie_word_embeddings=True, max_position_embeddings=1024,
+    hidden_activation="gelu_pytorch_tanh", initializer_range=0.05,
+)
+CONFIGS = {"A": (TINY_A, 0, 0.1), "B": (TINY_B, 1, 0.2), "C": (TINY_C, 2, 0.3), "D": (TINY_D, 3, 0.1)}
 
 
 def write_model(name: str, out_dir: str, dtype=torch.float32, std: float | None = None) -> str:

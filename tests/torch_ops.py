@@ -14,7 +14,7 @@ import torch
 PRECISE = False
 
 EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
-ALGO_AUTO, ALGO_GENERIC = 0, 1
+ALGO_AUTO, ALGO_GENERIC, ALGO_SKINNY, ALGO_TILED = 0, 1, 2, 3
 
 
 def _f(t: torch.Tensor) -> torch.Tensor:
@@ -74,7 +74,7 @@ def rope_cache_write(qkv, positions, timescale, scale_factor, q_div, num_heads, 
         P = k_pages.shape[2]
         page, off = slot_mapping[:T] // P, slot_mapping[:T] % P
         k_pages[page, :, off] = k.to(k_pages.dtype)
-        v_pages[page, :, off] = v.to(v_pages.dtype)
+        v_pages[page, :, :, off] = v.to(v_pages.dtype)     # value pages are [page, head, hd, page_size]
 
 
 def rope(x, positions, timescale, scale_factor, div, num_heads, head_dim):
@@ -100,7 +100,7 @@ def gelu_tanh(x):
     return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
 
 
-def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0):
+def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, splits=0):
     out_dtype = out_dtype or a.dtype
     c = _f(a) @ _f(w).T
     if w2 is not None:
@@ -129,7 +129,7 @@ def paged_attention(q, k_pages, v_pages, block_table, token_seq, positions, num_
         pages = block_table[int(token_seq[t]), keys // P].long()
         assert (pages >= 0).all(), "attention reads a key that has no page"
         k = _f(k_pages[pages, :, keys % P])          # [n, Kh, hd]
-        v = _f(v_pages[pages, :, keys % P])
+        v = _f(v_pages[pages, :, :, keys % P])       # [n, Kh, hd]
         qt = _f(q[t, :H * hd]).reshape(Kh, G, hd)
         s = torch.einsum("kgd,nkd->kgn", qt, k)
         if soft_cap:
@@ -140,6 +140,10 @@ def paged_attention(q, k_pages, v_pages, block_table, token_seq, positions, num_
         out.copy_(res)
         return out
     return res
+
+
+def decode_attention_takes(q, k_pages, num_heads, max_q_len):
+    return False
 
 
 # ---- sampling: the same counter-based generator as the kernel, in integer arithmetic
