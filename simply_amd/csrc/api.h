@@ -13,8 +13,9 @@ const char* sa_last_error();
 int sa_version();
 
 // out[t, :] = table[tokens[t], :] * scale (32-bit output: the residual stream).
+// packed: the table is tiled like a matrix-product weight (see sa_gemm).
 int sa_embed(const void* table, int table_dtype, const int* tokens, float* out, int T, int D, int V, float scale,
-             hipStream_t stream);
+             int packed, hipStream_t stream);
 
 // out = x * rsqrt(mean(x^2) + eps) * (w + plus_one), row by row.
 int sa_rmsnorm(const void* x, int x_dtype, int64_t x_stride, const void* w, int w_dtype, void* out, int out_dtype,
@@ -44,11 +45,13 @@ int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t stream);
 // C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1: gelu_tanh(A.W^T) * (A.W2^T);
 // 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
 // few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel (2 and 3 refuse what they do not take).
-// workspace (bytes) and counters (32-bit words, zero before the first call and left zero by every
-// call) are scratch memory for kernels that cut K over workgroups; splits > 0 fixes the number of cuts.
+// packed: W (and W2) are tiled instead of row-major: [ceil(N / 16)][ceil(K / 32)][64][8] bfloat16, block (i, j)
+// holding rows 16 i .. 16 i + 15 and columns 32 j .. 32 j + 31 as element [(k % 32) / 8 * 16 + n % 16][k % 8],
+// zero beyond N and K (one MFMA operand per block, in register order).
+// shape > 0 fixes how the few-rows kernel cuts its work: rows of W per workgroup (4, 8 or 16) * 100 + waves.
 int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C, int c_dtype,
-            int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, void* workspace,
-            int64_t workspace_bytes, void* counters, int num_counters, int splits, hipStream_t stream);
+            int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, int packed, int shape,
+            hipStream_t stream);
 
 // Attention of T query tokens over paged keys and values.
 //   q[t, h, :] at q + t * q_stride + h * hd; key pages are [num_pages, Kh, page_size, hd], value pages
@@ -65,13 +68,12 @@ int sa_paged_attention(const void* q, int dtype, int64_t q_stride, const void* k
 // row, index of the request's first token in this step, number of its tokens, position of its first token), each
 // with (query heads per key head) * tokens <= 16: bfloat16, head size 64, 128 or 256, page size a multiple of 16.
 // max_kv_len bounds the keys of any of them (for the choice of how many ways to cut the keys; num_splits > 0 fixes
-// it).  workspace and counters as for sa_gemm.
+// it).  workspace (bytes): scratch memory for the partial results of the key ranges.
 int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                               const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
                               int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
                               int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
-                              void* workspace, int64_t workspace_bytes, void* counters, int num_counters,
-                              hipStream_t stream);
+                              void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // One token per row of 32-bit logits.  temperature 0 or top_k 1: argmax.  top_k <= 0 and top_p >= 1: off.
 int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature, const int* top_k,
@@ -84,17 +86,16 @@ void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* 
 
 namespace sa {
 int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
-                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, hipStream_t stream);
+                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, int packed, hipStream_t stream);
 bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2);
 int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
-                int N, int K, int epi, float cap, void* workspace, size_t workspace_bytes, void* counters,
-                int num_counters, int splits, hipStream_t stream);
+                int N, int K, int epi, float cap, int packed, int shape, hipStream_t stream);
 bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q);
 int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           void* counters, int num_counters, hipStream_t stream);
+                           hipStream_t stream);
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,

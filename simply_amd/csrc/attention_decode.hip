@@ -12,8 +12,9 @@
 // The second product needs no data movement: S^T comes out of the first MFMA in the register
 // layout that the second MFMA wants for its B operand, and value pages are stored transposed
 // ([hd, page_size]) so that the A operand is a plain load as well.  The four waves take tiles in
-// turn and merge their (maximum, sum, output) through LDS; key ranges are merged through a
-// workspace by the workgroup that finishes last, in a fixed order.
+// turn and merge their (maximum, sum, output) through LDS; key ranges are merged by a second, small
+// kernel from a workspace, in a fixed order (a merge by the workgroup that finishes last would need a
+// device-wide fence, which on this GPU writes back the whole L2).
 #include "api.h"
 #include "common.h"
 
@@ -46,14 +47,14 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ seq_meta, int seq_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
-    float* __restrict__ workspace, unsigned* __restrict__ counters) {
+    float* __restrict__ workspace) {
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;  // output blocks of 16 dimensions
   __shared__ float o_s[2][16][HD + 1];   // a wave's output [row][d], while two waves are merged
   __shared__ float m_s[2][16], l_s[2][16];
-  __shared__ int is_last_s;
 
-  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // the same for the whole wave: kept in a scalar register
   const int r = lane % 16, grp = lane / 16;
   const int split = blockIdx.x, num_splits = gridDim.x, kh = blockIdx.y, seq = seq_begin + blockIdx.z;
   const SeqMeta sm = seq_meta[seq];
@@ -89,33 +90,66 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   for (int db = 0; db < NDB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;  // per row (lane % 16); l_run is this lane group's share
 
-  for (int tile = tb + wave; tile < te; tile += 4) {
+  // The loop is software-pipelined so that a wave always has loads in flight: the keys of the next tile are
+  // requested before the scores of this tile are turned into probabilities, and the values of this tile are
+  // requested before its scores are computed.
+  struct SubTile {
+    bool ok;            // some key of the sub-tile is in [lo, hi): its page exists
+    const bf16* k;      // this lane's key row, at its 8 dimensions of chunk 0
+    const bf16* v;      // this lane's value row (dimension r of block 0), at its 4 keys
+  };
+  auto locate = [&](int tile, int t) {
+    SubTile st;
+    const int sk0 = tile * kTile + t * 16;
+    st.ok = tile < te && sk0 < hi && sk0 + 16 > lo;  // wave-uniform
+    st.k = nullptr;
+    st.v = nullptr;
+    if (st.ok) {
+      const int page = table[sk0 / page_size];
+      const int off = sk0 % page_size;  // a multiple of 16
+      const size_t head = static_cast<size_t>(page) * Kh + kh;
+      st.k = k_pages + (head * page_size + off + r) * HD + grp * 8;
+      st.v = v_pages + (head * HD + r) * page_size + off + grp * 4;
+    }
+    return st;
+  };
+  const bf16x8 zero8 = {};
+  const bf16x4 zero4 = {};
+
+  int tile = tb + wave;
+  SubTile cur[2] = {locate(tile, 0), locate(tile, 1)};
+  bf16x8 kf[2][NDC];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int dc = 0; dc < NDC; ++dc) kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 32) : zero8;
+
+  for (; tile < te; tile += 4) {
     const int key0 = tile * kTile;
-    // ---- scores of two sub-tiles of 16 keys
+    // ---- request this tile's values
+    bf16x4 vf[2][NDB];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+        vf[t][db] = cur[t].ok ? *reinterpret_cast<const bf16x4*>(cur[t].v + static_cast<size_t>(db) * 16 * page_size) : zero4;
+    // ---- scores of the two sub-tiles of 16 keys
     floatx4 s[2];
-    bool sub_ok[2];
-    const bf16* vbase[2];
-    int voff[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int sk0 = key0 + t * 16;                    // first key of the sub-tile
-      sub_ok[t] = sk0 < hi && sk0 + 16 > lo;            // wave-uniform
       s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-      vbase[t] = nullptr;
-      voff[t] = 0;
-      if (sub_ok[t]) {
-        const int page = table[sk0 / page_size];
-        const int off = sk0 % page_size;                // multiple of 16
-        const bf16* kp = k_pages + ((static_cast<size_t>(page) * Kh + kh) * page_size + off + r) * HD + grp * 8;
-        bf16x8 kf[NDC];
 #pragma unroll
-        for (int dc = 0; dc < NDC; ++dc) kf[dc] = *reinterpret_cast<const bf16x8*>(kp + dc * 32);
-#pragma unroll
-        for (int dc = 0; dc < NDC; ++dc) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[dc], qf[dc], s[t], 0, 0, 0);
-        vbase[t] = v_pages + (static_cast<size_t>(page) * Kh + kh) * HD * page_size;
-        voff[t] = off + grp * 4;
-      }
+      for (int dc = 0; dc < NDC; ++dc) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][dc], qf[dc], s[t], 0, 0, 0);
     }
+    const bool sub_ok[2] = {cur[0].ok, cur[1].ok};
+    // ---- request the next tile's keys
+    cur[0] = locate(tile + 4, 0);
+    cur[1] = locate(tile + 4, 1);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int dc = 0; dc < NDC; ++dc)
+        kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 32) : zero8;
     // ---- cap, mask, online softmax.  Lane (row r, grp) holds keys sk0 + 4 * grp + v of each sub-tile.
     float p[2][4];
     float mx = -INFINITY;
@@ -153,26 +187,21 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     const bool tail = key0 + kTile > hi;  // keys at or beyond hi may be unwritten: their values count as 0
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
-      bf16x8 vf = {};
+      bf16x8 a;
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        if (sub_ok[t]) {
-          const bf16x4 x = *reinterpret_cast<const bf16x4*>(vbase[t] + static_cast<size_t>(db * 16 + r) * page_size +
-                                                           voff[t]);
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int v = 0; v < 4; ++v) vf[t * 4 + v] = x[v];
-        }
-      }
+        for (int v = 0; v < 4; ++v) a[t * 4 + v] = vf[t][db][v];
       if (tail) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int key = key0 + (e / 4) * 16 + grp * 4 + (e % 4);
-          if (key >= hi) vf[e] = to_bf16_raw(0.f);
+          if (key >= hi) a[e] = to_bf16_raw(0.f);
         }
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[db][v] *= alpha;
-      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[db], 0, 0, 0);
+      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, acc[db], 0, 0, 0);
     }
   }
 
@@ -233,35 +262,40 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
       }
     }
   }
-  if (KS == 1) return;
-  // ---- the workgroup that finishes last for this (request, head) adds the key ranges up, in their order
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) is_last_s = atomicAdd(&counters[unit], 1u) == static_cast<unsigned>(KS - 1);
-  __syncthreads();
-  if (!is_last_s) return;
-  __threadfence();
-  if (tid == 0) counters[unit] = 0u;
-  const int orow = tid / 16, oc = tid % 16;  // thread -> (row, 16 threads over d)
-  if (orow >= rows) return;
+}
+
+// Adds up the key ranges of each (request, head, row), in their order: one workgroup per row, one thread per
+// output dimension; the ranges' weights exp(m_y - max) are computed once into LDS.
+constexpr int kMaxSplits = 256;
+__global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ workspace, int KS, int HD,
+                                                                    const SeqMeta* __restrict__ seq_meta, int seq_begin,
+                                                                    bf16* __restrict__ out, int64_t out_stride, int Kh,
+                                                                    int G) {
+  __shared__ float w_s[kMaxSplits];
+  __shared__ float scratch[16];
+  const int tid = threadIdx.x, kh = blockIdx.x, z = blockIdx.y, orow = blockIdx.z;
+  const SeqMeta sm = seq_meta[seq_begin + z];
+  if (orow >= G * sm.q_len) return;
+  const size_t row_words = HD + 2;
+  const size_t unit = static_cast<size_t>(z) * Kh + kh;
   const float* base = workspace + (unit * KS * 16 + orow) * row_words;
   const size_t stride = 16 * row_words;
-  float Mg = -INFINITY;
-  for (int y = 0; y < KS; ++y) Mg = fmaxf(Mg, __builtin_nontemporal_load(base + y * stride + HD));
-  float Lg = 0.f;
-  for (int y = 0; y < KS; ++y) {
-    const float my = __builtin_nontemporal_load(base + y * stride + HD);
-    Lg += __builtin_nontemporal_load(base + y * stride + HD + 1) * (my == -INFINITY ? 0.f : __expf(my - Mg));
-  }
+  const float my = tid < KS ? base[tid * stride + HD] : -INFINITY;
+  const float ly = tid < KS ? base[tid * stride + HD + 1] : 0.f;
+  // maximum over the ranges
+  float mx = wave_max(my);
+  if (tid % kWave == 0) scratch[tid / kWave] = mx;
+  __syncthreads();
+  const float Mg = fmaxf(fmaxf(scratch[0], scratch[1]), fmaxf(scratch[2], scratch[3]));
+  const float wy = my == -INFINITY ? 0.f : __expf(my - Mg);
+  if (tid < KS) w_s[tid] = wy;
+  const float Lg = block_sum(ly * wy, scratch + 4);  // has its own barriers; w_s is complete after them
   const int oq = orow / G, og = orow % G;
   bf16* op = out + static_cast<size_t>(sm.q_start + oq) * out_stride + static_cast<size_t>(kh * G + og) * HD;
   const float inv = 1.f / Lg;
-  for (int d = oc; d < HD; d += 16) {
+  for (int d = tid; d < HD; d += 256) {
     float o = 0.f;
-    for (int y = 0; y < KS; ++y) {
-      const float my = __builtin_nontemporal_load(base + y * stride + HD);
-      o += __builtin_nontemporal_load(base + y * stride + d) * (my == -INFINITY ? 0.f : __expf(my - Mg));
-    }
+    for (int y = 0; y < KS; ++y) o += base[y * stride + d] * w_s[y];
     op[d] = float_to_bf16(o * inv);
   }
 }
@@ -276,7 +310,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           void* counters, int num_counters, hipStream_t stream) {
+                           hipStream_t stream) {
   if (seq_count == 0) return 0;
   const int G = H / Kh;
   const int units = seq_count * Kh;
@@ -285,16 +319,15 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   const int max_tiles = (span + kTile - 1) / kTile + 1;
   int KS = num_splits;
   if (KS <= 0) {
-    KS = (256 * 4 + units - 1) / units;      // about four workgroups per CU
-    const int cap_by_work = (max_tiles + 7) / 8;  // at least 8 tiles (256 keys) per workgroup
+    KS = (256 + units / 2) / units;               // about one workgroup per CU: longer ranges amortise the set-up
+    const int cap_by_work = (max_tiles + 3) / 4;  // at least 4 tiles (128 keys) per workgroup
     if (KS > cap_by_work) KS = cap_by_work;
   }
   if (KS > max_tiles) KS = max_tiles;
+  if (KS > kMaxSplits) KS = kMaxSplits;
   if (KS < 1) KS = 1;
   const size_t per_split = static_cast<size_t>(units) * 16 * (hd + 2) * sizeof(float);
-  while (KS > 1 && (workspace == nullptr || counters == nullptr || units > num_counters ||
-                    per_split * KS > workspace_bytes))
-    --KS;
+  while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
   const dim3 grid(KS, Kh, seq_count);
   const bf16* qp = static_cast<const bf16*>(q);
   const bf16* kp = static_cast<const bf16*>(k_pages);
@@ -302,11 +335,10 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   const SeqMeta* sm = reinterpret_cast<const SeqMeta*>(seq_meta);
   bf16* op = static_cast<bf16*>(out);
   float* ws = static_cast<float*>(workspace);
-  unsigned* cn = static_cast<unsigned*>(counters);
 #define SA_LAUNCH(NDC)                                                                                              \
   paged_attention_decode_kernel<NDC><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, sm, \
                                                                seq_begin, op, out_stride, Kh, G, page_size, window,  \
-                                                               soft_cap, ws, cn)
+                                                               soft_cap, ws)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
   else if (hd == 256) SA_LAUNCH(8);
@@ -315,7 +347,13 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
     return 1;
   }
 #undef SA_LAUNCH
-  return check_launch("paged_attention_decode");
+  if (check_launch("paged_attention_decode")) return 1;
+  if (KS > 1) {
+    paged_attention_merge_kernel<<<dim3(Kh, seq_count, 16), 256, 0, stream>>>(ws, KS, hd, sm, seq_begin, op, out_stride,
+                                                                             Kh, G);
+    return check_launch("paged_attention_merge");
+  }
+  return 0;
 }
 
 }  // namespace sa

@@ -9,14 +9,19 @@ namespace sa {
 
 // ------------------------------------------------------------------ embedding
 // out[t, :] = float(table[tokens[t], :]) * scale.   simply/utils/module.py:450-481
+// `packed`: the table is tiled like a matrix-product weight, [V / 16][ceil(D / 32)][kq 4][row 16][8].
 __global__ void embed_kernel(const void* __restrict__ table, int table_dtype, const int* __restrict__ tokens,
-                             float* __restrict__ out, int D, int V, float scale) {
+                             float* __restrict__ out, int D, int V, float scale, int packed) {
   const int t = blockIdx.x;
   int tok = tokens[t];
   tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);  // the host has already refused ids outside the table
   const size_t base = static_cast<size_t>(tok) * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x)
-    out[static_cast<size_t>(t) * D + d] = load_f(table, table_dtype, base + d) * scale;
+  const int chunks = (D + 31) / 32;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const size_t i = packed ? ((static_cast<size_t>(tok / 16) * chunks + d / 32) * 64 + ((d % 32) / 8) * 16 + tok % 16) * 8 + d % 8
+                            : base + d;
+    out[static_cast<size_t>(t) * D + d] = load_f(table, table_dtype, i) * scale;
+  }
 }
 
 // ------------------------------------------------------------------ RMSNorm
@@ -170,11 +175,11 @@ static int row_threads(int D) {
 using namespace sa;
 
 extern "C" int sa_embed(const void* table, int table_dtype, const int* tokens, float* out, int T, int D, int V,
-                        float scale, hipStream_t stream) {
+                        float scale, int packed, hipStream_t stream) {
   if (T == 0) return 0;
   SA_REQUIRE(table_dtype == kF32 || table_dtype == kBF16, "embed: unknown table dtype %d", table_dtype);
   SA_REQUIRE(T > 0 && D > 0 && V > 0, "embed: bad sizes T=%d D=%d V=%d", T, D, V);
-  embed_kernel<<<T, row_threads(D), 0, stream>>>(table, table_dtype, tokens, out, D, V, scale);
+  embed_kernel<<<T, row_threads(D), 0, stream>>>(table, table_dtype, tokens, out, D, V, scale, packed);
   return check_launch("embed");
 }
 

@@ -17,8 +17,15 @@ __device__ inline float gelu_tanh(float x) {
   return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
 }
 
+// Index of W[n][k] in memory: row-major, or tiled [N / 16][chunks][kq 4][row 16][8] (chunks = ceil(K / 32)).
+template <bool PACKED>
+__device__ inline size_t w_index(int n, int k, int K, int chunks) {
+  if (!PACKED) return static_cast<size_t>(n) * K + k;
+  return ((static_cast<size_t>(n / 16) * chunks + k / 32) * 64 + ((k % 32) / 8) * 16 + n % 16) * 8 + k % 8;
+}
+
 // EPI: 0 plain, 1 gated (C = gelu(A.W^T) * (A.W2^T)), 2 soft-cap (C = cap * tanh(A.W^T / cap))
-template <typename TA, typename TW, typename TC, int EPI>
+template <typename TA, typename TW, typename TC, int EPI, bool PACKED>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, int64_t lda,
                                                            const TW* __restrict__ W, const TW* __restrict__ W2,
                                                            TC* __restrict__ C, int64_t ldc, int M, int N, int K,
@@ -31,6 +38,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   float acc[TM][TN] = {};
   float acc2[EPI == 1 ? TM : 1][TN] = {};
+  const int chunks = (K + 31) / 32;
   const int lr = tid / 4;         // tile row 0..63
   const int lk = (tid % 4) * 4;   // k offset 0,4,8,12
   for (int k0 = 0; k0 < K; k0 += BK) {
@@ -39,8 +47,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       const int k = k0 + lk + i;
       const int m = m0 + lr, n = n0 + lr;
       As[lk + i][lr] = (m < M && k < K) ? to_float(A[static_cast<size_t>(m) * lda + k]) : 0.f;
-      Ws[lk + i][lr] = (n < N && k < K) ? to_float(W[static_cast<size_t>(n) * K + k]) : 0.f;
-      if (EPI == 1) W2s[lk + i][lr] = (n < N && k < K) ? to_float(W2[static_cast<size_t>(n) * K + k]) : 0.f;
+      Ws[lk + i][lr] = (n < N && k < K) ? to_float(W[w_index<PACKED>(n, k, K, chunks)]) : 0.f;
+      if (EPI == 1) W2s[lk + i][lr] = (n < N && k < K) ? to_float(W2[w_index<PACKED>(n, k, K, chunks)]) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -84,7 +92,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
   }
 }
 
-template <typename TA, typename TW, typename TC>
+template <typename TA, typename TW, typename TC, bool PACKED>
 static void launch_generic(const void* A, int64_t lda, const void* W, const void* W2, void* C, int64_t ldc, int M, int N,
                            int K, int epi, float cap, hipStream_t stream) {
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
@@ -92,21 +100,29 @@ static void launch_generic(const void* A, int64_t lda, const void* W, const void
   const TW* w = static_cast<const TW*>(W);
   const TW* w2 = static_cast<const TW*>(W2);
   TC* c = static_cast<TC*>(C);
-  if (epi == 0) gemm_generic_kernel<TA, TW, TC, 0><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
-  else if (epi == 1) gemm_generic_kernel<TA, TW, TC, 1><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
-  else gemm_generic_kernel<TA, TW, TC, 2><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
+  if (epi == 0)
+    gemm_generic_kernel<TA, TW, TC, 0, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
+  else if (epi == 1)
+    gemm_generic_kernel<TA, TW, TC, 1, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
+  else
+    gemm_generic_kernel<TA, TW, TC, 2, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
 }
 
 int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
-                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, hipStream_t stream) {
-  if (a_dtype == kF32 && w_dtype == kF32 && c_dtype == kF32)
-    launch_generic<float, float, float>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
-  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kBF16)
-    launch_generic<bf16, bf16, bf16>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
-  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32)
-    launch_generic<bf16, bf16, float>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, int packed, hipStream_t stream) {
+  if (a_dtype == kF32 && w_dtype == kF32 && c_dtype == kF32 && !packed)
+    launch_generic<float, float, float, false>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kBF16 && !packed)
+    launch_generic<bf16, bf16, bf16, false>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32 && !packed)
+    launch_generic<bf16, bf16, float, false>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kBF16 && packed)
+    launch_generic<bf16, bf16, bf16, true>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+  else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32 && packed)
+    launch_generic<bf16, bf16, float, true>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
   else {
-    set_error("gemm: unsupported element types a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
+    set_error("gemm: unsupported element types a=%d w=%d c=%d (tiled weights: bfloat16 only)", a_dtype, w_dtype,
+              c_dtype);
     return 1;
   }
   return check_launch("gemm_generic");

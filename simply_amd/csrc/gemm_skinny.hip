@@ -6,10 +6,13 @@
 // four lanes reading 64 contiguous bytes), takes the matching activations from the cache hierarchy
 // (they are small and shared by all waves), and accumulates with v_mfma_f32_16x16x32_bf16: the
 // weight rows are the MFMA's A operand, up to four blocks of 16 activation rows its B operands.
-// The four waves of a workgroup take four consecutive K ranges of the same rows and add their
-// results through LDS; if K is cut over more workgroups than one (needed to fill 256 CUs when N is
-// small), each writes its partial tile to a workspace and the workgroup that finishes last adds
-// the partials in a fixed order, so the result does not depend on timing.
+// W may be row-major [N, K] or tiled (pack_tiles in the Python package): [N / 16][K / 32][64 lanes][8], each
+// 1 KiB block being one MFMA operand of 16 rows x 32 columns in register order, so that a wave's load is one
+// contiguous KiB (row-major rows give 64-byte pieces, which reach about half the bandwidth).
+// The 4 to 16 waves of a workgroup take consecutive K ranges of the same rows and add their results
+// through LDS in a fixed order.  When N is small a workgroup owns only 8 or 4 rows (the other
+// operand rows are zero), so that there are enough workgroups for 256 CUs without cutting K over
+// workgroups: that would need a device-wide fence, which on this GPU writes back the whole L2.
 #include "api.h"
 #include "common.h"
 
@@ -26,22 +29,23 @@ __device__ inline float gelu_tanh_f(float x) {
 __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
 constexpr int kUnroll = 4;
+constexpr int kMaxWaves = 16;
 
-template <int MB, int EPI>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ A, int64_t lda,
-                                                          const bf16* __restrict__ W, const bf16* __restrict__ W2,
-                                                          void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N,
-                                                          int K, int chunks, float cap, float* __restrict__ workspace,
-                                                          unsigned* __restrict__ counters) {
+// blockDim.x = 64 * NW (NW waves share the K range); a workgroup owns `tile_rows` (16, 8 or 4) rows of W.
+template <int MB, int EPI, bool PACKED>
+__global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restrict__ A, int64_t lda,
+                                                           const bf16* __restrict__ W, const bf16* __restrict__ W2,
+                                                           void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N,
+                                                           int K, int chunks, int tile_rows, float cap) {
   constexpr int NP = EPI == 1 ? 2 : 1;  // planes: gate and up for the gated epilogue
-  __shared__ float red[4][NP][MB][16 * 17];
-  __shared__ int is_last_s;
-  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  extern __shared__ float red[];        // [NW][NP][MB][16 * 17]
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform over the wave: kept in a scalar register
+  const int NW = blockDim.x / kWave;
   const int r = lane % 16, kq = lane / 16;
-  const int n0 = blockIdx.x * 16;
-  const int S = gridDim.y * 4, s = blockIdx.y * 4 + wave;
-  const int c0 = static_cast<int>(static_cast<int64_t>(chunks) * s / S);
-  const int c1 = static_cast<int>(static_cast<int64_t>(chunks) * (s + 1) / S);
+  const int n0 = blockIdx.x * tile_rows;
+  const int c0 = static_cast<int>(static_cast<int64_t>(chunks) * wave / NW);
+  const int c1 = static_cast<int>(static_cast<int64_t>(chunks) * (wave + 1) / NW);
 
   floatx4 acc[NP][MB];
 #pragma unroll
@@ -49,153 +53,157 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[p][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const bool row_ok = n0 + r < N;
-  const bf16* wrow = W + static_cast<size_t>(row_ok ? n0 + r : 0) * K;
-  const bf16* w2row = EPI == 1 ? W2 + static_cast<size_t>(row_ok ? n0 + r : 0) * K : nullptr;
+  const bool row_ok = r < tile_rows && n0 + r < N;
+  // row-major W: this lane's row, 8 elements at k.  Tiled W (see pack_tiles): tile (n0 / 16), chunk c is one
+  // contiguous 1 KiB block of which this lane owns 16 bytes, padded with zeros beyond N and K.
+  const size_t tile_elems = static_cast<size_t>(chunks) * 512;
+  const bf16* wrow = PACKED ? W + (n0 / 16) * tile_elems + lane * 8 : W + static_cast<size_t>(row_ok ? n0 + r : 0) * K;
+  const bf16* w2row = EPI != 1 ? nullptr
+                      : PACKED ? W2 + (n0 / 16) * tile_elems + lane * 8
+                               : W2 + static_cast<size_t>(row_ok ? n0 + r : 0) * K;
   const bf16x8 zero = {};
 
-  for (int c = c0; c < c1; c += kUnroll) {
-    bf16x8 a[kUnroll], a2[kUnroll], b[kUnroll][MB];
+  // Two register sets of kUnroll chunks each: while one set is multiplied, the loads of the other are in flight.
+  bf16x8 a[2][kUnroll], a2[2][kUnroll], b[2][kUnroll][MB];
+  auto load_set = [&](int set, int c) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int k = (c + u) * 32 + kq * 8;
       const bool ok = c + u < c1 && k < K;
-      a[u] = (ok && row_ok) ? load_frag(wrow + k) : zero;
-      if (EPI == 1) a2[u] = (ok && row_ok) ? load_frag(w2row + k) : zero;
+      if (PACKED) a[set][u] = c + u < c1 ? load_frag(wrow + static_cast<size_t>(c + u) * 512) : zero;
+      else a[set][u] = (ok && row_ok) ? load_frag(wrow + k) : zero;
+      if (EPI == 1) {
+        if (PACKED) a2[set][u] = c + u < c1 ? load_frag(w2row + static_cast<size_t>(c + u) * 512) : zero;
+        else a2[set][u] = (ok && row_ok) ? load_frag(w2row + k) : zero;
+      }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int m = mb * 16 + r;
-        b[u][mb] = (ok && m < M) ? load_frag(A + static_cast<size_t>(m) * lda + k) : zero;
+        b[set][u][mb] = (ok && m < M) ? load_frag(A + static_cast<size_t>(m) * lda + k) : zero;
       }
     }
+  };
+  auto mul_set = [&](int set) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][mb], acc[0][mb], 0, 0, 0);
-        if (EPI == 1) acc[1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[u], b[u][mb], acc[1][mb], 0, 0, 0);
+        acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[set][u], b[set][u][mb], acc[0][mb], 0, 0, 0);
+        if (EPI == 1)
+          acc[1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[set][u], b[set][u][mb], acc[1][mb], 0, 0, 0);
       }
+  };
+  load_set(0, c0);
+  for (int c = c0; c < c1; c += 2 * kUnroll) {
+    load_set(1, c + kUnroll);
+    mul_set(0);
+    load_set(0, c + 2 * kUnroll);
+    mul_set(1);
   }
 
-  // lane holds D[n = 4 * (lane / 16) + v][m = lane % 16]
+  // lane holds D[n = 4 * (lane / 16) + v][m = lane % 16]; the waves' tiles are added up through LDS, in wave order
+  auto red_at = [&](int w, int p, int mb) { return red + ((static_cast<size_t>(w) * NP + p) * MB + mb) * (16 * 17); };
 #pragma unroll
   for (int p = 0; p < NP; ++p)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) red[wave][p][mb][(4 * kq + v) * 17 + r] = acc[p][mb][v];
+      for (int v = 0; v < 4; ++v) red_at(wave, p, mb)[(4 * kq + v) * 17 + r] = acc[p][mb][v];
   __syncthreads();
-
-  const int ml = tid / 16, nl = tid % 16;  // this thread's output element within each 16 x 16 block
-  float sum[NP][MB];
-#pragma unroll
-  for (int p = 0; p < NP; ++p)
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-      sum[p][mb] = ((red[0][p][mb][nl * 17 + ml] + red[1][p][mb][nl * 17 + ml]) + red[2][p][mb][nl * 17 + ml]) +
-                   red[3][p][mb][nl * 17 + ml];
-
-  const int KS = gridDim.y;
-  const int Mpad = MB * 16;
-  if (KS > 1) {
-    // partial tile -> workspace[plane][split][m][n]; the last workgroup of this tile adds them up in order
-#pragma unroll
-    for (int p = 0; p < NP; ++p)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        if (n0 + nl < N)
-          workspace[((static_cast<size_t>(p) * KS + blockIdx.y) * Mpad + mb * 16 + ml) * N + n0 + nl] = sum[p][mb];
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) is_last_s = atomicAdd(&counters[blockIdx.x], 1u) == static_cast<unsigned>(KS - 1);
-    __syncthreads();
-    if (!is_last_s) return;
-    __threadfence();
-#pragma unroll
-    for (int p = 0; p < NP; ++p)
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        float t = 0.f;
-        if (n0 + nl < N)
-          for (int y = 0; y < KS; ++y)
-            t += __builtin_nontemporal_load(
-                &workspace[((static_cast<size_t>(p) * KS + y) * Mpad + mb * 16 + ml) * N + n0 + nl]);
-        sum[p][mb] = t;
-      }
-    if (tid == 0) counters[blockIdx.x] = 0u;  // ready for the next launch
-  }
-
+  for (int e = tid; e < 256; e += blockDim.x) {
+  const int ml = e / 16, nl = e % 16;  // an output element within each 16 x 16 block
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int m = mb * 16 + ml, n = n0 + nl;
-    if (m >= M || n >= N) continue;
-    float v = sum[0][mb];
+    if (m >= M || nl >= tile_rows || n >= N) continue;
+    float sum[NP];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      float t = 0.f;
+      for (int w = 0; w < NW; ++w) t += red_at(w, p, mb)[nl * 17 + ml];
+      sum[p] = t;
+    }
+    float v = sum[0];
     if (EPI == 1) {
       // both products are rounded to bfloat16 first, as separate matrix products would be
-      v = gelu_tanh_f(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1][mb]));
+      v = gelu_tanh_f(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
     } else if (EPI == 2) {
       v = cap * tanhf(v / cap);
     }
     store_f(C, c_dtype, static_cast<size_t>(m) * ldc + n, v);
   }
+  }
 }
 
-// How many ways to cut K (a multiple of 4: the waves of a workgroup), so that about 8 waves per CU are in
-// flight and no wave gets less than two 32-wide chunks.
-static int choose_splits(int tiles, int chunks, int planes) {
-  const int target_waves = 256 * 12;
-  int S = (target_waves + tiles - 1) / tiles;
-  S = (S + 3) / 4 * 4;
-  const int max_s = chunks * planes / 2;  // at least ~2 KB of weights per wave
-  if (S > max_s) S = max_s / 4 * 4;
-  if (S < 4) S = 4;
-  if (S > 64) S = 64;
-  return S;
+// Rows of W per workgroup and waves per workgroup; no wave gets less than two 32-wide chunks of K; the LDS for the
+// waves' tiles stays under 64 KiB.  Nothing is cut over workgroups: on this GPU a device-wide fence writes the
+// whole L2 back.
+static void choose_shape(int N, int chunks, int planes, int MB, int* tile_rows, int* waves) {
+  // measured on MI355X at M = 8: tiles of 16 rows always win (narrower tiles leave load lanes idle); 8 waves
+  // per workgroup while there are few tiles, 4 when there are many
+  const int rows = 16;
+  const int tiles = (N + rows - 1) / rows;
+  int nw = tiles < 1024 ? 8 : 4;
+  if (nw > chunks / 2) nw = chunks / 2;
+  while (nw > 1 && static_cast<size_t>(nw) * planes * MB * 16 * 17 * sizeof(float) > 60 * 1024) --nw;
+  if (nw > kMaxWaves) nw = kMaxWaves;
+  if (nw < 1) nw = 1;
+  *tile_rows = rows;
+  *waves = nw;
 }
 
-template <int MB>
+template <int MB, bool PACKED>
 static void launch_skinny(const bf16* A, int64_t lda, const bf16* W, const bf16* W2, void* C, int c_dtype, int64_t ldc,
-                          int M, int N, int K, int epi, float cap, float* ws, unsigned* counters, int S,
-                          hipStream_t stream) {
+                          int M, int N, int K, int epi, float cap, int tile_rows, int waves, hipStream_t stream) {
   const int chunks = (K + 31) / 32;
-  const dim3 grid((N + 15) / 16, S / 4);
+  const dim3 grid((N + tile_rows - 1) / tile_rows);
+  const int threads = waves * kWave;
+  const size_t lds = static_cast<size_t>(waves) * (epi == 1 ? 2 : 1) * MB * 16 * 17 * sizeof(float);
   if (epi == 0)
-    gemm_skinny_kernel<MB, 0><<<grid, 256, 0, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks, cap, ws,
-                                                        counters);
+    gemm_skinny_kernel<MB, 0, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+                                                                      tile_rows, cap);
   else if (epi == 1)
-    gemm_skinny_kernel<MB, 1><<<grid, 256, 0, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks, cap, ws,
-                                                        counters);
+    gemm_skinny_kernel<MB, 1, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+                                                                      tile_rows, cap);
   else
-    gemm_skinny_kernel<MB, 2><<<grid, 256, 0, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks, cap, ws,
-                                                        counters);
+    gemm_skinny_kernel<MB, 2, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+                                                                      tile_rows, cap);
 }
 
 bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2) {
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  // K % 8: a lane's 8 activations lie within its row, and row-major weight rows start at 16-byte boundaries
   return M >= 1 && M <= 64 && K % 8 == 0 && lda % 8 == 0 && aligned(A) && aligned(W) && (W2 == nullptr || aligned(W2));
 }
 
+// shape > 0 fixes the cut: tile_rows * 100 + waves (for instance 816: 8 rows, 16 waves)
 int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
-                int N, int K, int epi, float cap, void* workspace, size_t workspace_bytes, void* counters,
-                int num_counters, int splits, hipStream_t stream) {
-  const int tiles = (N + 15) / 16, chunks = (K + 31) / 32, planes = epi == 1 ? 2 : 1;
-  int S = splits > 0 ? (splits + 3) / 4 * 4 : choose_splits(tiles, chunks, planes);
-  if (S > chunks) S = (chunks + 3) / 4 * 4;
-  if (S < 4) S = 4;
-  // fewer cuts if the workspace cannot hold the partial tiles (none needed with one workgroup per tile)
-  const int Mpad = M <= 16 ? 16 : (M <= 32 ? 32 : 64);  // as the kernel's template pads it
-  const size_t per_split = static_cast<size_t>(planes) * Mpad * N * sizeof(float);
-  while (S > 4 && (workspace == nullptr || counters == nullptr || tiles > num_counters ||
-                   per_split * (S / 4) > workspace_bytes))
-    S -= 4;
+                int N, int K, int epi, float cap, int packed, int shape, hipStream_t stream) {
+  const int chunks = (K + 31) / 32, planes = epi == 1 ? 2 : 1;
+  const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  int tile_rows, waves;
+  choose_shape(N, chunks, planes, MB, &tile_rows, &waves);
+  if (shape > 0) {
+    tile_rows = shape / 100;
+    waves = shape % 100;
+    if ((tile_rows != 4 && tile_rows != 8 && tile_rows != 16) || (packed && tile_rows != 16) || waves < 1 || waves > kMaxWaves ||
+        static_cast<size_t>(waves) * planes * MB * 16 * 17 * sizeof(float) > 64 * 1024) {
+      set_error("gemm: bad few-rows shape %d (rows 4, 8 or 16, times 100, plus 1..16 waves)", shape);
+      return 1;
+    }
+  }
   const bf16* a = static_cast<const bf16*>(A);
   const bf16* w = static_cast<const bf16*>(W);
   const bf16* w2 = static_cast<const bf16*>(W2);
-  float* ws = static_cast<float*>(workspace);
-  unsigned* cn = static_cast<unsigned*>(counters);
-  if (M <= 16) launch_skinny<1>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, ws, cn, S, stream);
-  else if (M <= 32) launch_skinny<2>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, ws, cn, S, stream);
-  else launch_skinny<4>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, ws, cn, S, stream);
+#define SA_SKINNY(MBV)                                                                                              \
+  do {                                                                                                              \
+    if (packed) launch_skinny<MBV, true>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, tile_rows, waves, stream); \
+    else launch_skinny<MBV, false>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, tile_rows, waves, stream);     \
+  } while (0)
+  if (MB == 1) SA_SKINNY(1);
+  else if (MB == 2) SA_SKINNY(2);
+  else SA_SKINNY(4);
+#undef SA_SKINNY
   return check_launch("gemm_skinny");
 }
 

@@ -34,8 +34,7 @@ extern "C" int sa_version() { return 1; }
 
 extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
                        int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo,
-                       void* workspace, int64_t workspace_bytes, void* counters, int num_counters, int splits,
-                       hipStream_t stream) {
+                       int packed, int shape, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   SA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
   SA_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld are below K=%d, N=%d", (long long)lda,
@@ -51,12 +50,10 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
                "operands; got M=%d K=%d lda=%lld", M, K, (long long)lda);
     if (takes)
-      return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, workspace,
-                         static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), counters, num_counters, splits,
-                         stream);
+      return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, shape, stream);
   }
   SA_REQUIRE(algo != 3, "gemm: the tiled MFMA kernel is not built in");
-  return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, stream);
+  return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, stream);
 }
 
 extern "C" int sa_paged_attention(const void* q, int dtype, int64_t q_stride, const void* k_pages,
@@ -80,8 +77,8 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
                                          const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
                                          int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd,
                                          int page_size, int window, float soft_cap, int max_kv_len, int max_q_len,
-                                         int num_splits, void* workspace, int64_t workspace_bytes, void* counters,
-                                         int num_counters, hipStream_t stream) {
+                                         int num_splits, void* workspace, int64_t workspace_bytes,
+                                         hipStream_t stream) {
   if (seq_count == 0) return 0;
   SA_REQUIRE(seq_count > 0 && seq_begin >= 0 && H > 0 && Kh > 0 && H % Kh == 0, "paged_attention_decode: bad counts");
   SA_REQUIRE(window >= 0 && table_stride > 0 && max_kv_len > 0, "paged_attention_decode: bad window, table or length");
@@ -91,6 +88,5 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
   SA_REQUIRE(out_stride >= static_cast<int64_t>(H) * hd, "paged_attention_decode: output rows are too short");
   return paged_attention_decode(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, seq_begin, seq_count,
                                 out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len, num_splits,
-                                workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), counters,
-                                num_counters, stream);
+                                workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
 }

@@ -54,6 +54,9 @@ class Executor:
         self._host = torch.empty(self._words, dtype=torch.int32, pin_memory=self._on_gpu)
         self._dev = torch.empty(self._words, dtype=torch.int32, device=self.device)
         self._copied = torch.cuda.Event() if self._on_gpu else None
+        # decode-only steps (one token per request) are captured once per number of requests and replayed
+        self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._graph_pool = None
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid: Hashable) -> int:
@@ -76,6 +79,27 @@ class Executor:
             raise ValueError(f"request {e.request_id!r}: a portion starting at {e.start} would leave positions "
                              f"{done}..{e.start - 1} without keys")
         return e.start
+
+    def _replay(self, T: int, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
+        """A decode-only step through a captured HIP graph.  Everything that differs between two such steps
+        with the same number of requests (tokens, positions, slots, block tables) lies in buffers at fixed
+        addresses that the kernels read, so the launches can be recorded once.  The returned logits are
+        overwritten by the next replay with as many requests."""
+        entry = self._graphs.get(T)
+        if entry is None:
+            # once eagerly (kernels compile their plans, scratch buffers get allocated; the step's writes to the
+            # cache are the same when repeated), then record
+            self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
+            entry = (graph, logits)
+            self._graphs[T] = entry
+        entry[0].replay()
+        return entry[1]
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
@@ -161,7 +185,11 @@ class Executor:
                           groups=groups, request_ids=ctx_ids, seq_slots=ctx_slots, seq_starts=ctx_starts, q_lens=ctx_q,
                           cu_q_lens=cu)
         logit_rows = dev[3 * cap:3 * cap + R] if R else None
-        logits = self.model.forward(dev[:T], ctx, cache.views, logit_rows)
+        decode_only = self._on_gpu and self.config.use_graphs and all(q == 1 for q in ctx_q) and R == len(entries)
+        if decode_only:
+            logits = self._replay(T, ctx, logit_rows)
+        else:
+            logits = self.model.forward(dev[:T], ctx, cache.views, logit_rows)
         for rid, start, q in wants:
             self.num_computed[rid] = (cache.admission[rid], start + q)
         return logits

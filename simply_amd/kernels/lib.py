@@ -23,17 +23,17 @@ _path: str | None = None
 
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
-    "sa_embed": [_P, _I, _P, _P, _I, _I, _I, _F, _P],
+    "sa_embed": [_P, _I, _P, _P, _I, _I, _I, _F, _I, _P],
     "sa_rmsnorm": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _F, _I, _P],
     "sa_add_rmsnorm": [_P, _I, _P, _I, _F, _I, _P, _P, _I, _F, _I, _P, _I, _I, _I, _P],
     "sa_rope_cache_write": [_P, _I, _L, _P, _P, _F, _F, _P, _P, _P, _I, _I, _I, _I, _I, _P],
     "sa_rope": [_P, _I, _L, _P, _P, _F, _F, _I, _I, _I, _P],
     "sa_gather_rows": [_P, _I, _P, _P, _I, _I, _I, _P],
     "sa_fill_u32": [_P, c_uint32, _L, _P],
-    "sa_gemm": [_P, _I, _L, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _F, _I, _P, _L, _P, _I, _I, _P],
+    "sa_gemm": [_P, _I, _L, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "sa_paged_attention": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _I, _P],
-    "sa_paged_attention_decode": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P,
-                                  _I, _P],
+    "sa_paged_attention_decode": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L,
+                                  _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P],
 }
 

@@ -12,6 +12,7 @@ import torch
 
 from . import lib as _lib
 from .lib import KernelError
+from .packing import TiledWeight
 
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
@@ -65,19 +66,23 @@ def _i32(t: torch.Tensor, what: str, n: int | None = None) -> None:
 # --------------------------------------------------------------------------- row-wise
 
 
-def embed(table: torch.Tensor, tokens: torch.Tensor, scale: float, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t] = float32(table[tokens[t]]) * scale."""
-    _dev(table, tokens, out)
+def embed(table: "torch.Tensor | TiledWeight", tokens: torch.Tensor, scale: float,
+          out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = float32(table[tokens[t]]) * scale.  The table may be row-major or tiled."""
+    packed = isinstance(table, TiledWeight)
+    data = table.data if packed else table
+    _dev(data, tokens, out)
     V, D = table.shape
     T = tokens.numel()
     _i32(tokens, "embed: tokens")
-    if not table.is_contiguous():
+    if not data.is_contiguous():
         raise KernelError("embed: the table must be contiguous")
     if out is None:
-        out = torch.empty((T, D), dtype=torch.float32, device=table.device)
+        out = torch.empty((T, D), dtype=torch.float32, device=data.device)
     if out.dtype != torch.float32 or not out.is_contiguous() or tuple(out.shape) != (T, D):
         raise KernelError("embed: the output must be a contiguous float32 [T, D] tensor")
-    _lib.call("sa_embed", _ptr(table), _code(table), _ptr(tokens), _ptr(out), T, D, V, float(scale), _stream())
+    _lib.call("sa_embed", _ptr(data), _code(data), _ptr(tokens), _ptr(out), T, D, V, float(scale), int(packed),
+              _stream())
     return out
 
 
@@ -211,37 +216,43 @@ def fill_(t: torch.Tensor, value_bits: int = 0) -> None:
 
 EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
 
-#: scratch memory of kernels that cut K over workgroups, one per device, allocated at the first product
+#: scratch memory for partial results (attention over key ranges), one per device, allocated at first use
 WORKSPACE_BYTES = 64 << 20
-NUM_COUNTERS = 1 << 16
 _scratch: dict = {}
 
 
-def _workspace(device):
+def _workspace(device) -> torch.Tensor:
     key = (device.type, device.index)
     if key not in _scratch:
-        _scratch[key] = (torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device),
-                         torch.zeros(NUM_COUNTERS, dtype=torch.int32, device=device))
+        _scratch[key] = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
     return _scratch[key]
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: torch.Tensor | None = None, soft_cap: float | None = None,
-         out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None, algo: int = ALGO_AUTO,
-         splits: int = 0) -> torch.Tensor:
-    """a[M, K] . w[N, K]^T.  With w2: gelu_tanh(a.w^T) * (a.w2^T).  With soft_cap: cap * tanh(. / cap)."""
-    _dev(a, w, w2, out)
+def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
+         soft_cap: float | None = None, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
+         algo: int = ALGO_AUTO, shape: int = 0) -> torch.Tensor:
+    """a[M, K] . w[N, K]^T.  With w2: gelu_tanh(a.w^T) * (a.w2^T).  With soft_cap: cap * tanh(. / cap).
+    w (and w2) are row-major tensors or `TiledWeight`s."""
+    packed = isinstance(w, TiledWeight)
+    wd = w.data if packed else w
+    w2d = None
+    if w2 is not None:
+        if isinstance(w2, TiledWeight) != packed:
+            raise KernelError("gemm: both weights must be tiled, or neither")
+        w2d = w2.data if packed else w2
+    _dev(a, wd, w2d, out)
     lda = _rows(a, "gemm: a")
     M, K = a.shape
-    if w.dim() != 2 or not w.is_contiguous() or w.shape[1] != K:
+    if not wd.is_contiguous() or (not packed and w.dim() != 2) or w.shape[1] != K:
         raise KernelError(f"gemm: weight {tuple(w.shape)} does not match a {tuple(a.shape)} (expects [N, K] contiguous)")
     N = w.shape[0]
-    if w.dtype != a.dtype:
-        raise KernelError(f"gemm: a is {a.dtype} but the weight is {w.dtype}")
+    if wd.dtype != a.dtype:
+        raise KernelError(f"gemm: a is {a.dtype} but the weight is {wd.dtype}")
     epi, cap = EPILOGUE_NONE, 0.0
     if w2 is not None:
         if soft_cap:
             raise KernelError("gemm: the gated and the soft-cap epilogue do not combine")
-        if w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous():
+        if tuple(w2.shape) != tuple(w.shape) or w2d.dtype != wd.dtype or not w2d.is_contiguous():
             raise KernelError("gemm: the second weight must match the first")
         epi = EPILOGUE_GATED_GELU
     elif soft_cap:
@@ -251,9 +262,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: torch.Tensor | None = None, so
     if tuple(out.shape) != (M, N):
         raise KernelError("gemm: bad output shape")
     ldc = _rows(out, "gemm: out")
-    ws, counters = _workspace(a.device)
-    _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(w), _ptr(w2), _code(w), _ptr(out), _code(out), ldc, M, N, K, epi,
-              cap, algo, _ptr(ws), ws.numel(), _ptr(counters), counters.numel(), int(splits), _stream())
+    _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(wd), _ptr(w2d), _code(wd), _ptr(out), _code(out), ldc, M, N, K, epi,
+              cap, algo, int(packed), int(shape), _stream())
     return out
 
 
@@ -314,11 +324,11 @@ def paged_attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torc
     if out.dtype != q.dtype or out.shape[0] != q.shape[0] or out.shape[1] != num_heads * hd:
         raise KernelError("paged_attention_decode: bad output")
     out_stride = _rows(out, "paged_attention_decode: out")
-    ws, counters = _workspace(q.device)
+    ws = _workspace(q.device)
     _lib.call("sa_paged_attention_decode", _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
               block_table.stride(0), _ptr(seq_meta), seq_begin, seq_count, _ptr(out), out_stride, num_heads, Kh, hd,
               page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
-              _ptr(ws), ws.numel(), _ptr(counters), counters.numel(), _stream())
+              _ptr(ws), ws.numel(), _stream())
     return out
 
 

@@ -1,0 +1,75 @@
+"""The tiled layout of bfloat16 weight matrices.
+
+A matrix W[N, K] is cut into blocks of 16 rows by 32 columns; each block is stored as the 1 KiB that
+one v_mfma_f32_16x16x32_bf16 operand occupies in registers: [lane 64][8], lane = (k % 32) // 8 * 16 +
+n % 16, element k % 8.  Blocks follow each other along K, then along N; rows and columns beyond N and K
+are zero.  A wavefront that streams a block therefore reads one contiguous KiB, where row-major rows
+would give it sixteen 64-byte pieces (about half the bandwidth on MI355X).
+"""
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+
+@dataclasses.dataclass
+class TiledWeight:
+    data: torch.Tensor   # [ceil(N / 16), ceil(K / 32), 64, 8] bfloat16, contiguous
+    rows: int            # N
+    cols: int            # K
+
+    @property
+    def shape(self) -> tuple[int, int]:
+        return (self.rows, self.cols)
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+
+_cache: dict[tuple, tuple[torch.Tensor, TiledWeight]] = {}   # the source is kept alive so that its address stays its own
+
+
+def pack_tiles(w: torch.Tensor, cached: bool = False) -> TiledWeight:
+    """Row-major [N, K] bfloat16 -> tiled.  With `cached`, the same storage is packed once (a tied
+    embedding table that is also the head); `clear_cache()` ends the sharing."""
+    if w.dim() != 2 or w.dtype != torch.bfloat16:
+        raise ValueError(f"pack_tiles: expected a 2-D bfloat16 tensor, got {tuple(w.shape)} {w.dtype}")
+    key = (w.data_ptr(), tuple(w.shape), str(w.device))
+    if cached and key in _cache:
+        return _cache[key][1]
+    N, K = w.shape
+    Np, Kp = -(-N // 16) * 16, -(-K // 32) * 32
+    if (Np, Kp) != (N, K):
+        padded = torch.zeros((Np, Kp), dtype=w.dtype, device=w.device)
+        padded[:N, :K] = w
+    else:
+        padded = w
+    # [N/16, 16 rows, K/32, 4 kq, 8] -> [N/16, K/32, 4 kq, 16 rows, 8]
+    data = padded.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(Np // 16, Kp // 32, 64, 8)
+    tw = TiledWeight(data, N, K)
+    if cached:
+        _cache[key] = (w, tw)
+    return tw
+
+
+def unpack_tiles(tw: TiledWeight) -> torch.Tensor:
+    nt, nc = tw.data.shape[:2]
+    full = tw.data.view(nt, nc, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nt * 16, nc * 32)
+    return full[:tw.rows, :tw.cols].contiguous()
+
+
+def clear_cache() -> None:
+    _cache.clear()
+
+
+def concat_rows(*ws: torch.Tensor) -> torch.Tensor:
+    return torch.cat(ws, dim=0).contiguous()

@@ -66,8 +66,13 @@ class DecoderModel:
 
     def load_tensors(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """`tensors`: name in the model folder -> device tensor in its final dtype."""
-        for part, ps in self._bindings():
-            part.load({local: tensors[ps.tensors[local]] for local in part.param_specs()})
+        from ..kernels import packing
+
+        try:
+            for part, ps in self._bindings():
+                part.load({local: tensors[ps.tensors[local]] for local in part.param_specs()})
+        finally:
+            packing.clear_cache()   # sharing of re-laid tensors (tied table and head) ends with the load
         self.loaded = True
 
     # ------------------------------------------------------------------ cache

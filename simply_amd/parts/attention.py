@@ -11,7 +11,7 @@ import torch
 from ..config.spec import PartSpec
 from ..kernels import ops
 from ..registry import MIXERS, POSITION_ENCODINGS
-from .base import Mixer, PagedKVNeed, ParamSpec
+from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight
 
 
 @MIXERS.register("paged_attention")
@@ -39,10 +39,12 @@ class PagedAttention(Mixer):
 
     def load(self, tensors):
         # one product for q, k and v: rows [q heads | k heads | v heads]
-        self.qkv_proj = torch.cat([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]], dim=0).contiguous()
-        self.o_proj = tensors["o_proj"]
+        device = tensors["o_proj"].device
+        self.qkv_proj = as_product_weight(torch.cat([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]], dim=0)
+                                          .contiguous())
+        self.o_proj = as_product_weight(tensors["o_proj"])
         if self.position_encoding is not None and hasattr(self.position_encoding, "to_device"):
-            self.position_encoding.to_device(self.o_proj.device)
+            self.position_encoding.to_device(device)
 
     def cache_need(self):
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)

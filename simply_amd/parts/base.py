@@ -58,6 +58,17 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
+def as_product_weight(t: torch.Tensor, shared: bool = False):
+    """A matrix in the form that the matrix-product kernels read fastest: bfloat16 matrices on the GPU are
+    re-laid in tiles (simply_amd/kernels/packing.py), anything else stays row-major.  `shared`: parts that are
+    handed the same tensor during one load (a tied table and head) get the same re-laid copy."""
+    from ..kernels.packing import pack_tiles
+
+    if t.dtype == torch.bfloat16 and t.is_cuda and t.dim() == 2:
+        return pack_tiles(t, cached=shared)
+    return t
+
+
 class Part:
     """Common base: parameter declaration and loading."""
 

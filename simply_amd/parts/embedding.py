@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import ParamSpec, Part
+from .base import ParamSpec, Part, as_product_weight
 
 
 class ScaledEmbedding(Part):
@@ -19,6 +19,10 @@ class ScaledEmbedding(Part):
 
     def param_specs(self):
         return {"table": ParamSpec((self.vocab_size, self.dim), role="matrix", init="weight")}
+
+    def load(self, tensors):
+        # tiled like a product weight when it is bfloat16 on the GPU: a tied head reads the same storage
+        self.table = as_product_weight(tensors["table"], shared=True)
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
         """tokens int32 [T] -> float32 residual stream [T, D]."""
@@ -35,6 +39,9 @@ class LinearHead(Part):
 
     def param_specs(self):
         return {"weight": ParamSpec((self.vocab_size, self.dim), role="matrix", init="weight")}
+
+    def load(self, tensors):
+        self.weight = as_product_weight(tensors["weight"], shared=True)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x [R, D] activations -> float32 logits [R, V]."""

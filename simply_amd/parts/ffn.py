@@ -6,7 +6,7 @@ import torch
 
 from ..kernels import ops
 from ..registry import ACTIVATIONS, FEED_FORWARDS
-from .base import FeedForward, ParamSpec
+from .base import FeedForward, ParamSpec, as_product_weight
 
 # activation name -> epilogue of the fused gate/up product
 ACTIVATIONS.register("gelu_tanh", ops.EPILOGUE_GATED_GELU)
@@ -24,6 +24,10 @@ class GatedDense(FeedForward):
     def param_specs(self):
         D, F = self.hidden_size, self.intermediate_size
         return {"gate_proj": ParamSpec((F, D)), "up_proj": ParamSpec((F, D)), "down_proj": ParamSpec((D, F))}
+
+    def load(self, tensors):
+        self.gate_proj, self.up_proj, self.down_proj = (as_product_weight(tensors[n])
+                                                        for n in ("gate_proj", "up_proj", "down_proj"))
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         z = ops.gemm(x, self.gate_proj, w2=self.up_proj)   # gelu(x.Wg^T) * (x.Wu^T), one kernel

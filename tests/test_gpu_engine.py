@@ -80,3 +80,42 @@ def test_cuts_match_plain_at_kernel_sizes(tmp_path, dtype):
         assert torch.isfinite(got).all()
         err = (got - want).abs().max().item() / scale
         assert err <= TOL[dtype], (cuts, err)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_match_eager(tmp_path, dtype):
+    """Decode-only steps run through captured HIP graphs: every replay (with the host's own work and
+    synchronisation between them) gives what the eager step gives, for changing numbers of requests."""
+    d = tiny.write_model("D", str(tmp_path / "D"), std=0.15)
+    vocab = plain.load(d)[1]["vocab_size"]
+    reqs = {f"r{i}": tiny.random_tokens(40 + 7 * i, vocab, 20 + i) for i in range(3)}
+    outs = {}
+    for graphs in (False, True):
+        cfg = EngineConfig(activation_dtype=dtype, page_size=16, batch_size=4, max_seq_len=128, max_num_issue_tokens=128,
+                           total_num_pages=32, device="cuda:0", use_graphs=graphs)
+        model, _ = load_model(d, cfg.dtype, "cuda:0")
+        ex = Executor(model, cfg)
+        got = {r: [] for r in reqs}
+        for r, t in reqs.items():
+            ex.add_request(r)
+            got[r].append(ex.step([StepEntry(r, t[:20], [19])]).cpu())
+        pos = {r: 20 for r in reqs}
+        live = list(reqs)
+        while live:
+            logits = ex.step([StepEntry(r, [reqs[r][pos[r]]], [0]) for r in live]).cpu()
+            for i, r in enumerate(live):
+                got[r].append(logits[i:i + 1])
+                pos[r] += 1
+            for r in [r for r in live if pos[r] == len(reqs[r])]:
+                ex.finish_request(r)
+                live.remove(r)
+        if graphs:
+            assert sorted(ex._graphs) == [1, 2, 3]
+        outs[graphs] = {r: torch.cat(v) for r, v in got.items()}
+    for r in reqs:
+        assert torch.equal(outs[False][r], outs[True][r]), r
+    w, cfg_ = plain.load(d)
+    for r, t in reqs.items():
+        want = plain_logits(d, t, dtype)[0][19:]
+        err = (outs[True][r].double() - want).abs().max().item() / want.abs().max().item()
+        assert err <= TOL[dtype], (r, err)

@@ -229,17 +229,20 @@ def test_sampling_frequencies():
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K", [(48, 64), (100, 72), (2304, 2048), (333, 1000), (4096, 2304)])
 def test_gemm_skinny(M, N, K):
-    """The few-rows bfloat16 kernel, also with K cut over several workgroups (partials through the workspace)."""
+    """The few-rows bfloat16 kernel, with its own choice of rows per workgroup and waves and with forced ones."""
     from simply_amd.kernels import ops
     a, w, w2 = rand((M, K), torch.bfloat16, 50), rand((N, K), torch.bfloat16, 51, 0.05), rand((N, K), torch.bfloat16, 52, 0.05)
-    for splits in (0, 4, 16):
-        kw = dict(algo=ops.ALGO_SKINNY, splits=splits)
+    blocks = 1 if M <= 16 else 2 if M <= 32 else 4
+    for shape in (0, 1604, 808, 407, 1601):
+        if (shape % 100) * 2 * blocks * 16 * 17 * 4 > 65536:
+            continue   # the waves' tiles of the gated product would not fit in LDS: the library refuses that
+        kw = dict(algo=ops.ALGO_SKINNY, shape=shape)
         torch.testing.assert_close(ops.gemm(a, w, **kw).float(), ref.gemm(a, w).float(), rtol=2e-2, atol=2e-2)
         torch.testing.assert_close(ops.gemm(a, w, w2=w2, **kw).float(), ref.gemm(a, w, w2=w2).float(), rtol=2e-2, atol=2e-2)
         got = ops.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32, **kw)
         torch.testing.assert_close(got, ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
     # the same call twice gives the same bits (the order of the partial sums is fixed)
-    assert torch.equal(ops.gemm(a, w, algo=ops.ALGO_SKINNY, splits=16), ops.gemm(a, w, algo=ops.ALGO_SKINNY, splits=16))
+    assert torch.equal(ops.gemm(a, w, algo=ops.ALGO_SKINNY, shape=804), ops.gemm(a, w, algo=ops.ALGO_SKINNY, shape=804))
     # a view with a row stride, as the attention output is
     wide = rand((M, K + 16), torch.bfloat16, 53)
     torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], w, algo=ops.ALGO_SKINNY).float(), ref.gemm(wide[:, 8:8 + K], w).float(),
@@ -299,7 +302,11 @@ def test_paged_attention_decode(H, Kh, hd, P, window, cap, splits):
     ops.paged_attention_decode(q, kp, vp, table, meta, 2, 3, H, window=window, soft_cap=cap, max_kv_len=max(lens),
                                max_q_len=max(q_lens), out=out2, num_splits=splits)
     a, b = int(meta[2, 1]), int(meta[4, 1] + meta[4, 2])
-    assert torch.equal(out2[a:b], out[a:b]) and (out2[:a] == 7).all() and (out2[b:] == 7).all()
+    # (with its own choice of key ranges the library cuts differently for 3 requests than for 8: equal up to rounding)
+    if splits:
+        assert torch.equal(out2[a:b], out[a:b])
+    torch.testing.assert_close(out2[a:b].float(), out[a:b].float(), rtol=2e-2, atol=2e-2)
+    assert (out2[:a] == 7).all() and (out2[b:] == 7).all()
 
 
 def test_paged_attention_decode_far_key():
@@ -322,3 +329,22 @@ def test_paged_attention_decode_far_key():
         ops.paged_attention_decode(q, kp, vp, table, meta, 0, 1, H, window=window, soft_cap=None, max_kv_len=L,
                                    max_q_len=1, out=out)
         assert (abs(out.float().mean().item() - 3.0) < 0.05) == sees, (window, out.float().mean().item())
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64, 100])
+@pytest.mark.parametrize("N,K", [(48, 64), (100, 72), (333, 1000), (2304, 2048), (1000, 2304)])
+def test_gemm_tiled_weights(M, N, K):
+    """Weights in the tiled layout: the few-rows kernel (M <= 64) and the other kernels read the same numbers."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_tiles, unpack_tiles
+    a, w, w2 = rand((M, K), torch.bfloat16, 70), rand((N, K), torch.bfloat16, 71, 0.05), rand((N, K), torch.bfloat16, 72, 0.05)
+    tw, tw2 = pack_tiles(w), pack_tiles(w2)
+    assert torch.equal(unpack_tiles(tw), w)
+    t = dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(ops.gemm(a, tw).float(), ref.gemm(a, w).float(), **t)
+    torch.testing.assert_close(ops.gemm(a, tw, w2=tw2).float(), ref.gemm(a, w, w2=w2).float(), **t)
+    torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32),
+                               ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+    torch.testing.assert_close(ops.gemm(a, tw, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w).float(), **t)
+    tokens = torch.randint(0, N, (9,), dtype=torch.int32).cuda()
+    torch.testing.assert_close(ops.embed(tw, tokens, 1.5), ref.embed(w, tokens, 1.5), rtol=1e-6, atol=1e-6)

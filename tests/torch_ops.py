@@ -17,7 +17,10 @@ EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
 ALGO_AUTO, ALGO_GENERIC, ALGO_SKINNY, ALGO_TILED = 0, 1, 2, 3
 
 
-def _f(t: torch.Tensor) -> torch.Tensor:
+def _f(t) -> torch.Tensor:
+    if hasattr(t, "rows"):   # a tiled weight
+        from simply_amd.kernels.packing import unpack_tiles
+        t = unpack_tiles(t)
     return t.to(torch.float64 if PRECISE else torch.float32)
 
 
@@ -100,7 +103,7 @@ def gelu_tanh(x):
     return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
 
 
-def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, splits=0):
+def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0):
     out_dtype = out_dtype or a.dtype
     c = _f(a) @ _f(w).T
     if w2 is not None:
