@@ -96,6 +96,9 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
                            hipStream_t stream);
+bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
+int gemm_tiled(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
+               int N, int K, int epi, float cap, hipStream_t stream);
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,

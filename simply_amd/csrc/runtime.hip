@@ -52,7 +52,13 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
     if (takes)
       return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, shape, stream);
   }
-  SA_REQUIRE(algo != 3, "gemm: the tiled MFMA kernel is not built in");
+  if (algo == 3 || (algo == 0 && bf16_in && packed && M > 64)) {
+    const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
+    SA_REQUIRE(takes || algo == 0,
+               "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
+               "aligned operands; got K=%d lda=%lld tiled=%d", K, (long long)lda, packed);
+    if (takes) return gemm_tiled(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, stream);
+  }
   return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, stream);
 }
 

@@ -34,6 +34,7 @@ class StepContext:
     seq_starts: list[int]         # tokens of the request that earlier steps have run
     q_lens: list[int]             # tokens of the request in this step
     cu_q_lens: list[int]          # [S + 1] offsets of the requests in the flat batch
+    _units: dict = dataclasses.field(default_factory=dict)
 
     @property
     def num_seqs(self) -> int:
@@ -54,3 +55,21 @@ class StepContext:
         while n < len(self.q_lens) and self.q_lens[n] <= max_tokens:
             n += 1
         return n, self.cu_q_lens[n]
+
+    def attention_units(self, tokens_per_unit: int) -> tuple[torch.Tensor, int, int]:
+        """The step's tokens cut into units of at most `tokens_per_unit` consecutive tokens of one request, in
+        the layout of `seq_meta` (slot, first token, tokens, first position): what an attention kernel that takes
+        few query rows at a time is launched over.  Returns (units int32 [U, 4] on the device, U, most tokens
+        in a unit).  If no request has more tokens than that, the units are the requests themselves."""
+        if self.max_q_len <= tokens_per_unit:
+            return self.seq_meta, self.num_seqs, self.max_q_len
+        cached = self._units.get(tokens_per_unit)
+        if cached is None:
+            rows = []
+            for slot, first, start, q in zip(self.seq_slots, self.cu_q_lens, self.seq_starts, self.q_lens):
+                for o in range(0, q, tokens_per_unit):
+                    rows.append((slot, first + o, min(tokens_per_unit, q - o), start + o))
+            units = torch.tensor(rows, dtype=torch.int32).to(self.positions.device, non_blocking=True)
+            cached = (units, len(rows), tokens_per_unit)
+            self._units[tokens_per_unit] = cached
+        return cached

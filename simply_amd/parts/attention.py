@@ -69,16 +69,14 @@ class PagedAttention(Mixer):
                                  slot_mapping=group.slot_mapping if write else None,
                                  k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
         o = torch.empty((qkv.shape[0], H * hd), dtype=qkv.dtype, device=qkv.device)
-        # requests with few tokens (decode) go to the kernel that reads each request's keys once for all of its
-        # query heads; the others to the kernel for portions of prompts
-        n_short = t_short = 0
         if ops.decode_attention_takes(qkv, cache.k_pages, H, 1):
-            n_short, t_short = ctx.short_requests(16 // (H // K))
-        if n_short:
-            ops.paged_attention_decode(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.seq_meta, 0, n_short, H,
+            # the MFMA kernel takes up to 16 query rows (tokens x heads per key head) at a time: decoding requests
+            # are one unit each, portions of prompts are cut into units of 16 / G tokens
+            units, num_units, max_q = ctx.attention_units(16 // (H // K))
+            ops.paged_attention_decode(qkv, cache.k_pages, cache.v_pages, group.block_table, units, 0, num_units, H,
                                        window=self.window, soft_cap=self.soft_cap, max_kv_len=ctx.max_kv_len,
-                                       max_q_len=ctx.q_lens[n_short - 1], out=o)
-        if t_short < ctx.num_tokens:
-            ops.paged_attention(qkv[t_short:], cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq[t_short:],
-                                ctx.positions[t_short:], H, window=self.window, soft_cap=self.soft_cap, out=o[t_short:])
+                                       max_q_len=max_q, out=o)
+        else:
+            ops.paged_attention(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions, H,
+                                window=self.window, soft_cap=self.soft_cap, out=o)
         return ops.gemm(o, self.o_proj)

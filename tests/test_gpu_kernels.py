@@ -348,3 +348,24 @@ def test_gemm_tiled_weights(M, N, K):
     torch.testing.assert_close(ops.gemm(a, tw, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w).float(), **t)
     tokens = torch.randint(0, N, (9,), dtype=torch.int32).cuda()
     torch.testing.assert_close(ops.embed(tw, tokens, 1.5), ref.embed(w, tokens, 1.5), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 48, 64), (100, 100, 72), (128, 333, 1000), (300, 2304, 2048), (1, 130, 96),
+                                   (513, 4096, 2304), (2048, 256, 136)])
+def test_gemm_tiled(M, N, K):
+    """The tiled MFMA kernel for many rows, all epilogues, edges in M, N and K."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_tiles
+    a, w, w2 = rand((M, K), torch.bfloat16, 80), rand((N, K), torch.bfloat16, 81, 0.05), rand((N, K), torch.bfloat16, 82, 0.05)
+    tw, tw2 = pack_tiles(w), pack_tiles(w2)
+    t = dict(rtol=2e-2, atol=2e-2)
+    kw = dict(algo=ops.ALGO_TILED)
+    torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), ref.gemm(a, w).float(), **t)
+    torch.testing.assert_close(ops.gemm(a, tw, w2=tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
+    torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw),
+                               ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+    wide = rand((M, K + 16), torch.bfloat16, 83)
+    torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], tw, **kw).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
+    from simply_amd.kernels.lib import KernelError
+    with pytest.raises(KernelError, match="tiled"):
+        ops.gemm(a, w, **kw)     # row-major weights are refused
