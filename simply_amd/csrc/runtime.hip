@@ -34,7 +34,7 @@ extern "C" int sa_version() { return 1; }
 
 extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
                        int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo,
-                       int packed, int shape, hipStream_t stream) {
+                       int packed, int shape, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   SA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
   SA_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld are below K=%d, N=%d", (long long)lda,
@@ -44,7 +44,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
   SA_REQUIRE(algo >= 0 && algo <= 3, "gemm: unknown algorithm %d", algo);
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
-  if (algo == 2 || (algo == 0 && bf16_in && M <= 64)) {
+  if (algo == 2 || (algo == 0 && bf16_in && M <= 16)) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
@@ -52,12 +52,14 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
     if (takes)
       return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, shape, stream);
   }
-  if (algo == 3 || (algo == 0 && bf16_in && packed && M > 64)) {
+  if (algo == 3 || (algo == 0 && bf16_in && packed && M > 16)) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
                "aligned operands; got K=%d lda=%lld tiled=%d", K, (long long)lda, packed);
-    if (takes) return gemm_tiled(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, stream);
+    if (takes)
+      return gemm_tiled(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, shape, workspace,
+                        static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
   }
   return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, stream);
 }

@@ -216,7 +216,8 @@ def fill_(t: torch.Tensor, value_bits: int = 0) -> None:
 
 EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
 
-#: scratch memory for partial results (attention over key ranges), one per device, allocated at first use
+#: scratch memory for partial results (attention over key ranges, products with K cut over workgroups), one per
+#: device, allocated at first use; kernels on one stream use it one after the other
 WORKSPACE_BYTES = 64 << 20
 _scratch: dict = {}
 
@@ -262,8 +263,9 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
     if tuple(out.shape) != (M, N):
         raise KernelError("gemm: bad output shape")
     ldc = _rows(out, "gemm: out")
+    ws = _workspace(a.device)
     _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(wd), _ptr(w2d), _code(wd), _ptr(out), _code(out), ldc, M, N, K, epi,
-              cap, algo, int(packed), int(shape), _stream())
+              cap, algo, int(packed), int(shape), _ptr(ws), ws.numel(), _stream())
     return out
 
 

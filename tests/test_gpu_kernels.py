@@ -351,7 +351,7 @@ def test_gemm_tiled_weights(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 48, 64), (100, 100, 72), (128, 333, 1000), (300, 2304, 2048), (1, 130, 96),
-                                   (513, 4096, 2304), (2048, 256, 136)])
+                                   (513, 4096, 2304), (2048, 256, 136), (17, 100, 200), (64, 2304, 9216), (33, 600, 328)])
 def test_gemm_tiled(M, N, K):
     """The tiled MFMA kernel for many rows, all epilogues, edges in M, N and K."""
     from simply_amd.kernels import ops
@@ -360,10 +360,13 @@ def test_gemm_tiled(M, N, K):
     tw, tw2 = pack_tiles(w), pack_tiles(w2)
     t = dict(rtol=2e-2, atol=2e-2)
     kw = dict(algo=ops.ALGO_TILED)
-    torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), ref.gemm(a, w).float(), **t)
-    torch.testing.assert_close(ops.gemm(a, tw, w2=tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
-    torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw),
-                               ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+    for cuts in (0, 1, 3):   # K whole, or cut over workgroups with the partial tiles added by a second kernel
+        kw = dict(algo=ops.ALGO_TILED, shape=cuts)
+        torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), ref.gemm(a, w).float(), **t)
+        torch.testing.assert_close(ops.gemm(a, tw, w2=tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
+        torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw),
+                                   ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+    kw = dict(algo=ops.ALGO_TILED)
     wide = rand((M, K + 16), torch.bfloat16, 83)
     torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], tw, **kw).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
     from simply_amd.kernels.lib import KernelError
