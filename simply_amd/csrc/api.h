@@ -47,7 +47,9 @@ int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t stream);
 // few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel (2 and 3 refuse what they do not take).
 // packed: W (and W2) are tiled instead of row-major: [ceil(N / 16)][ceil(K / 32)][64][8] bfloat16, block (i, j)
 // holding rows 16 i .. 16 i + 15 and columns 32 j .. 32 j + 31 as element [(k % 32) / 8 * 16 + n % 16][k % 8],
-// zero beyond N and K (one MFMA operand per block, in register order).
+// zero beyond N and K (one MFMA operand per block, in register order).  With epilogue 1 a packed W holds both
+// matrices, their row blocks in turn (block row 2 i: rows 16 i .. of the gate, 2 i + 1: of the other factor), and
+// W2 is null.
 // shape > 0 fixes how a kernel cuts its work: for the few-rows kernel rows of W per workgroup (4, 8 or 16) * 100 +
 // waves, for the tiled kernel the number of cuts of K.  workspace (bytes): scratch memory for partial results
 // when K is cut over workgroups.
@@ -99,9 +101,8 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
                            hipStream_t stream);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
-int gemm_tiled(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
-               int N, int K, int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes,
-               hipStream_t stream);
+int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
+               int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,

@@ -17,11 +17,14 @@ __device__ inline float gelu_tanh(float x) {
   return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
 }
 
-// Index of W[n][k] in memory: row-major, or tiled [N / 16][chunks][kq 4][row 16][8] (chunks = ceil(K / 32)).
+// Index of W[n][k] in memory: row-major, or tiled [N / 16][chunks][kq 4][row 16][8] (chunks = ceil(K / 32)).  With
+// `paired` (the gated epilogue on tiled weights) the tiles of the gate and of the other factor alternate: the gate's
+// tile n / 16 is tile 2 (n / 16), the factor's follows it.
 template <bool PACKED>
-__device__ inline size_t w_index(int n, int k, int K, int chunks) {
+__device__ inline size_t w_index(int n, int k, int K, int chunks, int paired = 0, int second = 0) {
   if (!PACKED) return static_cast<size_t>(n) * K + k;
-  return ((static_cast<size_t>(n / 16) * chunks + k / 32) * 64 + ((k % 32) / 8) * 16 + n % 16) * 8 + k % 8;
+  const size_t tile = paired ? 2 * static_cast<size_t>(n / 16) + second : static_cast<size_t>(n / 16);
+  return ((tile * chunks + k / 32) * 64 + ((k % 32) / 8) * 16 + n % 16) * 8 + k % 8;
 }
 
 // EPI: 0 plain, 1 gated (C = gelu(A.W^T) * (A.W2^T)), 2 soft-cap (C = cap * tanh(A.W^T / cap))
@@ -47,8 +50,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       const int k = k0 + lk + i;
       const int m = m0 + lr, n = n0 + lr;
       As[lk + i][lr] = (m < M && k < K) ? to_float(A[static_cast<size_t>(m) * lda + k]) : 0.f;
-      Ws[lk + i][lr] = (n < N && k < K) ? to_float(W[w_index<PACKED>(n, k, K, chunks)]) : 0.f;
-      if (EPI == 1) W2s[lk + i][lr] = (n < N && k < K) ? to_float(W2[w_index<PACKED>(n, k, K, chunks)]) : 0.f;
+      Ws[lk + i][lr] = (n < N && k < K) ? to_float(W[w_index<PACKED>(n, k, K, chunks, EPI == 1, 0)]) : 0.f;
+      if (EPI == 1)
+        W2s[lk + i][lr] = (n < N && k < K) ? to_float((PACKED ? W : W2)[w_index<PACKED>(n, k, K, chunks, 1, 1)]) : 0.f;
     }
     __syncthreads();
 #pragma unroll

@@ -56,10 +56,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
   const bool row_ok = r < tile_rows && n0 + r < N;
   // row-major W: this lane's row, 8 elements at k.  Tiled W (see pack_tiles): tile (n0 / 16), chunk c is one
   // contiguous 1 KiB block of which this lane owns 16 bytes, padded with zeros beyond N and K.
+  // With the gated epilogue a tiled W holds the two matrices' tiles in turn: tile 2 i the gate, 2 i + 1 the factor.
   const size_t tile_elems = static_cast<size_t>(chunks) * 512;
-  const bf16* wrow = PACKED ? W + (n0 / 16) * tile_elems + lane * 8 : W + static_cast<size_t>(row_ok ? n0 + r : 0) * K;
+  const size_t tile = (EPI == 1 ? 2 : 1) * static_cast<size_t>(n0 / 16);
+  const bf16* wrow = PACKED ? W + tile * tile_elems + lane * 8 : W + static_cast<size_t>(row_ok ? n0 + r : 0) * K;
   const bf16* w2row = EPI != 1 ? nullptr
-                      : PACKED ? W2 + (n0 / 16) * tile_elems + lane * 8
+                      : PACKED ? wrow + tile_elems
                                : W2 + static_cast<size_t>(row_ok ? n0 + r : 0) * K;
   const bf16x8 zero = {};
 

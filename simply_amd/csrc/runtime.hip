@@ -40,7 +40,8 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld are below K=%d, N=%d", (long long)lda,
              (long long)ldc, K, N);
   SA_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm: unknown epilogue %d", epilogue);
-  SA_REQUIRE(epilogue != 1 || W2 != nullptr, "gemm: the gated epilogue needs a second weight");
+  SA_REQUIRE(epilogue != 1 || (W2 != nullptr) != (packed != 0),
+             "gemm: the gated epilogue takes two row-major weights, or one tiled weight that holds both");
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
   SA_REQUIRE(algo >= 0 && algo <= 3, "gemm: unknown algorithm %d", algo);
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
@@ -58,7 +59,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
                "aligned operands; got K=%d lda=%lld tiled=%d", K, (long long)lda, packed);
     if (takes)
-      return gemm_tiled(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, shape, workspace,
+      return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, cap, shape, workspace,
                         static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
   }
   return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, stream);

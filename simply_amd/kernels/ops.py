@@ -232,15 +232,18 @@ def _workspace(device) -> torch.Tensor:
 def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
          soft_cap: float | None = None, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
          algo: int = ALGO_AUTO, shape: int = 0) -> torch.Tensor:
-    """a[M, K] . w[N, K]^T.  With w2: gelu_tanh(a.w^T) * (a.w2^T).  With soft_cap: cap * tanh(. / cap).
-    w (and w2) are row-major tensors or `TiledWeight`s."""
+    """a[M, K] . w[N, K]^T.  With w2 (row-major weights) or a paired `TiledWeight`: gelu_tanh(a.wg^T) * (a.wu^T).
+    With soft_cap: cap * tanh(. / cap).  w is a row-major tensor or a `TiledWeight`."""
     packed = isinstance(w, TiledWeight)
     wd = w.data if packed else w
     w2d = None
+    paired = packed and w.paired
+    if paired and (w2 is not None or soft_cap):
+        raise KernelError("gemm: a paired tiled weight is the gated product by itself")
     if w2 is not None:
-        if isinstance(w2, TiledWeight) != packed:
-            raise KernelError("gemm: both weights must be tiled, or neither")
-        w2d = w2.data if packed else w2
+        if packed or isinstance(w2, TiledWeight):
+            raise KernelError("gemm: tiled weights of a gated product come as one paired weight (pack_gate_up)")
+        w2d = w2
     _dev(a, wd, w2d, out)
     lda = _rows(a, "gemm: a")
     M, K = a.shape
@@ -250,7 +253,9 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
     if wd.dtype != a.dtype:
         raise KernelError(f"gemm: a is {a.dtype} but the weight is {wd.dtype}")
     epi, cap = EPILOGUE_NONE, 0.0
-    if w2 is not None:
+    if paired:
+        epi = EPILOGUE_GATED_GELU
+    elif w2 is not None:
         if soft_cap:
             raise KernelError("gemm: the gated and the soft-cap epilogue do not combine")
         if tuple(w2.shape) != tuple(w.shape) or w2d.dtype != wd.dtype or not w2d.is_contiguous():

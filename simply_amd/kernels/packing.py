@@ -15,9 +15,10 @@ import torch
 
 @dataclasses.dataclass
 class TiledWeight:
-    data: torch.Tensor   # [ceil(N / 16), ceil(K / 32), 64, 8] bfloat16, contiguous
+    data: torch.Tensor   # [ceil(N / 16), ceil(K / 32), 64, 8] bfloat16, contiguous ([2 * ceil(N / 16), ...] if paired)
     rows: int            # N
     cols: int            # K
+    paired: bool = False  # two matrices [N, K], their 16-row tiles in turn (gate, factor, gate, factor, ...)
 
     @property
     def shape(self) -> tuple[int, int]:
@@ -61,7 +62,26 @@ def pack_tiles(w: torch.Tensor, cached: bool = False) -> TiledWeight:
     return tw
 
 
+def pack_gate_up(gate: torch.Tensor, up: torch.Tensor) -> TiledWeight:
+    """Both factors of a gated product as one tiled weight whose 16-row tiles alternate (gate tile i, then the
+    other factor's tile i): a wave that computes 16 output columns streams 2 KiB contiguous blocks, and gate and
+    factor of a column meet in one lane's registers."""
+    if gate.shape != up.shape:
+        raise ValueError("pack_gate_up: the two matrices differ in shape")
+    g, u = pack_tiles(gate).data, pack_tiles(up).data
+    data = torch.stack([g, u], dim=1).reshape(2 * g.shape[0], *g.shape[1:]).contiguous()
+    return TiledWeight(data, gate.shape[0], gate.shape[1], paired=True)
+
+
+def unpack_gate_up(tw: TiledWeight) -> tuple[torch.Tensor, torch.Tensor]:
+    d = tw.data.view(tw.data.shape[0] // 2, 2, *tw.data.shape[1:])
+    return (unpack_tiles(TiledWeight(d[:, 0].contiguous(), tw.rows, tw.cols)),
+            unpack_tiles(TiledWeight(d[:, 1].contiguous(), tw.rows, tw.cols)))
+
+
 def unpack_tiles(tw: TiledWeight) -> torch.Tensor:
+    if tw.paired:
+        raise ValueError("unpack_tiles: a paired weight holds two matrices (unpack_gate_up)")
     nt, nc = tw.data.shape[:2]
     full = tw.data.view(nt, nc, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nt * 16, nc * 32)
     return full[:tw.rows, :tw.cols].contiguous()

@@ -19,16 +19,24 @@ class GatedDense(FeedForward):
         if ACTIVATIONS.get(activation) != ops.EPILOGUE_GATED_GELU:
             raise ValueError(f"gated_dense: activation {activation!r} has no fused kernel")
         self.activation = activation
-        self.gate_proj = self.up_proj = self.down_proj = None
+        self.gate_proj = self.up_proj = self.down_proj = self.gate_up = None
 
     def param_specs(self):
         D, F = self.hidden_size, self.intermediate_size
         return {"gate_proj": ParamSpec((F, D)), "up_proj": ParamSpec((F, D)), "down_proj": ParamSpec((D, F))}
 
     def load(self, tensors):
-        self.gate_proj, self.up_proj, self.down_proj = (as_product_weight(tensors[n])
-                                                        for n in ("gate_proj", "up_proj", "down_proj"))
+        gate, up = tensors["gate_proj"], tensors["up_proj"]
+        if gate.dtype == torch.bfloat16 and gate.is_cuda:
+            # one tiled weight for both factors, their tiles in turn: the fused kernels stream it once
+            from ..kernels.packing import pack_gate_up
+
+            self.gate_up, self.gate_proj, self.up_proj = pack_gate_up(gate, up), None, None
+        else:
+            self.gate_up, self.gate_proj, self.up_proj = None, gate, up
+        self.down_proj = as_product_weight(tensors["down_proj"])
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
-        z = ops.gemm(x, self.gate_proj, w2=self.up_proj)   # gelu(x.Wg^T) * (x.Wu^T), one kernel
+        # gelu(x.Wg^T) * (x.Wu^T), one kernel
+        z = ops.gemm(x, self.gate_up) if self.gate_up is not None else ops.gemm(x, self.gate_proj, w2=self.up_proj)
         return ops.gemm(z, self.down_proj)

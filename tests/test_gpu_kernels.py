@@ -336,13 +336,15 @@ def test_paged_attention_decode_far_key():
 def test_gemm_tiled_weights(M, N, K):
     """Weights in the tiled layout: the few-rows kernel (M <= 64) and the other kernels read the same numbers."""
     from simply_amd.kernels import ops
-    from simply_amd.kernels.packing import pack_tiles, unpack_tiles
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles, unpack_gate_up, unpack_tiles
     a, w, w2 = rand((M, K), torch.bfloat16, 70), rand((N, K), torch.bfloat16, 71, 0.05), rand((N, K), torch.bfloat16, 72, 0.05)
-    tw, tw2 = pack_tiles(w), pack_tiles(w2)
+    tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
     assert torch.equal(unpack_tiles(tw), w)
+    assert all(torch.equal(x, y) for x, y in zip(unpack_gate_up(tw2), (w, w2)))
     t = dict(rtol=2e-2, atol=2e-2)
     torch.testing.assert_close(ops.gemm(a, tw).float(), ref.gemm(a, w).float(), **t)
-    torch.testing.assert_close(ops.gemm(a, tw, w2=tw2).float(), ref.gemm(a, w, w2=w2).float(), **t)
+    torch.testing.assert_close(ops.gemm(a, tw2).float(), ref.gemm(a, w, w2=w2).float(), **t)
+    torch.testing.assert_close(ops.gemm(a, tw2, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w, w2=w2).float(), **t)
     torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32),
                                ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
     torch.testing.assert_close(ops.gemm(a, tw, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w).float(), **t)
@@ -355,15 +357,15 @@ def test_gemm_tiled_weights(M, N, K):
 def test_gemm_tiled(M, N, K):
     """The tiled MFMA kernel for many rows, all epilogues, edges in M, N and K."""
     from simply_amd.kernels import ops
-    from simply_amd.kernels.packing import pack_tiles
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles
     a, w, w2 = rand((M, K), torch.bfloat16, 80), rand((N, K), torch.bfloat16, 81, 0.05), rand((N, K), torch.bfloat16, 82, 0.05)
-    tw, tw2 = pack_tiles(w), pack_tiles(w2)
+    tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
     t = dict(rtol=2e-2, atol=2e-2)
     kw = dict(algo=ops.ALGO_TILED)
     for cuts in (0, 1, 3):   # K whole, or cut over workgroups with the partial tiles added by a second kernel
         kw = dict(algo=ops.ALGO_TILED, shape=cuts)
         torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), ref.gemm(a, w).float(), **t)
-        torch.testing.assert_close(ops.gemm(a, tw, w2=tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
+        torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
         torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw),
                                    ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
     kw = dict(algo=ops.ALGO_TILED)

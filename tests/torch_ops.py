@@ -105,6 +105,9 @@ def gelu_tanh(x):
 
 def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0):
     out_dtype = out_dtype or a.dtype
+    if getattr(w, "paired", False):
+        from simply_amd.kernels.packing import unpack_gate_up
+        w, w2 = unpack_gate_up(w)
     c = _f(a) @ _f(w).T
     if w2 is not None:
         up = _f(a) @ _f(w2).T
