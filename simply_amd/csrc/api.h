@@ -58,7 +58,8 @@ int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* 
             void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // Attention of T query tokens over paged keys and values.
-//   q[t, h, :] at q + t * q_stride + h * hd; key pages are [num_pages, Kh, page_size, hd], value pages
+//   q[t, h, :] at q + t * q_stride + h * hd; key pages are [num_pages, Kh, page_size, hd] (each page row-major, or
+//   in blocks of operand order if page_size % 16 == 0 and hd % 32 == 0: see key_index in common.h), value pages
 //   [num_pages, Kh, hd, page_size];
 //   token_seq[t] is the row of block_table of the token's request, positions[t] its absolute position;
 //   window 0: all earlier keys, else the last `window` keys including the token's own; soft_cap 0: none.

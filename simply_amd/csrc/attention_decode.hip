@@ -6,7 +6,8 @@
 // columns of one MFMA tile, so keys and values are read once for all of them.  Per tile of 32 keys a
 // wave computes
 //     S^T[key, row] = K[key, :] . Q[row, :]     v_mfma_f32_16x16x32_bf16, K rows as the A operand,
-//                                               loaded straight from the page (16 keys = 8 KiB)
+//                                               loaded straight from the page, where 16 keys x 32
+//                                               dimensions are stored as one operand (a contiguous KiB)
 //     soft-cap, mask, running maximum and sum per row (float32)
 //     O^T[d, row]  += V^T[d, key] . P^T[key, row]
 // The second product needs no data movement: S^T comes out of the first MFMA in the register
@@ -108,7 +109,8 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
       const int page = table[sk0 / page_size];
       const int off = sk0 % page_size;  // a multiple of 16
       const size_t head = static_cast<size_t>(page) * Kh + kh;
-      st.k = k_pages + (head * page_size + off + r) * HD + grp * 8;
+      // keys are stored in 16-key x 32-dimension blocks of operand order: block (off / 16, dc) is a contiguous KiB
+      st.k = k_pages + head * page_size * HD + static_cast<size_t>(off / 16) * (NDC * 512) + lane * 8;
       st.v = v_pages + (head * HD + r) * page_size + off + grp * 4;
     }
     return st;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int dc = 0; dc < NDC; ++dc) kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 32) : zero8;
+    for (int dc = 0; dc < NDC; ++dc) kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 512) : zero8;
 
   for (; tile < te; tile += 4) {
     const int key0 = tile * kTile;
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int dc = 0; dc < NDC; ++dc)
-        kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 32) : zero8;
+        kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 512) : zero8;
     // ---- cap, mask, online softmax.  Lane (row r, grp) holds keys sk0 + 4 * grp + v of each sub-tile.
     float p[2][4];
     float mx = -INFINITY;

@@ -37,6 +37,7 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
   int* page_s = reinterpret_cast<int*>(a_s + G);  // [kChunk] page of each key of the chunk
 
   const int t = blockIdx.x, kh = blockIdx.y, tid = threadIdx.x;
+  const bool tiled = keys_tiled(page_size, hd);
   const int seq = token_seq[t];
   const int pos = positions[t];
   const int hi = pos + 1;
@@ -78,9 +79,10 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
         for (int g = 0; g < 8; ++g) dot[g] = 0.f;
         if (valid) {
           const int key = c0 + j;
-          const T* kp = k_pages + ((static_cast<size_t>(page_s[j]) * Kh + kh) * page_size + key % page_size) * hd;
+          const T* kp = k_pages + (static_cast<size_t>(page_s[j]) * Kh + kh) * page_size * hd;
+          const int kin = key % page_size;
           for (int d = part; d < hd; d += 4) {
-            const float kv = to_float(kp[d]);
+            const float kv = to_float(kp[key_index(tiled, page_size, hd, kin, d)]);
 #pragma unroll
             for (int g = 0; g < 8; ++g)
               if (g < gn) dot[g] = fmaf(q_s[(g0 + g) * hd + d], kv, dot[g]);

@@ -75,6 +75,16 @@ __device__ inline float block_sum(float v, float* scratch /* >= 16 floats */) {
   return total;
 }
 
+// Layout of a page of keys [page_size keys][hd]: row-major, or, when the sizes allow it, in 16-key x 32-dimension
+// blocks of MFMA operand order (as weight tiles are): [page_size / 16][hd / 32][lane 64][8] with
+// lane = (d % 32) / 8 * 16 + key % 16, so that a wave reads a block of 16 keys as contiguous KiB.
+__host__ __device__ inline bool keys_tiled(int page_size, int hd) { return page_size % 16 == 0 && hd % 32 == 0; }
+__host__ __device__ inline size_t key_index(bool tiled, int page_size, int hd, int key_in_page, int d) {
+  if (!tiled) return static_cast<size_t>(key_in_page) * hd + d;
+  return ((static_cast<size_t>(key_in_page / 16) * (hd / 32) + d / 32) * 64 + ((d % 32) / 8) * 16 + key_in_page % 16) * 8 +
+         d % 8;
+}
+
 // Error channel: entry points return 0 on success, non-zero after set_error().
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);

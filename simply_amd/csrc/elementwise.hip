@@ -46,12 +46,56 @@ __global__ void rmsnorm_kernel(const void* __restrict__ x, int x_dtype, int64_t 
 
 // residual[t, :] += norm(y[t, :]; w_post);  then, if w_next: out[t, :] = norm(residual[t, :]; w_next).
 // The residual stream is 32-bit.  simply/model_lib.py:2681-2683 and :2690.
+// Rows of up to kRowRegs * blockDim elements are held in registers: every input is read once and all loads are
+// issued before the first reduction, so that the kernel pays the memory latency once (it runs a hundred times
+// per decode step on a handful of rows).
+constexpr int kRowRegs = 4;
 __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, const void* __restrict__ w_post,
                                    int w_post_dtype, float eps_post, float plus_one_post, float* __restrict__ residual,
                                    const void* __restrict__ w_next, int w_next_dtype, float eps_next,
                                    float plus_one_next, void* __restrict__ out, int out_dtype, int D) {
   __shared__ float scratch[16];
   const size_t rb = static_cast<size_t>(blockIdx.x) * D;
+  if (D <= kRowRegs * static_cast<int>(blockDim.x)) {
+    float yv[kRowRegs], hv[kRowRegs], wp[kRowRegs], wn[kRowRegs];
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+      const int d = threadIdx.x + j * blockDim.x;
+      const bool ok = d < D;
+      yv[j] = ok ? load_f(y, y_dtype, rb + d) : 0.f;
+      hv[j] = ok ? residual[rb + d] : 0.f;
+      wp[j] = (ok && w_post != nullptr) ? load_f(w_post, w_post_dtype, d) + plus_one_post : 1.f;
+      wn[j] = (ok && w_next != nullptr) ? load_f(w_next, w_next_dtype, d) + plus_one_next : 1.f;
+    }
+    float r = 1.f;
+    if (w_post != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < kRowRegs; ++j) ss += yv[j] * yv[j];
+      ss = block_sum(ss, scratch);
+      r = rsqrtf(ss / static_cast<float>(D) + eps_post);
+    }
+    float ss2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+      const int d = threadIdx.x + j * blockDim.x;
+      const float v = w_post != nullptr ? yv[j] * r * wp[j] : yv[j];
+      hv[j] += v;
+      if (d < D) {
+        residual[rb + d] = hv[j];
+        ss2 += hv[j] * hv[j];
+      }
+    }
+    if (w_next == nullptr) return;
+    ss2 = block_sum(ss2, scratch);
+    const float r2 = rsqrtf(ss2 / static_cast<float>(D) + eps_next);
+#pragma unroll
+    for (int j = 0; j < kRowRegs; ++j) {
+      const int d = threadIdx.x + j * blockDim.x;
+      if (d < D) store_f(out, out_dtype, rb + d, hv[j] * r2 * wn[j]);
+    }
+    return;
+  }
   float ss = 0.f;
   if (w_post != nullptr) {
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
@@ -81,7 +125,7 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
 // ------------------------------------------------------------------ rotary + cache write
 // One block per (token, head) of a fused [T, (H + 2K) * hd] projection.
 //   q heads: rotate, divide by query_scale, write back in place.
-//   k heads: rotate, write into the key pages at slot_mapping[t].
+//   k heads: rotate, write into the key pages at slot_mapping[t] (pages in the layout of key_index()).
 //   v heads: copy into the value pages (stored transposed: [page, head, hd, page_size]).
 // Angles: pos / timescale[i] / scale_factor, pairs (i, i + hd/2).  simply/utils/position_encoding.py:83-110;
 // the query scale comes after the rotation (simply/model_lib.py:2010-2019).
@@ -98,13 +142,18 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
   if (head < H + K) {
     const bool is_q = head < H;
     T* dst = src;
+    bool to_pages = false;
+    int koff = 0;
     if (!is_q) {
       if (k_pages == nullptr) return;
       const int64_t slot = slot_mapping[t];
       if (slot < 0) return;
-      const int64_t page = slot / page_size, off = slot % page_size;
-      dst = k_pages + ((page * K + (head - H)) * page_size + off) * hd;
+      const int64_t page = slot / page_size;
+      koff = static_cast<int>(slot % page_size);
+      dst = k_pages + (page * K + (head - H)) * page_size * hd;
+      to_pages = true;
     }
+    const bool tiled = to_pages && keys_tiled(page_size, hd);
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
       const float x1 = to_float(src[i]), x2 = to_float(src[i + half]);
       float o1 = x1, o2 = x2;
@@ -119,8 +168,13 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
         o1 = o1 / q_div;
         o2 = o2 / q_div;
       }
-      dst[i] = from_float<T>(o1);
-      dst[i + half] = from_float<T>(o2);
+      if (to_pages) {
+        dst[key_index(tiled, page_size, hd, koff, i)] = from_float<T>(o1);
+        dst[key_index(tiled, page_size, hd, koff, i + half)] = from_float<T>(o2);
+      } else {
+        dst[i] = from_float<T>(o1);
+        dst[i + half] = from_float<T>(o2);
+      }
     }
   } else {
     if (v_pages == nullptr) return;

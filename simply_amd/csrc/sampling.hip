@@ -38,12 +38,14 @@ __host__ __device__ inline Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
   return o;
 }
 
-// Standard Gumbel noise for vocabulary entry `index` of draw `counter` under `seed`.
-__device__ inline float gumbel_noise(uint64_t seed, uint32_t counter, uint32_t index) {
-  const Philox4 r = philox4x32_10(index >> 2, counter, 0u, 0u, static_cast<uint32_t>(seed),
-                                  static_cast<uint32_t>(seed >> 32));
-  const float u = (static_cast<float>(r.v[index & 3u] >> 8) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
-  return -logf(-logf(u));
+// Gumbel noise for the four vocabulary entries 4 b .. 4 b + 3 (one generator block).
+__device__ inline void gumbel_noise4(uint64_t seed, uint32_t counter, uint32_t block, float out[4]) {
+  const Philox4 r = philox4x32_10(block, counter, 0u, 0u, static_cast<uint32_t>(seed), static_cast<uint32_t>(seed >> 32));
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float u = (static_cast<float>(r.v[j] >> 8) + 0.5f) * (1.0f / 16777216.0f);
+    out[j] = -logf(-logf(u));
+  }
 }
 
 // Maps a float to an unsigned key with the same order.
@@ -152,9 +154,26 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const int k = top_k[r];
   const float p = top_p[r];
 
+  // rows are read four entries at a time where their address allows it (every row does if the stride is a
+  // multiple of four); the few entries before and after the aligned part are read singly
+  const int head = static_cast<int>((4 - (reinterpret_cast<uintptr_t>(row) / 4) % 4) % 4) < V
+                       ? static_cast<int>((4 - (reinterpret_cast<uintptr_t>(row) / 4) % 4) % 4) : V;
+  const int quads = (V - head) / 4;
+  const float4* row4 = reinterpret_cast<const float4*>(row + head);
+  const int tail0 = head + 4 * quads;
+
   if (temp == 0.f || k == 1) {
     ArgMax a{-INFINITY, 0x7fffffff};
-    for (int i = threadIdx.x; i < V; i += blockDim.x) a = better(a, ArgMax{row[i], i});
+    for (int i = threadIdx.x; i < head; i += blockDim.x) a = better(a, ArgMax{row[i], i});
+    for (int b = threadIdx.x; b < quads; b += blockDim.x) {
+      const float4 x = row4[b];
+      const int i = head + 4 * b;
+      a = better(a, ArgMax{x.x, i});
+      a = better(a, ArgMax{x.y, i + 1});
+      a = better(a, ArgMax{x.z, i + 2});
+      a = better(a, ArgMax{x.w, i + 3});
+    }
+    for (int i = tail0 + threadIdx.x; i < V; i += blockDim.x) a = better(a, ArgMax{row[i], i});
     a = block_argmax(a, am_scratch);
     if (threadIdx.x == 0) {
       tokens[r] = a.i;
@@ -165,7 +184,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
   const float inv_t = 1.f / temp;
   float mx = -INFINITY;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
+  for (int i = threadIdx.x; i < head; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
+  for (int b = threadIdx.x; b < quads; b += blockDim.x) {
+    const float4 x = row4[b];
+    mx = fmaxf(fmaxf(mx, x.x * inv_t), fmaxf(fmaxf(x.y * inv_t, x.z * inv_t), x.w * inv_t));
+  }
+  for (int i = tail0 + threadIdx.x; i < V; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
   mx = block_max(mx, f_scratch);
 
   // Entries whose key is >= floor_key stay (the mask of the reference, as a threshold).
@@ -200,11 +224,19 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const uint32_t ctr = static_cast<uint32_t>(counter[r]);
   ArgMax a{-INFINITY, 0x7fffffff};
   float sum = 0.f;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
-    const float x = row[i] * inv_t;
-    if (ordered_key(x) < floor_key) continue;
-    sum += expf(x - mx);
-    a = better(a, ArgMax{x + gumbel_noise(sd, ctr, static_cast<uint32_t>(i)), i});
+  // one generator block gives the noise of four consecutive entries
+  for (int b = threadIdx.x; 4 * b < V; b += blockDim.x) {
+    float g[4];
+    gumbel_noise4(sd, ctr, static_cast<uint32_t>(b), g);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = 4 * b + j;
+      if (i >= V) break;
+      const float x = row[i] * inv_t;
+      if (ordered_key(x) < floor_key) continue;
+      sum += expf(x - mx);
+      a = better(a, ArgMax{x + g[j], i});
+    }
   }
   a = block_argmax(a, am_scratch);
   sum = block_sum(sum, f_scratch);

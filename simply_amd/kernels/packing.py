@@ -93,3 +93,27 @@ def clear_cache() -> None:
 
 def concat_rows(*ws: torch.Tensor) -> torch.Tensor:
     return torch.cat(ws, dim=0).contiguous()
+
+
+# ---- pages of keys
+
+def keys_tiled(page_size: int, head_dim: int) -> bool:
+    """Whether the kernels keep a page of keys in 16-key x 32-dimension blocks of MFMA operand order
+    ([page_size / 16][head_dim / 32][64][8]) rather than row-major [page_size][head_dim]."""
+    return page_size % 16 == 0 and head_dim % 32 == 0
+
+
+def keys_to_rows(k_pages: torch.Tensor) -> torch.Tensor:
+    """[pages, heads, page_size, head_dim] as the kernels store it -> row-major copy (tests, inspection)."""
+    n, h, P, hd = k_pages.shape
+    if not keys_tiled(P, hd):
+        return k_pages.clone()
+    return k_pages.reshape(n, h, P // 16, hd // 32, 4, 16, 8).permute(0, 1, 2, 5, 3, 4, 6).reshape(n, h, P, hd).contiguous()
+
+
+def rows_to_keys(rows: torch.Tensor) -> torch.Tensor:
+    """Row-major [pages, heads, page_size, head_dim] -> the kernels' storage order (same shape)."""
+    n, h, P, hd = rows.shape
+    if not keys_tiled(P, hd):
+        return rows.clone()
+    return rows.reshape(n, h, P // 16, 16, hd // 32, 4, 8).permute(0, 1, 2, 4, 5, 3, 6).reshape(n, h, P, hd).contiguous()

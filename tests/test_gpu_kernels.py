@@ -137,7 +137,8 @@ def paged_setup(dtype, S, H, Kh, hd, P, lens, seed):
             n = min(P, l - b * P)
             kp[page, :, :n] = torch.randn((Kh, n, hd), generator=g).to(dtype)
             vp[page, :, :, :n] = torch.randn((Kh, hd, n), generator=g).to(dtype)
-    return kp.cuda(), vp.cuda(), table.cuda()
+    from simply_amd.kernels.packing import rows_to_keys
+    return rows_to_keys(kp).cuda(), vp.cuda(), table.cuda()
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -171,12 +172,14 @@ def test_paged_attention_far_key_and_window_edge():
     from simply_amd.kernels import ops
     H = Kh = 1
     hd, P, L = 32, 16, 300
+    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
     kp, vp, table = paged_setup(torch.float32, 1, H, Kh, hd, P, [L], 31)
-    kp.mul_(0.01)
+    kp = keys_to_rows(kp) * 0.01
     far = 37
     page, off = int(table[0, far // P]), far % P
     kp[page, 0, off] = 0.0
     kp[page, 0, off, 3] = 50.0
+    kp = rows_to_keys(kp)
     vp[page, 0, :, off] = 7.0
     q = torch.zeros((1, hd)).cuda()
     q[0, 3] = 1.0
@@ -313,12 +316,14 @@ def test_paged_attention_decode_far_key():
     """A key 3000 positions back with a score that stands out, among keys cut over many workgroups."""
     from simply_amd.kernels import ops
     H, Kh, hd, P, L = 2, 1, 128, 16, 3100
+    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
     kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 63)
-    kp.mul_(0.01)
+    kp = keys_to_rows(kp) * 0.01
     far = 71
     page, off = int(table[0, far // P]), far % P
     kp[page, 0, off] = 0.0
     kp[page, 0, off, 5] = 60.0
+    kp = rows_to_keys(kp)
     vp[page, 0, :, off] = 3.0
     meta, ts, ps = seq_meta_for([L], [1])
     q = torch.zeros((1, 4 * hd), dtype=torch.bfloat16).cuda()
@@ -374,3 +379,36 @@ def test_gemm_tiled(M, N, K):
     from simply_amd.kernels.lib import KernelError
     with pytest.raises(KernelError, match="tiled"):
         ops.gemm(a, w, **kw)     # row-major weights are refused
+
+
+def test_add_rmsnorm_wide_rows():
+    """Rows wider than the kernel keeps in registers take its second code path."""
+    from simply_amd.kernels import ops
+    T, D = 3, 5000
+    y, h = rand((T, D), torch.bfloat16, 90, 2.0), rand((T, D), torch.float32, 91, 5.0)
+    w1, w2 = rand((D,), torch.bfloat16, 92, 0.3), rand((D,), torch.bfloat16, 93, 0.3)
+    h_ref = h.clone()
+    o = ops.add_rmsnorm(y, h, post_weight=w1, post_eps=1e-6, next_weight=w2, next_eps=1e-6, out_dtype=torch.bfloat16)
+    o_ref = ref.add_rmsnorm(y, h_ref, post_weight=w1, post_eps=1e-6, next_weight=w2, next_eps=1e-6, out_dtype=torch.bfloat16)
+    torch.testing.assert_close(h, h_ref, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(o.float(), o_ref.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_sampling_rows_at_odd_addresses():
+    """Rows whose stride is no multiple of four entries: the kernel's four-at-a-time reads start at an aligned
+    entry and the rest is read singly."""
+    from simply_amd.kernels import ops
+    V, R = 1001, 5
+    wide = rand((R, V + 2), torch.float32, 94, 3.0)
+    logits = wide[:, 1:1 + V]
+    temperature = torch.tensor([0.0, 0.8, 0.0, 1.2, 0.0]).cuda()
+    top_k = torch.tensor([-1, -1, -1, 30, -1], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 1.0, 1.0, 0.9, 1.0]).cuda()
+    seed = torch.tensor([9, 8, 7, 6, 5], dtype=torch.int64).cuda()
+    counter = torch.tensor([0, 1, 2, 3, 4], dtype=torch.int32).cuda()
+    tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
+    rtok, rlp = ref.sample(logits, temperature, top_k, top_p, seed, counter)
+    assert tok.tolist() == rtok.tolist()
+    torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+    for r in (0, 2, 4):
+        assert tok[r].item() == int(logits[r].argmax())

@@ -74,9 +74,12 @@ def rope_cache_write(qkv, positions, timescale, scale_factor, q_div, num_heads, 
     q = q / q_div
     qkv[:, :H * hd] = q.reshape(T, H * hd).to(qkv.dtype)
     if k_pages is not None:
+        from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
         P = k_pages.shape[2]
         page, off = slot_mapping[:T] // P, slot_mapping[:T] % P
-        k_pages[page, :, off] = k.to(k_pages.dtype)
+        rows = keys_to_rows(k_pages)      # the kernels' storage order of keys -> row-major, and back
+        rows[page, :, off] = k.to(k_pages.dtype)
+        k_pages.copy_(rows_to_keys(rows))
         v_pages[page, :, :, off] = v.to(v_pages.dtype)     # value pages are [page, head, hd, page_size]
 
 
@@ -123,8 +126,10 @@ def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shap
 
 def paged_attention(q, k_pages, v_pages, block_table, token_seq, positions, num_heads, *, window, soft_cap, out=None,
                     algo=0):
+    from simply_amd.kernels.packing import keys_to_rows
     T = q.shape[0]
     _, Kh, P, hd = k_pages.shape
+    k_pages = keys_to_rows(k_pages)
     H = num_heads
     G = H // Kh
     res = torch.empty((T, H * hd), dtype=q.dtype, device=q.device)
