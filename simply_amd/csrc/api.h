@@ -57,6 +57,15 @@ int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* 
             int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, int packed, int shape,
             void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
+// For 1..16 rows of bfloat16: h_out = h_in + norm(y; w_post) (y null: h_out is h_in and is not written; w_post null:
+// h_out = h_in + y), a = norm(h_out; w_next), C = epilogue(a . W^T) with W tiled (paired tiles for epilogue 1).
+// h_in, h_out: float32 [M, K], different buffers; y: bfloat16 [M, K]; norm weights float32 or bfloat16 [K].
+int sa_gemm_normed_takes(int M, int N, int K);
+int sa_gemm_normed(const void* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype, float eps_post,
+                   int plus_one_post, const void* w_next, int w_next_dtype, float eps_next, int plus_one_next,
+                   const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap,
+                   hipStream_t stream);
+
 // Attention of T query tokens over paged keys and values.
 //   q[t, h, :] at q + t * q_stride + h * hd; key pages are [num_pages, Kh, page_size, hd] (each page row-major, or
 //   in blocks of operand order if page_size % 16 == 0 and hd % 32 == 0: see key_index in common.h), value pages

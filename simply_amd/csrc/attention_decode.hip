@@ -91,12 +91,13 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   for (int db = 0; db < NDB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;  // per row (lane % 16); l_run is this lane group's share
 
-  // The loop is software-pipelined so that a wave always has loads in flight: the keys of the next tile are
-  // requested before the scores of this tile are turned into probabilities, and the values of this tile are
-  // requested before its scores are computed.
+  // The loop is software-pipelined over two sets of registers (A and B), each holding the keys and the values of
+  // one tile: while a tile is computed from one set, the loads of the next tile are in flight into the other, and
+  // each half of a set (keys, values) is requested again for the tile after next as soon as it has been used.  A
+  // wave thus keeps about 48 KiB of loads in flight; with one workgroup per CU that is what hides the latency.
   struct SubTile {
     bool ok;            // some key of the sub-tile is in [lo, hi): its page exists
-    const bf16* k;      // this lane's key row, at its 8 dimensions of chunk 0
+    const bf16* k;      // this lane's 16 bytes of the sub-tile's first key block
     const bf16* v;      // this lane's value row (dimension r of block 0), at its 4 keys
   };
   auto locate = [&](int tile, int t) {
@@ -117,41 +118,47 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   };
   const bf16x8 zero8 = {};
   const bf16x4 zero4 = {};
-
-  int tile = tb + wave;
-  SubTile cur[2] = {locate(tile, 0), locate(tile, 1)};
-  bf16x8 kf[2][NDC];
-#pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int dc = 0; dc < NDC; ++dc) kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 512) : zero8;
-
-  for (; tile < te; tile += 4) {
-    const int key0 = tile * kTile;
-    // ---- request this tile's values
+  struct TileRegs {
+    SubTile st[2];
+    bf16x8 kf[2][NDC];
     bf16x4 vf[2][NDB];
+  };
+  auto request_keys = [&](TileRegs& b, int tile) {
+    b.st[0] = locate(tile, 0);
+    b.st[1] = locate(tile, 1);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int dc = 0; dc < NDC; ++dc)
+        b.kf[t][dc] = b.st[t].ok ? *reinterpret_cast<const bf16x8*>(b.st[t].k + dc * 512) : zero8;
+  };
+  auto request_values = [&](TileRegs& b) {  // of the tile whose keys were requested last
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
-        vf[t][db] = cur[t].ok ? *reinterpret_cast<const bf16x4*>(cur[t].v + static_cast<size_t>(db) * 16 * page_size) : zero4;
+        b.vf[t][db] = b.st[t].ok ? *reinterpret_cast<const bf16x4*>(b.st[t].v + static_cast<size_t>(db) * 16 * page_size)
+                                 : zero4;
+  };
+  // One tile from the registers of `b`; its keys, then its values, are requested anew for tile `next`.
+  auto process = [&](TileRegs& b, int tile, int next) {
+    const int key0 = tile * kTile;
+    const bool sub_ok[2] = {b.st[0].ok, b.st[1].ok};
     // ---- scores of the two sub-tiles of 16 keys
     floatx4 s[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int dc = 0; dc < NDC; ++dc) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][dc], qf[dc], s[t], 0, 0, 0);
+      for (int dc = 0; dc < NDC; ++dc) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.kf[t][dc], qf[dc], s[t], 0, 0, 0);
     }
-    const bool sub_ok[2] = {cur[0].ok, cur[1].ok};
-    // ---- request the next tile's keys
-    cur[0] = locate(tile + 4, 0);
-    cur[1] = locate(tile + 4, 1);
+    // the values of this tile are still needed: only the key half of the set is requested now
+    bf16x4 vcur[2][NDB];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int dc = 0; dc < NDC; ++dc)
-        kf[t][dc] = cur[t].ok ? *reinterpret_cast<const bf16x8*>(cur[t].k + dc * 512) : zero8;
+      for (int db = 0; db < NDB; ++db) vcur[t][db] = b.vf[t][db];
+    request_keys(b, next);
     // ---- cap, mask, online softmax.  Lane (row r, grp) holds keys sk0 + 4 * grp + v of each sub-tile.
     float p[2][4];
     float mx = -INFINITY;
@@ -193,7 +200,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) a[t * 4 + v] = vf[t][db][v];
+        for (int v = 0; v < 4; ++v) a[t * 4 + v] = vcur[t][db][v];
       if (tail) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -205,6 +212,18 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
       for (int v = 0; v < 4; ++v) acc[db][v] *= alpha;
       acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, acc[db], 0, 0, 0);
     }
+    request_values(b);
+  };
+
+  TileRegs A, B;
+  int tile = tb + wave;
+  request_keys(A, tile);
+  request_values(A);
+  request_keys(B, tile + 4);
+  request_values(B);
+  for (; tile < te; tile += 8) {
+    process(A, tile, tile + 8);
+    if (tile + 4 < te) process(B, tile + 4, tile + 12);
   }
 
   // ---- merge the four waves in two rounds through LDS (waves 2, 3 into 0, 1; then 1 into 0).

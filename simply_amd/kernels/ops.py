@@ -274,6 +274,45 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
     return out
 
 
+def gemm_normed_takes(M: int, w) -> bool:
+    """Whether `gemm_normed` takes M rows against the weight `w`."""
+    if not isinstance(w, TiledWeight) or not w.data.is_cuda:
+        return False
+    return bool(_lib.load().sa_gemm_normed_takes(int(M), int(w.rows), int(w.cols)))
+
+
+def gemm_normed(y: torch.Tensor | None, h_in: torch.Tensor, h_out: torch.Tensor | None, w: TiledWeight, *,
+                post_weight: torch.Tensor | None, post_eps: float, post_plus_one: bool, next_weight: torch.Tensor,
+                next_eps: float, next_plus_one: bool, soft_cap: float | None = None,
+                out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """h_out = h_in + norm(y; post) (y None: the residual stays h_in); returns epilogue(norm(h_out; next) . w^T),
+    in one kernel, for up to 16 rows.  The residual buffers are float32 [M, K] and must differ."""
+    _dev(y, h_in, h_out, post_weight, next_weight, w.data)
+    M, K = h_in.shape
+    if h_in.dtype != torch.float32 or not h_in.is_contiguous() or w.cols != K:
+        raise KernelError("gemm_normed: the residual must be contiguous float32 [M, K] with K the weight's width")
+    if y is not None:
+        if y.dtype != torch.bfloat16 or tuple(y.shape) != (M, K) or not y.is_contiguous():
+            raise KernelError("gemm_normed: y must be contiguous bfloat16 [M, K]")
+        if h_out is None or h_out.dtype != torch.float32 or tuple(h_out.shape) != (M, K) or not h_out.is_contiguous() \
+                or h_out.data_ptr() == h_in.data_ptr():
+            raise KernelError("gemm_normed: the updated residual needs its own contiguous float32 [M, K] buffer")
+    for t in (post_weight, next_weight):
+        if t is not None and (t.numel() != K or not t.is_contiguous()):
+            raise KernelError("gemm_normed: a norm weight does not match the width")
+    epi, cap = EPILOGUE_NONE, 0.0
+    if w.paired:
+        epi = EPILOGUE_GATED_GELU
+    elif soft_cap:
+        epi, cap = EPILOGUE_SOFT_CAP, float(soft_cap)
+    out = torch.empty((M, w.rows), dtype=out_dtype, device=h_in.device)
+    _lib.call("sa_gemm_normed", _ptr(y), _ptr(h_in), _ptr(h_out), _ptr(post_weight),
+              _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one),
+              _ptr(next_weight), _code(next_weight), float(next_eps), int(next_plus_one), _ptr(w.data), _ptr(out),
+              _code(out), out.stride(0), M, w.rows, K, epi, cap, _stream())
+    return out
+
+
 # --------------------------------------------------------------------------- attention
 
 

@@ -13,7 +13,7 @@ import torch
 from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.spec import LayerSpec, ModelSpec, PartSpec
 from ..kernels import ops
-from ..parts.base import Block, ParamSpec, Part
+from ..parts.base import Block, ParamSpec, Part, PendingNorm
 from ..parts.embedding import EMBEDDINGS, HEADS
 from ..registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 
@@ -91,8 +91,9 @@ class DecoderModel:
             block = self.layers[entry.layer]
             nxt = self.layers[schedule[i + 1].layer].first_norm() if i + 1 < len(schedule) else None
             h, normed = block.forward(h, ctx, cache_views[i], normed, nxt)
+        if isinstance(normed, PendingNorm):
+            h = normed.settle()      # the last block's residual sum, if it is still pending
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         rows = ops.gather_rows(h, logit_rows)
-        x = self.final_norm.forward(rows, ctx.dtype)
-        return self.head.forward(x)
+        return self.head.forward(PendingNorm(rows, None, None, self.final_norm, ctx.dtype))

@@ -11,11 +11,13 @@ import torch
 from ..config.spec import PartSpec
 from ..kernels import ops
 from ..registry import MIXERS, POSITION_ENCODINGS
-from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight
+from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight, project
 
 
 @MIXERS.register("paged_attention")
 class PagedAttention(Mixer):
+    accepts_pending = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, query_scale: float,
                  soft_cap: float | None = None, window: int | None = None,
                  position_encoding: PartSpec | None = None):
@@ -52,7 +54,7 @@ class PagedAttention(Mixer):
     def forward(self, x, ctx, cache):
         H, K, hd = self.num_heads, self.num_kv_heads, self.head_dim
         group = ctx.groups[cache.group_id]
-        qkv = ops.gemm(x, self.qkv_proj)
+        qkv = project(x, self.qkv_proj)
         pe = self.position_encoding
         rotary = pe.rotary_table() if pe is not None else None
         write = cache.write

@@ -14,6 +14,9 @@ Parts, per kind, and what each must provide:
 * Mixer:            cache_need(); forward(x, ctx, cache) -> y
 * FeedForward:      forward(x, ctx) -> y
 * Block:            first_norm(); forward(h, ctx, cache, normed, next_norm) -> (h, normed_for_next)
+
+A mixer or feed-forward that sets `accepts_pending` may be handed a `PendingNorm` instead of x: the norm (and the
+residual sum before it) that has not been computed yet, which `project` folds into the part's first product.
 """
 from __future__ import annotations
 
@@ -69,6 +72,71 @@ def as_product_weight(t: torch.Tensor, shared: bool = False):
     return t
 
 
+@dataclasses.dataclass
+class PendingNorm:
+    """Activations that are not computed yet: next_norm(residual + post_norm(y)), or next_norm(residual) if y is
+    None.  A block hands this to a part that says `accepts_pending`, so that the part's first matrix product can do
+    the residual sum and both norms in its own kernel (`project`); any other consumer calls `materialize()`.
+    After either, `residual` is the updated residual stream (possibly another buffer) and `y` is None."""
+
+    residual: torch.Tensor          # float32 [T, D]
+    y: torch.Tensor | None          # [T, D] activations to be normed and added, or None
+    post_norm: "Norm | None"        # applied to y before the sum (None: y is added as it is)
+    next_norm: "Norm | None"        # applied to the sum (None: only the sum is wanted)
+    dtype: torch.dtype
+
+    def settle(self) -> torch.Tensor:
+        """Does the residual sum if it is still pending; returns the updated residual stream."""
+        if self.y is not None:
+            from ..kernels import ops
+
+            if self.post_norm is not None:
+                self.post_norm.add_into(self.residual, self.y, None, self.dtype)
+            else:
+                ops.add_rmsnorm(self.y, self.residual)
+            self.y = None
+        return self.residual
+
+    def materialize(self) -> torch.Tensor:
+        """The activations, computed with the separate kernels."""
+        if self.next_norm is None:
+            raise ValueError("a pending sum without a following norm has no activations")
+        if self.y is not None and self.post_norm is not None:
+            y, self.y = self.y, None
+            return self.post_norm.add_into(self.residual, y, self.next_norm, self.dtype)
+        return self.next_norm.forward(self.settle(), self.dtype)
+
+
+def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x . w^T (gated if w is a paired tiled weight) for activations x or a `PendingNorm`.  A pending norm is done
+    inside the product's kernel when that kernel takes the sizes (bfloat16, up to 16 rows, tiled weight, RMSNorms);
+    otherwise it is materialized first."""
+    from ..kernels import ops
+    from ..kernels.packing import TiledWeight
+
+    if isinstance(x, PendingNorm):
+        pn, nn = x.post_norm, x.next_norm
+        fusable = (x.dtype == torch.bfloat16 and nn is not None and getattr(nn, "fusable_rms", False)
+                   and nn.scale.dtype == torch.bfloat16
+                   and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
+                   and isinstance(w, TiledWeight) and w.rows <= 16 * 2048   # every workgroup redoes the norms
+                   and ops.gemm_normed_takes(x.residual.shape[0], w)
+                   and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
+        if fusable:
+            h_out = torch.empty_like(x.residual) if x.y is not None else None
+            out = ops.gemm_normed(
+                x.y, x.residual, h_out, w,
+                post_weight=pn.scale if (pn is not None and x.y is not None) else None,
+                post_eps=pn.eps if pn is not None else 0.0, post_plus_one=pn.scale_plus_one if pn is not None else True,
+                next_weight=nn.scale, next_eps=nn.eps, next_plus_one=nn.scale_plus_one, soft_cap=soft_cap,
+                out_dtype=out_dtype or x.dtype)
+            if x.y is not None:
+                x.residual, x.y = h_out, None
+            return out
+        x = x.materialize()
+    return ops.gemm(x, w, soft_cap=soft_cap, out_dtype=out_dtype)
+
+
 class Part:
     """Common base: parameter declaration and loading."""
 
@@ -107,6 +175,9 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    #: True if forward() takes a `PendingNorm` in place of x (and consumes it with `project`)
+    accepts_pending = False
+
     def cache_need(self) -> PagedKVNeed | StateNeed | None:
         return None
 
@@ -117,6 +188,9 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    #: True if forward() takes a `PendingNorm` in place of x (and consumes it with `project`)
+    accepts_pending = False
+
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         raise NotImplementedError
 
@@ -134,8 +208,9 @@ class Block(Part):
         compute it together with its last residual sum."""
         return None
 
-    def forward(self, h: torch.Tensor, ctx: Any, cache: Any, normed: torch.Tensor | None,
-                next_norm: Norm | None) -> tuple[torch.Tensor, torch.Tensor | None]:
-        """h: float32 residual stream [T, D], updated in place and returned.  `normed` is
-        first_norm()(h) if the caller has it already.  Returns (h, next_norm(h) or None)."""
+    def forward(self, h: torch.Tensor, ctx: Any, cache: Any, normed: "torch.Tensor | PendingNorm | None",
+                next_norm: Norm | None) -> "tuple[torch.Tensor, torch.Tensor | PendingNorm | None]":
+        """h: float32 residual stream [T, D].  `normed` is first_norm()(h) if the caller has it already, or a
+        `PendingNorm` whose residual sum is still to be done (then h is the stream before that sum).  Returns
+        (h, x) with x = next_norm(h), None, or a `PendingNorm` that carries the block's last sum."""
         raise NotImplementedError

@@ -7,8 +7,10 @@ norm after it where those are RMSNorms.
 """
 from __future__ import annotations
 
+import torch
+
 from ..registry import BLOCKS
-from .base import Block
+from .base import Block, PendingNorm
 
 
 @BLOCKS.register("sandwich")
@@ -26,6 +28,10 @@ class SandwichBlock(Block):
 
     def forward(self, h, ctx, cache, normed, next_norm):
         n = self.norms
+        if ctx.dtype == torch.bfloat16 and ctx.num_tokens <= 16:
+            return self._forward_few_rows(h, ctx, cache, normed, next_norm)
+        if isinstance(normed, PendingNorm):
+            normed, h = normed.materialize(), normed.residual
         if normed is None:
             normed = n["pre_mixer"].forward(h, ctx.dtype)
         y = self.mixer.forward(normed, ctx, cache)
@@ -33,3 +39,22 @@ class SandwichBlock(Block):
         y = self.feed_forward.forward(normed, ctx)
         normed_next = n["post_ffn"].add_into(h, y, next_norm, ctx.dtype)
         return h, normed_next
+
+    def _forward_few_rows(self, h, ctx, cache, normed, next_norm):
+        """The same block for a handful of rows (decoding): every "residual sum, norm" between two parts is handed
+        on as a `PendingNorm`, which the next part's first product computes in its own kernel."""
+        n = self.norms
+
+        def give(part, x):
+            if isinstance(x, PendingNorm) and not part.accepts_pending:
+                return x.materialize()
+            return x
+
+        x = normed if normed is not None else PendingNorm(h, None, None, n["pre_mixer"], ctx.dtype)
+        y = self.mixer.forward(give(self.mixer, x), ctx, cache)
+        if isinstance(x, PendingNorm):
+            h = x.settle()
+        x = PendingNorm(h, y, n["post_mixer"], n["pre_ffn"], ctx.dtype)
+        y = self.feed_forward.forward(give(self.feed_forward, x), ctx)
+        h = x.settle()
+        return h, PendingNorm(h, y, n["post_ffn"], next_norm, ctx.dtype)

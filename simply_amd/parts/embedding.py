@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import ParamSpec, Part, as_product_weight
+from .base import ParamSpec, Part, as_product_weight, project
 
 
 class ScaledEmbedding(Part):
@@ -44,8 +44,8 @@ class LinearHead(Part):
         self.weight = as_product_weight(tensors["weight"], shared=True)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """x [R, D] activations -> float32 logits [R, V]."""
-        return ops.gemm(x, self.weight, soft_cap=self.soft_cap, out_dtype=torch.float32)
+        """x [R, D] activations (or a `PendingNorm` of them) -> float32 logits [R, V]."""
+        return project(x, self.weight, soft_cap=self.soft_cap, out_dtype=torch.float32)
 
 
 EMBEDDINGS = {"scaled_embedding": ScaledEmbedding}

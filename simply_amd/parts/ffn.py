@@ -6,7 +6,7 @@ import torch
 
 from ..kernels import ops
 from ..registry import ACTIVATIONS, FEED_FORWARDS
-from .base import FeedForward, ParamSpec, as_product_weight
+from .base import FeedForward, ParamSpec, PendingNorm, as_product_weight, project
 
 # activation name -> epilogue of the fused gate/up product
 ACTIVATIONS.register("gelu_tanh", ops.EPILOGUE_GATED_GELU)
@@ -14,6 +14,8 @@ ACTIVATIONS.register("gelu_tanh", ops.EPILOGUE_GATED_GELU)
 
 @FEED_FORWARDS.register("gated_dense")
 class GatedDense(FeedForward):
+    accepts_pending = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh"):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         if ACTIVATIONS.get(activation) != ops.EPILOGUE_GATED_GELU:
@@ -38,5 +40,10 @@ class GatedDense(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         # gelu(x.Wg^T) * (x.Wu^T), one kernel
-        z = ops.gemm(x, self.gate_up) if self.gate_up is not None else ops.gemm(x, self.gate_proj, w2=self.up_proj)
+        if self.gate_up is not None:
+            z = project(x, self.gate_up)
+        else:
+            if isinstance(x, PendingNorm):
+                x = x.materialize()
+            z = ops.gemm(x, self.gate_proj, w2=self.up_proj)
         return ops.gemm(z, self.down_proj)

@@ -11,6 +11,9 @@ from .base import Norm, ParamSpec
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    #: the fused norm-and-product kernel computes exactly this norm from (scale, eps, scale_plus_one)
+    fusable_rms = True
+
     def __init__(self, dim: int, eps: float, scale_plus_one: bool = True):
         self.dim = int(dim)
         self.eps = float(eps)

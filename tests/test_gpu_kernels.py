@@ -412,3 +412,40 @@ def test_sampling_rows_at_odd_addresses():
     torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
     for r in (0, 2, 4):
         assert tok[r].item() == int(logits[r].argmax())
+
+
+@pytest.mark.parametrize("M", [1, 8, 13, 16])
+@pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (4608, 64), (96, 40), (72, 64)])
+def test_gemm_normed(M, K, N):
+    """Residual sum, two norms and the product in one kernel against the separate references."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles
+    y, h = rand((M, K), torch.bfloat16, 100, 2.0), rand((M, K), torch.float32, 101, 4.0)
+    wp, wn = rand((K,), torch.bfloat16, 102, 0.3), rand((K,), torch.bfloat16, 103, 0.3)
+    w, w2 = rand((N, K), torch.bfloat16, 104, 0.05), rand((N, K), torch.bfloat16, 105, 0.05)
+    tw, tg = pack_tiles(w), pack_gate_up(w, w2)
+    fits = (8 if M <= 8 else 16) * (K + 8) * 2 + 8 * 2 * 16 * 17 * 4 <= 160 * 1024   # activations and tiles in LDS
+    assert ops.gemm_normed_takes(M, tw) == (fits and K % 32 == 0 and K <= 2560)
+    if not ops.gemm_normed_takes(M, tw):
+        return
+    kw = dict(post_weight=wp, post_eps=1e-6, post_plus_one=True, next_weight=wn, next_eps=1e-5, next_plus_one=True)
+    t = dict(rtol=2e-2, atol=2e-2)
+    for with_y in (True, False):
+        h_ref = h.clone()
+        a_ref = ref.add_rmsnorm(y, h_ref, post_weight=wp, post_eps=1e-6, next_weight=wn, next_eps=1e-5,
+                                out_dtype=torch.bfloat16) if with_y else ref.rmsnorm(h, wn, 1e-5, True, torch.bfloat16)
+        h_out = torch.full_like(h, 7.0)
+        got = ops.gemm_normed(y if with_y else None, h, h_out if with_y else None, tw, **kw)
+        torch.testing.assert_close(got.float(), ref.gemm(a_ref, w).float(), **t)
+        if with_y:
+            torch.testing.assert_close(h_out, h_ref, rtol=1e-5, atol=1e-5)
+        got = ops.gemm_normed(y if with_y else None, h, h_out if with_y else None, tg, **kw)
+        torch.testing.assert_close(got.float(), ref.gemm(a_ref, w, w2=w2).float(), **t)
+        got = ops.gemm_normed(y if with_y else None, h, h_out if with_y else None, tw, soft_cap=3.0,
+                              out_dtype=torch.float32, **kw)
+        torch.testing.assert_close(got, ref.gemm(a_ref, w, soft_cap=3.0, out_dtype=torch.float32), rtol=5e-3, atol=5e-3)
+    # without a post-norm the residual takes y as it is
+    h_out = torch.empty_like(h)
+    ops.gemm_normed(y, h, h_out, tw, **dict(kw, post_weight=None))
+    torch.testing.assert_close(h_out, h + y.float(), rtol=1e-6, atol=1e-6)
+    assert not ops.gemm_normed_takes(17, tw) and not ops.gemm_normed_takes(M, w)
