@@ -89,6 +89,16 @@ int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pag
                               int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                               void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
+// The same for portions of prompts: the units (rows of seq_meta, each with (query heads per key head) * tokens <= 16)
+// unit_begin .. unit_begin + unit_count - 1 are taken four at a time by one workgroup, which reads the keys once for
+// all of them.  unit_count is a multiple of 4 and the four units of a workgroup belong to one request; units with
+// no tokens fill up a request's last four.
+int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                               const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
+                               int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
+                               int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
+                               void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
 // One token per row of 32-bit logits.  temperature 0 or top_k 1: argmax.  top_k <= 0 and top_p >= 1: off.
 int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature, const int* top_k,
               const float* top_p, const uint64_t* seed, const int* counter, int* tokens, float* logprobs,
@@ -110,6 +120,13 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
                            hipStream_t stream);
+bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q,
+                                   int64_t out_stride, const void* out);
+int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                            const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
+                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
+                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
+                            hipStream_t stream);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
                int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream);

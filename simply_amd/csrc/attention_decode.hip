@@ -17,30 +17,15 @@
 // kernel from a workspace, in a fixed order (a merge by the workgroup that finishes last would need a
 // device-wide fence, which on this GPU writes back the whole L2).
 #include "api.h"
-#include "common.h"
+#include "attention_common.h"
 
 namespace sa {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) float floatx4;
-
-constexpr int kTile = 32;  // keys per MFMA tile
 
 __device__ inline float fast_tanh(float x) {
   // tanh(x) = 1 - 2 / (exp(2x) + 1); exact at both ends, relative error ~1e-6 in between
   const float e = __expf(2.f * x);
   return 1.f - 2.f / (e + 1.f);
 }
-
-__device__ inline __bf16 to_bf16_raw(float f) {
-  const bf16 b = float_to_bf16(f);
-  return __builtin_bit_cast(__bf16, b.bits);
-}
-
-struct SeqMeta {
-  int slot, q_start, q_len, pos0;
-};
 
 // NDC = head size / 32
 template <int NDC>
@@ -287,7 +272,6 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 
 // Adds up the key ranges of each (request, head, row), in their order: one workgroup per row, one thread per
 // output dimension; the ranges' weights exp(m_y - max) are computed once into LDS.
-constexpr int kMaxSplits = 256;
 __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ workspace, int KS, int HD,
                                                                     const SeqMeta* __restrict__ seq_meta, int seq_begin,
                                                                     bf16* __restrict__ out, int64_t out_stride, int Kh,
@@ -369,12 +353,15 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   }
 #undef SA_LAUNCH
   if (check_launch("paged_attention_decode")) return 1;
-  if (KS > 1) {
-    paged_attention_merge_kernel<<<dim3(Kh, seq_count, 16), 256, 0, stream>>>(ws, KS, hd, sm, seq_begin, op, out_stride,
-                                                                             Kh, G);
-    return check_launch("paged_attention_merge");
-  }
+  if (KS > 1) return attention_merge_ranges(ws, KS, hd, sm, seq_begin, seq_count, op, out_stride, Kh, G, stream);
   return 0;
+}
+
+int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
+                           int unit_count, bf16* out, int64_t out_stride, int Kh, int G, hipStream_t stream) {
+  paged_attention_merge_kernel<<<dim3(Kh, unit_count, 16), 256, 0, stream>>>(workspace, num_ranges, hd, units, unit_begin,
+                                                                            out, out_stride, Kh, G);
+  return check_launch("paged_attention_merge");
 }
 
 }  // namespace sa

@@ -22,8 +22,11 @@ __host__ __device__ inline float to_float(bf16 x) {
 }
 __host__ __device__ inline float to_float(float x) { return x; }
 
-// Round to nearest even; NaN stays NaN.
+// Round to nearest even; NaN stays NaN.  On the device this is gfx950's own conversion instruction.
 __host__ __device__ inline bf16 float_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_bit_cast(bf16, static_cast<__bf16>(f));
+#endif
   union { uint32_t u; float f; } c;
   c.f = f;
   uint32_t u = c.u;

@@ -99,3 +99,24 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
                                 out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len, num_splits,
                                 workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
 }
+
+extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                          const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
+                                          int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd,
+                                          int page_size, int window, float soft_cap, int max_kv_len, int max_q_len,
+                                          int num_splits, void* workspace, int64_t workspace_bytes,
+                                          hipStream_t stream) {
+  if (unit_count == 0) return 0;
+  SA_REQUIRE(unit_count > 0 && unit_count % 4 == 0 && unit_begin >= 0 && H > 0 && Kh > 0 && H % Kh == 0,
+             "paged_attention_prefill: bad counts (units come in fours)");
+  SA_REQUIRE(window >= 0 && table_stride > 0 && max_kv_len > 0, "paged_attention_prefill: bad window, table or length");
+  SA_REQUIRE(paged_attention_prefill_takes(H, Kh, hd, page_size, max_q_len, q_stride, q, out_stride, out),
+             "paged_attention_prefill takes head size 64, 128 or 256, a page size that is a multiple of 16 and "
+             "(heads per key head) * tokens <= 16 per unit; got hd=%d P=%d G=%d tokens=%d", hd, page_size, H / Kh,
+             max_q_len);
+  SA_REQUIRE(out_stride >= static_cast<int64_t>(H) * hd, "paged_attention_prefill: output rows are too short");
+  return paged_attention_prefill(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, unit_begin,
+                                 unit_count, out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len,
+                                 num_splits, workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes),
+                                 stream);
+}

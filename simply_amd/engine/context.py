@@ -56,20 +56,29 @@ class StepContext:
             n += 1
         return n, self.cu_q_lens[n]
 
-    def attention_units(self, tokens_per_unit: int) -> tuple[torch.Tensor, int, int]:
+    def attention_units(self, tokens_per_unit: int, group: int = 1) -> tuple[torch.Tensor, int, int, int]:
         """The step's tokens cut into units of at most `tokens_per_unit` consecutive tokens of one request, in
         the layout of `seq_meta` (slot, first token, tokens, first position): what an attention kernel that takes
-        few query rows at a time is launched over.  Returns (units int32 [U, 4] on the device, U, most tokens
-        in a unit).  If no request has more tokens than that, the units are the requests themselves."""
+        few query rows at a time is launched over.  Requests that fit into one unit come first, one unit each;
+        then the units of the longer requests, each request's units filled up with empty ones to a multiple of
+        `group`, so that a kernel that takes `group` units at a time never mixes requests.  Returns (units
+        int32 [U, 4] on the device, number of one-unit requests, number of units after them, most tokens in a
+        unit)."""
         if self.max_q_len <= tokens_per_unit:
-            return self.seq_meta, self.num_seqs, self.max_q_len
-        cached = self._units.get(tokens_per_unit)
+            return self.seq_meta, self.num_seqs, 0, self.max_q_len
+        key = (tokens_per_unit, group)
+        cached = self._units.get(key)
         if cached is None:
-            rows = []
+            few, many = [], []
             for slot, first, start, q in zip(self.seq_slots, self.cu_q_lens, self.seq_starts, self.q_lens):
+                if q <= tokens_per_unit:
+                    few.append((slot, first, q, start))
+                    continue
                 for o in range(0, q, tokens_per_unit):
-                    rows.append((slot, first + o, min(tokens_per_unit, q - o), start + o))
-            units = torch.tensor(rows, dtype=torch.int32).to(self.positions.device, non_blocking=True)
-            cached = (units, len(rows), tokens_per_unit)
-            self._units[tokens_per_unit] = cached
+                    many.append((slot, first + o, min(tokens_per_unit, q - o), start + o))
+                while len(many) % group:
+                    many.append((slot, first + q, 0, start + q))
+            units = torch.tensor(few + many, dtype=torch.int32).to(self.positions.device, non_blocking=True)
+            cached = (units, len(few), len(many), tokens_per_unit)
+            self._units[key] = cached
         return cached

@@ -34,6 +34,8 @@ _SIGNATURES = {
     "sa_paged_attention": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "sa_paged_attention_decode": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L,
                                   _P],
+    "sa_paged_attention_prefill": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L,
+                                   _P],
     "sa_gemm_normed": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _I, _I, _F, _P],
     "sa_gemm_normed_takes": [_I, _I, _I],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P],

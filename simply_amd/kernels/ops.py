@@ -350,32 +350,56 @@ def decode_attention_takes(q: torch.Tensor, k_pages: torch.Tensor, num_heads: in
             and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
 
 
+def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, begin, count, num_heads, window, soft_cap,
+                     max_kv_len, max_q_len, out, num_splits):
+    _dev(q, k_pages, v_pages, block_table, seq_meta, out)
+    name = entry[3:]
+    if q.dtype != torch.bfloat16:
+        raise KernelError(f"{name}: bfloat16 only")
+    q_stride = _rows(q, f"{name}: q")
+    _check_pages(k_pages, v_pages, q.dtype, name)
+    _, Kh, page_size, hd = k_pages.shape
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError(f"{name}: block_table must be int32 [sequences, blocks]")
+    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
+            or begin < 0 or begin + count > seq_meta.shape[0]:
+        raise KernelError(f"{name}: seq_meta must be int32 [S, 4] covering the requested range")
+    if out.dtype != q.dtype or out.shape[0] != q.shape[0] or out.shape[1] != num_heads * hd:
+        raise KernelError(f"{name}: bad output")
+    out_stride = _rows(out, f"{name}: out")
+    ws = _workspace(q.device)
+    _lib.call(entry, _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+              block_table.stride(0), _ptr(seq_meta), begin, count, _ptr(out), out_stride, num_heads, Kh, hd,
+              page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
+              _ptr(ws), ws.numel(), _stream())
+    return out
+
+
 def paged_attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                            seq_meta: torch.Tensor, seq_begin: int, seq_count: int, num_heads: int, *,
                            window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
                            out: torch.Tensor, num_splits: int = 0) -> torch.Tensor:
     """Attention of requests seq_begin .. seq_begin + seq_count - 1 of seq_meta, each with few tokens
     ((heads per key head) * tokens <= 16).  q and out are the whole step's rows."""
-    _dev(q, k_pages, v_pages, block_table, seq_meta, out)
-    if q.dtype != torch.bfloat16:
-        raise KernelError("paged_attention_decode: bfloat16 only")
-    q_stride = _rows(q, "paged_attention_decode: q")
-    _check_pages(k_pages, v_pages, q.dtype, "paged_attention_decode")
-    _, Kh, page_size, hd = k_pages.shape
-    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
-        raise KernelError("paged_attention_decode: block_table must be int32 [sequences, blocks]")
-    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
-            or seq_begin < 0 or seq_begin + seq_count > seq_meta.shape[0]:
-        raise KernelError("paged_attention_decode: seq_meta must be int32 [S, 4] covering the requested range")
-    if out.dtype != q.dtype or out.shape[0] != q.shape[0] or out.shape[1] != num_heads * hd:
-        raise KernelError("paged_attention_decode: bad output")
-    out_stride = _rows(out, "paged_attention_decode: out")
-    ws = _workspace(q.device)
-    _lib.call("sa_paged_attention_decode", _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
-              block_table.stride(0), _ptr(seq_meta), seq_begin, seq_count, _ptr(out), out_stride, num_heads, Kh, hd,
-              page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
-              _ptr(ws), ws.numel(), _stream())
-    return out
+    return _attention_units("sa_paged_attention_decode", q, k_pages, v_pages, block_table, seq_meta, seq_begin,
+                            seq_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
+
+
+PREFILL_UNITS_PER_GROUP = 4
+
+
+def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                            units: torch.Tensor, unit_begin: int, unit_count: int, num_heads: int, *,
+                            window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
+                            out: torch.Tensor, num_splits: int = 0) -> torch.Tensor:
+    """Attention of portions of prompts cut into units of few tokens ((heads per key head) * tokens <= 16), rows
+    unit_begin .. unit_begin + unit_count - 1 of `units` in the layout of seq_meta.  One workgroup takes four
+    consecutive units, which must belong to one request (units without tokens fill up the last four), and
+    reads the keys once for all of them."""
+    if unit_count % PREFILL_UNITS_PER_GROUP:
+        raise KernelError("paged_attention_prefill: units come in fours")
+    return _attention_units("sa_paged_attention_prefill", q, k_pages, v_pages, block_table, units, unit_begin,
+                            unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
 
 
 # --------------------------------------------------------------------------- sampling

@@ -72,12 +72,16 @@ class PagedAttention(Mixer):
                                  k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
         o = torch.empty((qkv.shape[0], H * hd), dtype=qkv.dtype, device=qkv.device)
         if ops.decode_attention_takes(qkv, cache.k_pages, H, 1):
-            # the MFMA kernel takes up to 16 query rows (tokens x heads per key head) at a time: decoding requests
-            # are one unit each, portions of prompts are cut into units of 16 / G tokens
-            units, num_units, max_q = ctx.attention_units(16 // (H // K))
-            ops.paged_attention_decode(qkv, cache.k_pages, cache.v_pages, group.block_table, units, 0, num_units, H,
-                                       window=self.window, soft_cap=self.soft_cap, max_kv_len=ctx.max_kv_len,
-                                       max_q_len=max_q, out=o)
+            # the MFMA kernels take up to 16 query rows (tokens x heads per key head) as a unit: a decoding request
+            # is one unit and its keys are cut over workgroups; portions of prompts are cut into units of 16 / G
+            # tokens, of which one workgroup takes four
+            units, few, many, max_q = ctx.attention_units(16 // (H // K), ops.PREFILL_UNITS_PER_GROUP)
+            kw = dict(window=self.window, soft_cap=self.soft_cap, max_kv_len=ctx.max_kv_len, max_q_len=max_q, out=o)
+            if few:
+                ops.paged_attention_decode(qkv, cache.k_pages, cache.v_pages, group.block_table, units, 0, few, H, **kw)
+            if many:
+                ops.paged_attention_prefill(qkv, cache.k_pages, cache.v_pages, group.block_table, units, few, many, H,
+                                            **kw)
         else:
             ops.paged_attention(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions, H,
                                 window=self.window, soft_cap=self.soft_cap, out=o)

@@ -449,3 +449,104 @@ def test_gemm_normed(M, K, N):
     ops.gemm_normed(y, h, h_out, tw, **dict(kw, post_weight=None))
     torch.testing.assert_close(h_out, h + y.float(), rtol=1e-6, atol=1e-6)
     assert not ops.gemm_normed_takes(17, tw) and not ops.gemm_normed_takes(M, w)
+
+
+def prefill_units(lens, q_lens, per_unit):
+    """Units of at most per_unit tokens of requests whose last q tokens are this step's, each request's units
+    filled up to a multiple of four: what the host hands to the prompt-portion kernel."""
+    units, t0 = [], 0
+    for s, (l, q) in enumerate(zip(lens, q_lens)):
+        for o in range(0, q, per_unit):
+            units.append((s, t0 + o, min(per_unit, q - o), l - q + o))
+        while len(units) % 4:
+            units.append((s, t0 + q, 0, l))
+        t0 += q
+    return torch.tensor(units, dtype=torch.int32).cuda()
+
+
+@pytest.mark.parametrize("H,Kh,hd,P,window,cap", [
+    (8, 4, 256, 16, None, 50.0), (8, 4, 256, 16, 100, 50.0), (4, 2, 64, 16, 33, None), (16, 1, 128, 32, None, 30.0),
+    (2, 2, 128, 64, 200, None), (6, 3, 64, 16, 1, 20.0), (6, 2, 128, 16, 40, 50.0), (5, 1, 64, 48, None, None)])
+@pytest.mark.parametrize("splits", [0, 1, 3])
+def test_paged_attention_prefill(H, Kh, hd, P, window, cap, splits):
+    """The prompt-portion bfloat16 kernel against the plain reference: portions that start at 0 and after a
+    history, with lengths around unit, tile and page edges, unwritten page tails holding NaN, keys also cut
+    over workgroups."""
+    from simply_amd.kernels import ops
+    G = H // Kh
+    per_unit = 16 // G
+    lens = [300, 77, 1000, 64, 129, 5]
+    q_lens = [300, 40, 130, 64, 2, 5]
+    kp, vp, table = paged_setup(torch.bfloat16, len(lens), H, Kh, hd, P, lens, 71)
+    _, ts, ps = seq_meta_for(lens, q_lens)
+    units = prefill_units(lens, q_lens, per_unit)
+    T = ts.numel()
+    q = rand((T, (H + 2 * Kh) * hd), torch.bfloat16, 72, 0.3)
+    out = torch.zeros((T, H * hd), dtype=torch.bfloat16).cuda()
+    ops.paged_attention_prefill(q, kp, vp, table, units, 0, units.shape[0], H, window=window, soft_cap=cap,
+                                max_kv_len=max(lens), max_q_len=per_unit, out=out, num_splits=splits)
+    want = ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap)
+    assert torch.isfinite(out.float()).all()
+    torch.testing.assert_close(out.float(), want.float(), rtol=2e-2, atol=2e-2)
+    # the few-rows kernel on the same units gives the same up to rounding
+    out2 = torch.zeros_like(out)
+    ops.paged_attention_decode(q, kp, vp, table, units, 0, units.shape[0], H, window=window, soft_cap=cap,
+                               max_kv_len=max(lens), max_q_len=per_unit, out=out2)
+    torch.testing.assert_close(out.float(), out2.float(), rtol=2e-2, atol=2e-2)
+    # a sub-range of the units: the other rows stay untouched
+    first = next(i for i in range(units.shape[0]) if int(units[i, 0]) == 2)
+    count = sum(1 for i in range(units.shape[0]) if int(units[i, 0]) == 2)
+    out3 = torch.full_like(out, 7.0)
+    ops.paged_attention_prefill(q, kp, vp, table, units, first, count, H, window=window, soft_cap=cap,
+                                max_kv_len=max(lens), max_q_len=per_unit, out=out3, num_splits=splits)
+    a, b = sum(q_lens[:2]), sum(q_lens[:3])
+    torch.testing.assert_close(out3[a:b].float(), out[a:b].float(), rtol=2e-2, atol=2e-2)
+    assert (out3[:a] == 7).all() and (out3[b:] == 7).all()
+    with pytest.raises(Exception, match="fours"):
+        ops.paged_attention_prefill(q, kp, vp, table, units, 0, 3, H, window=window, soft_cap=cap,
+                                    max_kv_len=max(lens), max_q_len=per_unit, out=out3)
+
+
+def test_paged_attention_prefill_far_key_and_window_edge():
+    """Every query row of a long portion must find one key far back whose score stands out, and a windowed
+    layer must see it exactly while it is inside each row's own window."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
+    H, Kh, hd, P, L, Q = 2, 1, 128, 16, 2500, 600
+    kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 73)
+    kp = keys_to_rows(kp) * 0.01
+    far = 1871
+    page, off = int(table[0, far // P]), far % P
+    kp[page, 0, off] = 0.0
+    kp[page, 0, off, 5] = 60.0
+    kp = rows_to_keys(kp)
+    vp[page, 0, :, off] = 3.0
+    units = prefill_units([L], [Q], 8)
+    q = torch.zeros((Q, 4 * hd), dtype=torch.bfloat16).cuda()
+    q[:, 5] = 1.0
+    q[:, hd + 5] = 1.0
+    positions = torch.arange(L - Q, L)
+    for window in (None, 300):
+        out = torch.zeros((Q, H * hd), dtype=torch.bfloat16).cuda()
+        ops.paged_attention_prefill(q, kp, vp, table, units, 0, units.shape[0], H, window=window, soft_cap=None,
+                                    max_kv_len=L, max_q_len=8, out=out)
+        found = (out.float().mean(dim=1) - 3.0).abs().cpu() < 0.05
+        sees = (positions >= far) & ((positions - far < window) if window else torch.ones_like(positions, dtype=torch.bool))
+        assert torch.equal(found, sees), (window, (found != sees).nonzero().flatten().tolist()[:10])
+
+
+def test_bfloat16_rounding_of_the_kernels():
+    """The device's conversion to bfloat16 rounds to nearest even, as torch does: all exponents, ties, subnormals."""
+    from simply_amd.kernels import ops
+    g = torch.Generator().manual_seed(5)
+    bits = torch.randint(-2**31, 2**31 - 1, (64, 4096), generator=g, dtype=torch.int64).to(torch.int32)
+    bits[0, :2048] = (torch.arange(2048, dtype=torch.int32) << 16) | 0x8000          # exact ties, even and odd
+    bits[1, :2048] = (torch.arange(2048, dtype=torch.int32) << 16) | 0x7fff
+    bits[2, :2048] = (torch.arange(2048, dtype=torch.int32) << 16) | 0x8001
+    x = bits.view(torch.float32).cuda()
+    idx = torch.arange(64, dtype=torch.int32).cuda()
+    got = ops.gather_rows(x, idx, out_dtype=torch.bfloat16)
+    want = x.to(torch.bfloat16)
+    nan = torch.isnan(x)
+    assert torch.equal(torch.isnan(got.float()), nan)
+    assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan])
