@@ -1,54 +1,80 @@
 // Paged attention in bfloat16 for portions of prompts: many query tokens of one request over the keys that the
 // request has so far.  Bound by the matrix cores and the softmax arithmetic, no longer by reading the keys: a
-// workgroup of four waves takes 4 consecutive units of up to 16 query rows each (rows = tokens x query heads of
-// one key/value head; the host cuts a request's tokens into such units) and one key/value head, and walks over the
-// keys once for all 64 rows.  Each tile of 32 keys and its values go through LDS:
+// workgroup of four waves takes 4 * R consecutive units of up to 16 query rows each (rows = tokens x query heads of
+// one key/value head; the host cuts a request's tokens into such units) and one key/value head, and walks over
+// the keys once for all of its rows.
 //
-//     global -> registers         issued one tile ahead, while the current tile is computed
-//     registers -> LDS            keys stay in their 16-key x 32-dimension blocks of MFMA operand order (a plain
-//                                 copy); values, stored [hd, page_size] in their pages, are re-ordered into operand
-//                                 blocks of 16 dimensions x 32 keys on the way
-//     LDS -> MFMA                 every wave reads every block with one 16-byte read per lane and computes, for
-//                                 its own 16 rows, S^T = K . Q^T, the soft-cap, mask and online softmax in float32,
-//                                 and O^T += V^T . P^T, exactly as the few-rows kernel does
+// Keys and values go from the pages straight into LDS (global_load_lds: no staging registers), into two buffers
+// of one 32-key tile each, so that the loads of the next tile are in flight while one tile is computed; two
+// workgroups fit on a compute unit and fill each other's waits.  Both lie in LDS as they lie in their pages: keys in 16-key x 32-dimension blocks of MFMA operand
+// order, values per 16-key sub-tile as blocks of 16 dimensions, [keys 0..7 | keys 8..15][dimension][8 keys].  Every wave reads every block of a tile and computes,
+// for its own rows,
+//     S^T = K . Q^T            keys as the A operand, one 16-byte LDS read per lane and block
+//     soft-cap, mask and online softmax in float32 (base-2 exponentials, log2(e) folded into the constants)
+//     O^T += V^T . P^T         S^T comes out of the first product in the layout that the second wants for P^T;
+//                              the value operand is two 8-byte LDS reads per lane, one from each sub-tile
+// exactly as the few-rows kernel does from global memory.  A wave with R units keeps R tiles of rows and uses each
+// operand it reads for all of them.  A wave skips tiles that none of its rows can see and the mask arithmetic on
+// tiles that all of its rows see whole.
 //
-// A wave skips tiles that none of its rows can see, and the mask arithmetic on tiles that all of its rows see
-// whole.  The exponentials are taken to base 2 with log2(e) folded into the constants.  When few workgroups would
-// result (a short portion over a long context), the keys are also cut into ranges over workgroups, and the ranges
-// are merged by the second kernel of the few-rows path.
+// The two buffers are kept in step by one workgroup barrier per tile.  The barrier is the bare instruction, with the
+// count of outstanding loads given by hand: the usual barrier with its fence would wait for all loads in flight,
+// which is the pipeline.  Each buffer is an array of its own so that the compiler can tell a read of one buffer
+// from the loads in flight into the others.
+//
+// When few workgroups would result (a short portion over a long context), the keys are also cut into ranges over
+// workgroups, and the ranges are merged by the second kernel of the few-rows path.
 #include "api.h"
 #include "attention_common.h"
 
 namespace sa {
 namespace prefill {
 
-constexpr int kUnitsPerGroup = 4;  // waves of a workgroup, each with a unit of up to 16 rows
+constexpr int kWaves = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 
-template <int NDC>
+// s_waitcnt for "at most n vector-memory loads outstanding" and nothing else (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8)
+constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+// The workgroup barrier alone; the empty statements keep the compiler from moving memory accesses across it.
+__device__ inline void bare_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// 16 bytes per lane from global memory into LDS at dst + 16 * lane (dst is the same for the whole wave).  In a
+// function of its own: written into the kernel's body, the host pass of the compiler drops the kernel's stub.
+__device__ __forceinline__ void load_to_lds(const bf16* src, __bf16* dst) {
+  __builtin_amdgcn_global_load_lds(src, dst, 16, 0, 0);
+}
+
+template <int NDC, int R>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
     float* __restrict__ workspace) {
   constexpr int HD = NDC * 32;
-  constexpr int NDB = HD / 16;          // output blocks of 16 dimensions
-  constexpr int PPT = NDC / 2;          // 16-byte pieces of keys (and of values) per thread and tile
-  constexpr int SUB = NDC * 64;         // pieces in a sub-tile of 16 keys
+  constexpr int NDB = HD / 16;            // output blocks of 16 dimensions
+  constexpr int CPW = NDC / 2;            // KiB chunks of keys (and of values) per wave and tile
+  constexpr int HALF = NDC * 1024;        // elements of a tile's keys (and of its values) in a buffer: 2 * NDC KiB
+  constexpr int GROUP = kWaves * R;       // units per workgroup
   static_assert(NDC % 2 == 0, "head size must be a multiple of 64");
-  __shared__ __attribute__((aligned(16))) __bf16 k_s[2 * NDC * 512];  // [sub-tile][dc][lane][8]
-  __shared__ __attribute__((aligned(16))) __bf16 v_s[NDB * 512];      // [db][lane][8]: 16 dimensions x 32 keys
+  // [keys: sub-tile, dc, lane, 8][values: sub-tile, d, 16]
+  __shared__ __attribute__((aligned(16))) __bf16 stage0[2 * HALF];
+  __shared__ __attribute__((aligned(16))) __bf16 stage1[2 * HALF];
 
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int r = lane % 16, grp = lane / 16;
   const int split = blockIdx.x, num_splits = gridDim.x, kh = blockIdx.y;
-  const int u0 = unit_begin + blockIdx.z * kUnitsPerGroup;
+  const int u0 = unit_begin + blockIdx.z * GROUP;
 
   // the keys that some row of the workgroup sees: [lo_g, hi_g)
   int lo_g = 0x7fffffff, hi_g = 0, slot = 0;
-#pragma unroll
-  for (int w = 0; w < kUnitsPerGroup; ++w) {
+  for (int w = 0; w < GROUP; ++w) {
     const SeqMeta m = units[u0 + w];
     if (m.q_len > 0) {
       const int lo_w = (window > 0 && m.pos0 - window + 1 > 0) ? m.pos0 - window + 1 : 0;
@@ -58,190 +84,272 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     }
   }
   if (hi_g == 0) return;  // no rows at all (uniform over the workgroup)
-  const int* table = block_table + static_cast<size_t>(slot) * table_stride;
+  const int* table = block_table + static_cast<size_t>(__builtin_amdgcn_readfirstlane(slot)) * table_stride;
   const int tile0 = lo_g / kTile, tile1 = (hi_g + kTile - 1) / kTile;
   const int ntiles = tile1 - tile0;
   const int tb = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * split / num_splits);
   const int te = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * (split + 1) / num_splits);
 
-  // this wave's unit and this lane's row of it: query token qi, query head g of the group
-  const SeqMeta sm = units[u0 + wave];
-  const int rows = G * sm.q_len;  // <= 16
+  // this wave's R units and this lane's row of each: query token qi, query head g of the group
   const int qi = r / G, g = r % G;
-  const bool row_ok = r < rows;
-  const int pos_r = sm.pos0 + qi;
-  const int lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
-  // over the wave's rows: positions [pos_first, pos_last], lower bounds [lo_first, lo_last]
-  const int pos_first = sm.pos0, pos_last = sm.pos0 + sm.q_len - 1;
-  const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
-  const int lo_last = (window > 0 && pos_last - window + 1 > 0) ? pos_last - window + 1 : 0;
-
-  // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
-  bf16x8 qf[NDC];
-  {
-    const bf16* qp = q + static_cast<size_t>(sm.q_start + (row_ok ? qi : 0)) * q_stride +
-                     static_cast<size_t>(kh * G + (row_ok ? g : 0)) * HD + grp * 8;
+  int rows[R], pos_r[R], lo_r[R], pos_first[R], pos_last[R], lo_first[R], lo_last[R], q_row[R];
+  bool row_ok[R];
+  bf16x8 qf[R][NDC];  // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
 #pragma unroll
-    for (int dc = 0; dc < NDC; ++dc) qf[dc] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + dc * 32) : bf16x8{};
+  for (int j = 0; j < R; ++j) {
+    const SeqMeta sm = units[u0 + wave * R + j];
+    rows[j] = G * sm.q_len;  // <= 16
+    row_ok[j] = r < rows[j];
+    pos_r[j] = sm.pos0 + qi;
+    lo_r[j] = (window > 0 && pos_r[j] - window + 1 > 0) ? pos_r[j] - window + 1 : 0;
+    // over the unit's rows: positions [pos_first, pos_last], lower bounds [lo_first, lo_last]
+    pos_first[j] = sm.pos0;
+    pos_last[j] = sm.pos0 + sm.q_len - 1;
+    lo_first[j] = (window > 0 && pos_first[j] - window + 1 > 0) ? pos_first[j] - window + 1 : 0;
+    lo_last[j] = (window > 0 && pos_last[j] - window + 1 > 0) ? pos_last[j] - window + 1 : 0;
+    q_row[j] = sm.q_start + qi;
+    const bf16* qp = q + static_cast<size_t>(row_ok[j] ? q_row[j] : sm.q_start) * q_stride +
+                     static_cast<size_t>(kh * G + (row_ok[j] ? g : 0)) * HD + grp * 8;
+#pragma unroll
+    for (int dc = 0; dc < NDC; ++dc)
+      qf[j][dc] = (row_ok[j] && tb < te) ? *reinterpret_cast<const bf16x8*>(qp + dc * 32) : bf16x8{};
   }
 
-  floatx4 acc[NDB];
+  floatx4 acc[R][NDB];
+  float m_run[R], l_run[R];  // per row, in units of log2; l_run is this lane group's share
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;  // per row, in units of log2; l_run is this lane group's share
+  for (int j = 0; j < R; ++j) {
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) acc[j][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+    m_run[j] = -INFINITY;
+    l_run[j] = 0.f;
+  }
 
   // scores in base-2 units: y = log2(e) * cap * tanh(s / cap) = c2 - 2 * c2 / (2^(s * c1) + 1), or log2(e) * s
   const float c1 = soft_cap > 0.f ? 2.f * kLog2e / soft_cap : kLog2e;
   const float c2 = soft_cap * kLog2e;
 
-  bf16x8 kreg[PPT], vreg[PPT];
-  const bf16x8 zero8 = {};
-  // global -> registers: piece p of the tile is 16 bytes of sub-tile p / SUB; of the keys it is piece p % SUB of
-  // the sub-tile's contiguous blocks, of the values it is keys 8h .. 8h+7 of dimension d (p % SUB = 2 * d + h)
-  auto fetch = [&](int tile) {
+  // Chunk c = wave + 4 * i of a tile's keys is the KiB (sub-tile t = c / NDC, dimensions 32 * (c % NDC) ..): 64 lanes
+  // x 16 bytes, contiguous in the page and in LDS.  Chunk c of its values is dimensions 32 * (c % NDC) .. + 31 of
+  // sub-tile t, 32 bytes (16 keys) each: a lane takes 8 keys of one dimension.  A wave's chunks lie in at most
+  // NT sub-tiles (one if the head has 64 dimensions, else both); what depends on the lane is computed once.
+  constexpr int NT = CPW < 2 ? 1 : 2;      // sub-tiles this wave reads from
+  constexpr int CPT = CPW / NT;            // chunks per sub-tile
+  uint32_t k_off[CPW], v_off[CPW], lds_off[CPW];  // in elements
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-      const int p = i * 256 + tid;
-      const int t = p / SUB, w = p % SUB;
-      const int sk0 = tile * kTile + t * 16;
-      const bool ok = sk0 < hi_g && sk0 + 16 > lo_g;
-      kreg[i] = zero8;
-      vreg[i] = zero8;
-      if (ok) {
-        const int page = table[sk0 / page_size];
-        const int off = sk0 % page_size;  // a multiple of 16
-        const size_t head = static_cast<size_t>(page) * Kh + kh;
-        const int d = w / 2, h = w % 2;
-        kreg[i] = *reinterpret_cast<const bf16x8*>(k_pages + head * page_size * HD +
-                                                   static_cast<size_t>(off / 16) * (NDC * 512) + w * 8);
-        vreg[i] = *reinterpret_cast<const bf16x8*>(v_pages + (head * HD + d) * page_size + off + h * 8);
-        if (sk0 + h * 8 + 8 > hi_g) {  // keys at or beyond hi_g may be unwritten: their values count as 0
+  for (int i = 0; i < CPW; ++i) {
+    const int c = wave + kWaves * i;
+    k_off[i] = (c % NDC) * 512 + lane * 8;
+    // lane -> (block of 16 dimensions lane / 32, keys 8h .. 8h + 7 with h = lane % 32 / 16, dimension lane % 16 of
+    // the block): in LDS a block is [h][dimension][8 keys], which the operand reads below take without bank conflicts
+    v_off[i] = ((c % NDC) * 32 + (lane / 32) * 16 + lane % 16) * page_size + ((lane % 32) / 16) * 8;
+    lds_off[i] = __builtin_amdgcn_readfirstlane(c * 512);
+  }
+  const int t_first = __builtin_amdgcn_readfirstlane(wave / NDC);  // sub-tile of chunk 0 (1 only for waves 2, 3 of NDC 2)
+  // Where sub-tile n of this wave lies for the tile asked for next: block blk[n] of the table, key off[n] of its
+  // page; kept by stepping, without divisions.  All of it is the same for the whole wave: scalar registers.
+  int blk[NT], off[NT];
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (sk0 + h * 8 + e >= hi_g) vreg[i][e] = to_bf16_raw(0.f);
-        }
+  for (int n = 0; n < NT; ++n) {
+    const int sk0 = tb * kTile + (t_first + n) * 16;
+    blk[n] = __builtin_amdgcn_readfirstlane(sk0 / page_size);
+    off[n] = __builtin_amdgcn_readfirstlane(sk0 % page_size);
+  }
+  const int64_t page_stride = static_cast<int64_t>(Kh) * page_size * HD;  // elements of a page, keys or values
+  const bf16* const k_head = k_pages + static_cast<int64_t>(kh) * page_size * HD;
+  const bf16* const v_head = v_pages + static_cast<int64_t>(kh) * page_size * HD;
+  // Asks for this wave's chunks of `tile` (called for consecutive tiles) into a buffer.  A sub-tile without a page
+  // (beyond the keys, or given back by a windowed layer) reads page 0; its values are dropped when they are used.
+  auto request = [&](int tile, __bf16* stage) __attribute__((always_inline)) {
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+      const int sk0 = tile * kTile + (t_first + n) * 16;
+      const bool ok = tile < te && sk0 < hi_g && sk0 + 16 > lo_g;
+      const int page = ok ? table[blk[n]] : 0;
+      const bf16* const kb = k_head + page * page_stride + (off[n] >> 4) * (NDC * 512);
+      const bf16* const vb = v_head + page * page_stride + off[n];
+#pragma unroll
+      for (int m = 0; m < CPT; ++m) {
+        const int i = n * CPT + m;
+        __bf16* const k_to = stage + lds_off[i];
+        __bf16* const v_to = k_to + HALF;
+        load_to_lds(kb + k_off[i], k_to);
+        load_to_lds(vb + v_off[i], v_to);
       }
-    }
-  };
-  // registers -> LDS
-  auto stash = [&]() {
+      off[n] += kTile;
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-      const int p = i * 256 + tid;
-      const int t = p / SUB, w = p % SUB;
-      *reinterpret_cast<bf16x8*>(k_s + static_cast<size_t>(p) * 8) = kreg[i];
-      const int d = w / 2, h = w % 2;
-      const int db = d / 16, dr = d % 16;
-      const bf16x4 first = {vreg[i][0], vreg[i][1], vreg[i][2], vreg[i][3]};
-      const bf16x4 second = {vreg[i][4], vreg[i][5], vreg[i][6], vreg[i][7]};
-      // operand lane (grp', dr) holds keys 4 * grp' .. + 3 of each sub-tile: elements t * 4 .. + 3
-      *reinterpret_cast<bf16x4*>(v_s + ((db * 64 + (2 * h) * 16 + dr) * 8 + t * 4)) = first;
-      *reinterpret_cast<bf16x4*>(v_s + ((db * 64 + (2 * h + 1) * 16 + dr) * 8 + t * 4)) = second;
+      for (int twice = 0; twice < 2; ++twice)
+        if (off[n] >= page_size) {
+          off[n] -= page_size;
+          ++blk[n];
+        }
     }
   };
+
   // one tile from LDS, for this wave's rows
-  auto compute = [&](int tile) {
+  auto compute = [&](int tile, const __bf16* stage) __attribute__((always_inline)) {
     const int key0 = tile * kTile;
-    if (rows == 0 || key0 > pos_last || key0 + kTile <= lo_first) return;  // no row of the wave sees a key of it
-    floatx4 s[2];
+    bool any = false;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < R; ++j) any = any || (rows[j] > 0 && key0 <= pos_last[j] && key0 + kTile > lo_first[j]);
+    if (tile >= te || !any) return;  // no row of the wave sees a key of it
+    const __bf16* k_s = stage;
+    const __bf16* v_s = stage + HALF;
+    // Operands come from LDS in batches that are issued together, so that their latency is paid once per batch.
+    constexpr int KB = NDC < 4 ? NDC : 4;  // dimension chunks per batch of key operands
+    floatx4 s[R][2];
 #pragma unroll
-      for (int dc = 0; dc < NDC; ++dc) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(k_s + ((t * NDC + dc) * 64 + lane) * 8);
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[dc], s[t], 0, 0, 0);
-      }
+    for (int j = 0; j < R; ++j) s[j][0] = s[j][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dc0 = 0; dc0 < NDC; dc0 += KB) {
+      bf16x8 kf[2][KB];
+#pragma unroll
+      for (int b = 0; b < KB; ++b)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          kf[t][b] = *reinterpret_cast<const bf16x8*>(k_s + ((t * NDC + dc0 + b) * 64 + lane) * 8);
+#pragma unroll
+      for (int b = 0; b < KB; ++b)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < R; ++j)
+            s[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][b], qf[j][dc0 + b], s[j][t], 0, 0, 0);
     }
-    // every row of the wave sees every key of the tile: no mask
-    const bool whole = rows == 16 && key0 + kTile - 1 <= pos_first && key0 >= lo_last;
-    float y[2][4];
-    float mx = -INFINITY;
+    bf16x8 pf[R];
+    float alpha[R];
+    bool rescale = false;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int j = 0; j < R; ++j) {
+      // every row of the unit sees every key of the tile: no mask
+      const bool whole = rows[j] == 16 && key0 + kTile - 1 <= pos_first[j] && key0 >= lo_last[j];
+      float y[2][4];
+      float mx = -INFINITY;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        float x = s[t][v] * c1;
-        if (soft_cap > 0.f) x = c2 - 2.f * c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x) + 1.f);
-        if (!whole) {
-          const int key = key0 + t * 16 + grp * 4 + v;
-          x = (row_ok && key <= pos_r && key >= lo_r) ? x : -INFINITY;
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float x = s[j][t][v] * c1;
+          if (soft_cap > 0.f) x = c2 - 2.f * c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x) + 1.f);
+          if (!whole) {
+            const int key = key0 + t * 16 + grp * 4 + v;
+            x = (row_ok[j] && key <= pos_r[j] && key >= lo_r[j]) ? x : -INFINITY;
+          }
+          y[t][v] = x;
+          mx = fmaxf(mx, x);
         }
-        y[t][v] = x;
-        mx = fmaxf(mx, x);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m_run[j], mx);
+      // a row that has seen no visible key yet keeps m = -inf; 2^(-inf - -inf) must not appear
+      alpha[j] = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run[j] - m_new);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float e = __builtin_amdgcn_exp2f(y[t][v] - m_use);  // 2^-inf = 0
+          psum += e;
+          pf[j][t * 4 + v] = to_bf16_raw(e);
+        }
+      l_run[j] = l_run[j] * alpha[j] + psum;
+      m_run[j] = m_new;
+      rescale = rescale || alpha[j] != 1.f;
+    }
+    if (__builtin_amdgcn_ballot_w64(rescale) != 0) {  // rarely, once the maxima have settled
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[j][db][v] *= alpha[j];
+    }
+    // Lane (d = r, grp) of the value operand holds V^T[db * 16 + r][keys 4 * grp .. + 3 of each sub-tile].  Values of
+    // keys that no row may use (unwritten, given back, another request's) count as 0; their scores are masked
+    // anyway.  That concerns the last tile of the keys and tiles at a window's lower edge.
+    constexpr int VB = 4;  // output blocks per batch of value operands
+    const bool fix = key0 + kTile > hi_g || key0 < lo_g;  // uniform
+#pragma unroll
+    for (int db0 = 0; db0 < NDB; db0 += VB) {
+      bf16x8 vf[VB];
+#pragma unroll
+      for (int b = 0; b < VB; ++b) {
+        const int at = (db0 + b) * 256 + (grp / 2) * 128 + r * 8 + (grp % 2) * 4;
+        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_s + at);
+        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_s + HD * 16 + at);
+        vf[b] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new = fmaxf(m_run, mx);
-    // a row that has seen no visible key yet keeps m = -inf; 2^(-inf - -inf) must not appear
-    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    float psum = 0.f;
-    bf16x8 pf;
+      if (fix) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+        for (int b = 0; b < VB; ++b)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const float e = __builtin_amdgcn_exp2f(y[t][v] - m_use);  // 2^-inf = 0
-        psum += e;
-        pf[t * 4 + v] = to_bf16_raw(e);
+          for (int e = 0; e < 8; ++e) {
+            const int key = key0 + (e / 4) * 16 + grp * 4 + (e % 4);
+            if (key >= hi_g || key < lo_g) vf[b][e] = to_bf16_raw(0.f);
+          }
       }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;  // rarely, once the maxima have settled
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) {
-      const bf16x8 vf = *reinterpret_cast<const bf16x8*>(v_s + (db * 64 + lane) * 8);
-      if (rescale) {
+      for (int b = 0; b < VB; ++b)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) acc[db][v] *= alpha;
-      }
-      acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, acc[db], 0, 0, 0);
+        for (int j = 0; j < R; ++j)
+          acc[j][db0 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf[j], acc[j][db0 + b], 0, 0, 0);
     }
   };
 
   if (tb < te) {
-    fetch(tb);
-    stash();
-    __syncthreads();
-    for (int tile = tb; tile < te; ++tile) {
-      const bool more = tile + 1 < te;
-      if (more) fetch(tile + 1);
-      compute(tile);
-      __syncthreads();  // every wave has read the tile
-      if (more) stash();
-      __syncthreads();
+    request(tb, stage0);
+    // tile `tile` has been asked for into `cur`; `other` held tile - 1 and takes tile + 1
+    auto step = [&](int tile, const __bf16* cur, __bf16* other) __attribute__((always_inline)) {
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's chunks of `tile` have arrived
+      bare_barrier();  // and everyone's; and every wave has finished tile - 1
+      request(tile + 1, other);
+      compute(tile, cur);
+    };
+    const int te2 = tb + (te - tb + 1) / 2 * 2;
+    for (int tile = tb; tile < te2; tile += 2) {
+      step(tile, stage0, stage1);
+      step(tile + 1, stage1, stage0);
     }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the load asked for beyond the range
   }
 
   // acc[db][v] is O^T[d = db * 16 + 4 * grp + v][row r]
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
-  if (!row_ok) return;
-  if (num_splits == 1) {
-    bf16* op = out + static_cast<size_t>(sm.q_start + qi) * out_stride + static_cast<size_t>(kh * G + g) * HD;
-    const float inv = 1.f / l_run;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) {
-      const bf16x4 o4 = {to_bf16_raw(acc[db][0] * inv), to_bf16_raw(acc[db][1] * inv), to_bf16_raw(acc[db][2] * inv),
-                         to_bf16_raw(acc[db][3] * inv)};
-      *reinterpret_cast<bf16x4*>(op + db * 16 + 4 * grp) = o4;
-    }
-  } else {
-    // the merge kernel works with natural logarithms
-    const size_t row_words = HD + 2;
-    const size_t unit = static_cast<size_t>(blockIdx.z * kUnitsPerGroup + wave) * Kh + kh;
-    float* wp = workspace + ((unit * num_splits + split) * 16 + r) * row_words;
+  for (int j = 0; j < R; ++j) {
+    float l = l_run[j];
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (!row_ok[j]) continue;
+    if (num_splits == 1) {
+      bf16* op = out + static_cast<size_t>(q_row[j]) * out_stride + static_cast<size_t>(kh * G + g) * HD;
+      const float inv = 1.f / l;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) *reinterpret_cast<floatx4*>(wp + db * 16 + 4 * grp) = acc[db];
-    if (grp == 0) {
-      wp[HD] = m_run * (1.f / kLog2e);
-      wp[HD + 1] = l_run;
+      for (int db = 0; db < NDB; ++db) {
+        const bf16x4 o4 = {to_bf16_raw(acc[j][db][0] * inv), to_bf16_raw(acc[j][db][1] * inv),
+                           to_bf16_raw(acc[j][db][2] * inv), to_bf16_raw(acc[j][db][3] * inv)};
+        *reinterpret_cast<bf16x4*>(op + db * 16 + 4 * grp) = o4;
+      }
+    } else {
+      // the merge kernel works with natural logarithms
+      const size_t row_words = HD + 2;
+      const size_t unit = static_cast<size_t>(blockIdx.z * GROUP + wave * R + j) * Kh + kh;
+      float* wp = workspace + ((unit * num_splits + split) * 16 + r) * row_words;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) *reinterpret_cast<floatx4*>(wp + db * 16 + 4 * grp) = acc[j][db];
+      if (grp == 0) {
+        wp[HD] = m_run[j] * (1.f / kLog2e);
+        wp[HD + 1] = l;
+      }
     }
   }
 }
 
 }  // namespace prefill
+
+constexpr int kPrefillRowTiles = 1;  // R: units per wave
+
+int paged_attention_prefill_group() { return prefill::kWaves * kPrefillRowTiles; }
 
 bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q,
                                    int64_t out_stride, const void* out) {
@@ -255,11 +363,12 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
                             hipStream_t stream) {
-  using prefill::kUnitsPerGroup;
+  constexpr int R = kPrefillRowTiles;
+  constexpr int kGroup = prefill::kWaves * R;
   if (unit_count == 0) return 0;
   const int G = H / Kh;
-  const int groups = unit_count / kUnitsPerGroup;
-  int span = window > 0 && window < max_kv_len ? window + 16 * kUnitsPerGroup : max_kv_len;  // keys a workgroup reads at most
+  const int groups = unit_count / kGroup;
+  int span = window > 0 && window < max_kv_len ? window + 16 * kGroup : max_kv_len;  // keys a workgroup reads at most
   if (span < 1) span = 1;
   const int max_tiles = (span + kTile - 1) / kTile + 1;
   int KS = num_splits;
@@ -281,11 +390,11 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   const SeqMeta* um = reinterpret_cast<const SeqMeta*>(units);
   bf16* op = static_cast<bf16*>(out);
   float* ws = static_cast<float*>(workspace);
-#define SA_LAUNCH(NDC)                                                                                          \
-  prefill::paged_attention_prefill_kernel<NDC><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table,      \
-                                                                         table_stride, um, unit_begin, op,      \
-                                                                         out_stride, Kh, G, page_size, window,  \
-                                                                         soft_cap, ws)
+#define SA_LAUNCH(NDC)                                                                                             \
+  prefill::paged_attention_prefill_kernel<NDC, R><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table,      \
+                                                                            table_stride, um, unit_begin, op,      \
+                                                                            out_stride, Kh, G, page_size, window,  \
+                                                                            soft_cap, ws)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
   else if (hd == 256) SA_LAUNCH(8);
