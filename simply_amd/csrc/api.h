@@ -118,14 +118,14 @@ bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_
 int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
-                           float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
+                           float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
                            hipStream_t stream);
 bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q,
                                    int64_t out_stride, const void* out);
 int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
-                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
+                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
                             hipStream_t stream);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,

@@ -22,7 +22,9 @@ __device__ inline __bf16 to_bf16_raw(float f) { return static_cast<__bf16>(f); }
 
 // Partial results of key ranges lie in the workspace as [unit * Kh + kh][range][16 rows][hd + 2] floats: the
 // unnormalised output, then the maximum and the sum of the row.  Adds them up, range by range in order, into `out`.
+// max_q_len: the most tokens in a unit.
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
-                           int unit_count, bf16* out, int64_t out_stride, int Kh, int G, hipStream_t stream);
+                           int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
+                           hipStream_t stream);
 
 }  // namespace sa

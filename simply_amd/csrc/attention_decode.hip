@@ -314,7 +314,7 @@ bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_
 int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
-                           float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
+                           float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
                            hipStream_t stream) {
   if (seq_count == 0) return 0;
   const int G = H / Kh;
@@ -353,13 +353,16 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   }
 #undef SA_LAUNCH
   if (check_launch("paged_attention_decode")) return 1;
-  if (KS > 1) return attention_merge_ranges(ws, KS, hd, sm, seq_begin, seq_count, op, out_stride, Kh, G, stream);
+  if (KS > 1) return attention_merge_ranges(ws, KS, hd, sm, seq_begin, seq_count, max_q_len, op, out_stride, Kh, G, stream);
   return 0;
 }
 
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
-                           int unit_count, bf16* out, int64_t out_stride, int Kh, int G, hipStream_t stream) {
-  paged_attention_merge_kernel<<<dim3(Kh, unit_count, 16), 256, 0, stream>>>(workspace, num_ranges, hd, units, unit_begin,
+                           int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
+                           hipStream_t stream) {
+  // one workgroup per row: rows beyond the longest unit's are not launched
+  const int max_rows = G * max_q_len < 16 ? G * max_q_len : 16;
+  paged_attention_merge_kernel<<<dim3(Kh, unit_count, max_rows), 256, 0, stream>>>(workspace, num_ranges, hd, units, unit_begin,
                                                                             out, out_stride, Kh, G);
   return check_launch("paged_attention_merge");
 }

@@ -50,7 +50,7 @@ __device__ __forceinline__ void load_to_lds(const bf16* src, __bf16* dst) {
   __builtin_amdgcn_global_load_lds(src, dst, 16, 0, 0);
 }
 
-template <int NDC, int R>
+template <int NDC, int R, bool CAP>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
@@ -70,7 +70,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int r = lane % 16, grp = lane / 16;
   const int split = blockIdx.x, num_splits = gridDim.x, kh = blockIdx.y;
-  const int u0 = unit_begin + blockIdx.z * GROUP;
+  // later units of a prompt see more keys: they are started first
+  const int group = gridDim.z - 1 - blockIdx.z;
+  const int u0 = unit_begin + group * GROUP;
 
   // the keys that some row of the workgroup sees: [lo_g, hi_g)
   int lo_g = 0x7fffffff, hi_g = 0, slot = 0;
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   }
 
   // scores in base-2 units: y = log2(e) * cap * tanh(s / cap) = c2 - 2 * c2 / (2^(s * c1) + 1), or log2(e) * s
-  const float c1 = soft_cap > 0.f ? 2.f * kLog2e / soft_cap : kLog2e;
+  const float c1 = CAP ? 2.f * kLog2e / soft_cap : kLog2e;
   const float c2 = soft_cap * kLog2e;
 
   // Chunk c = wave + 4 * i of a tile's keys is the KiB (sub-tile t = c / NDC, dimensions 32 * (c % NDC) ..): 64 lanes
@@ -155,19 +157,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     blk[n] = __builtin_amdgcn_readfirstlane(sk0 / page_size);
     off[n] = __builtin_amdgcn_readfirstlane(sk0 % page_size);
   }
-  const int64_t page_stride = static_cast<int64_t>(Kh) * page_size * HD;  // elements of a page, keys or values
+  const uint32_t page_stride = static_cast<uint32_t>(Kh) * page_size * HD;  // elements of a page, keys or values
   const bf16* const k_head = k_pages + static_cast<int64_t>(kh) * page_size * HD;
   const bf16* const v_head = v_pages + static_cast<int64_t>(kh) * page_size * HD;
+  // sub-tiles (of 16 keys) with a page that this workgroup may read: [sub_lo, sub_hi)
+  const int sub_lo = lo_g / 16, sub_hi = min((hi_g + 15) / 16, te * 2);
   // Asks for this wave's chunks of `tile` (called for consecutive tiles) into a buffer.  A sub-tile without a page
   // (beyond the keys, or given back by a windowed layer) reads page 0; its values are dropped when they are used.
   auto request = [&](int tile, __bf16* stage) __attribute__((always_inline)) {
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
-      const int sk0 = tile * kTile + (t_first + n) * 16;
-      const bool ok = tile < te && sk0 < hi_g && sk0 + 16 > lo_g;
-      const int page = ok ? table[blk[n]] : 0;
-      const bf16* const kb = k_head + page * page_stride + (off[n] >> 4) * (NDC * 512);
-      const bf16* const vb = v_head + page * page_stride + off[n];
+      const int sub = tile * 2 + t_first + n;
+      const uint32_t page = (sub >= sub_lo && sub < sub_hi) ? static_cast<uint32_t>(table[blk[n]]) : 0u;
+      const uint64_t at = static_cast<uint64_t>(page) * page_stride;
+      const bf16* const kb = k_head + at + static_cast<uint32_t>(off[n] >> 4) * (NDC * 512);
+      const bf16* const vb = v_head + at + static_cast<uint32_t>(off[n]);
 #pragma unroll
       for (int m = 0; m < CPT; ++m) {
         const int i = n * CPT + m;
@@ -230,14 +234,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           float x = s[j][t][v] * c1;
-          if (soft_cap > 0.f) x = c2 - 2.f * c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x) + 1.f);
-          if (!whole) {
-            const int key = key0 + t * 16 + grp * 4 + v;
-            x = (row_ok[j] && key <= pos_r[j] && key >= lo_r[j]) ? x : -INFINITY;
-          }
+          if (CAP) x = c2 - 2.f * c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x) + 1.f);
           y[t][v] = x;
-          mx = fmaxf(mx, x);
         }
+      if (!whole) {  // uniform over the wave
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int key = key0 + t * 16 + grp * 4 + v;
+            y[t][v] = (row_ok[j] && key <= pos_r[j] && key >= lo_r[j]) ? y[t][v] : -INFINITY;
+          }
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) mx = fmaxf(mx, y[t][v]);
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
       const float m_new = fmaxf(m_run[j], mx);
@@ -333,7 +345,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     } else {
       // the merge kernel works with natural logarithms
       const size_t row_words = HD + 2;
-      const size_t unit = static_cast<size_t>(blockIdx.z * GROUP + wave * R + j) * Kh + kh;
+      const size_t unit = static_cast<size_t>(group * GROUP + wave * R + j) * Kh + kh;
       float* wp = workspace + ((unit * num_splits + split) * 16 + r) * row_words;
 #pragma unroll
       for (int db = 0; db < NDB; ++db) *reinterpret_cast<floatx4*>(wp + db * 16 + 4 * grp) = acc[j][db];
@@ -361,7 +373,7 @@ bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max
 int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
-                            float soft_cap, int max_kv_len, int num_splits, void* workspace, size_t workspace_bytes,
+                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
                             hipStream_t stream) {
   constexpr int R = kPrefillRowTiles;
   constexpr int kGroup = prefill::kWaves * R;
@@ -374,7 +386,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   int KS = num_splits;
   if (KS <= 0) {
     const int wgs = groups * Kh;
-    KS = wgs >= 192 ? 1 : (256 + wgs / 2) / wgs;  // about one workgroup per CU at least
+    KS = wgs >= 384 ? 1 : (512 + wgs / 2) / wgs;  // about two workgroups per CU at least: they fill each other's waits
     const int cap_by_work = (max_tiles + 15) / 16;  // at least 16 tiles (512 keys) per workgroup
     if (KS > cap_by_work) KS = cap_by_work;
   }
@@ -390,11 +402,17 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   const SeqMeta* um = reinterpret_cast<const SeqMeta*>(units);
   bf16* op = static_cast<bf16*>(out);
   float* ws = static_cast<float*>(workspace);
-#define SA_LAUNCH(NDC)                                                                                             \
-  prefill::paged_attention_prefill_kernel<NDC, R><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table,      \
-                                                                            table_stride, um, unit_begin, op,      \
-                                                                            out_stride, Kh, G, page_size, window,  \
-                                                                            soft_cap, ws)
+#define SA_LAUNCH(NDC)                                                                                              \
+  do {                                                                                                              \
+    if (soft_cap > 0.f)                                                                                             \
+      prefill::paged_attention_prefill_kernel<NDC, R, true><<<grid, 256, 0, stream>>>(                              \
+          qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
+          soft_cap, ws);                                                                                            \
+    else                                                                                                            \
+      prefill::paged_attention_prefill_kernel<NDC, R, false><<<grid, 256, 0, stream>>>(                             \
+          qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
+          soft_cap, ws);                                                                                            \
+  } while (0)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
   else if (hd == 256) SA_LAUNCH(8);
@@ -404,7 +422,8 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   }
 #undef SA_LAUNCH
   if (check_launch("paged_attention_prefill")) return 1;
-  if (KS > 1) return attention_merge_ranges(ws, KS, hd, um, unit_begin, unit_count, op, out_stride, Kh, G, stream);
+  if (KS > 1)
+    return attention_merge_ranges(ws, KS, hd, um, unit_begin, unit_count, max_q_len, op, out_stride, Kh, G, stream);
   return 0;
 }
 

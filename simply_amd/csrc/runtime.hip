@@ -96,7 +96,7 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
              "(heads per key head) * tokens <= 16; got hd=%d P=%d G=%d tokens=%d", hd, page_size, H / Kh, max_q_len);
   SA_REQUIRE(out_stride >= static_cast<int64_t>(H) * hd, "paged_attention_decode: output rows are too short");
   return paged_attention_decode(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, seq_begin, seq_count,
-                                out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len, num_splits,
+                                out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len, max_q_len, num_splits,
                                 workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
 }
 
@@ -117,6 +117,6 @@ extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const
   SA_REQUIRE(out_stride >= static_cast<int64_t>(H) * hd, "paged_attention_prefill: output rows are too short");
   return paged_attention_prefill(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, unit_begin,
                                  unit_count, out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len,
-                                 num_splits, workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes),
+                                 max_q_len, num_splits, workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes),
                                  stream);
 }
