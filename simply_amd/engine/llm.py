@@ -54,10 +54,14 @@ class LMInterface:
                  activation_dtype: str = "bfloat16", batch_size: int = 8, max_seq_len: int | None = None,
                  page_size: int = 16, max_num_issue_tokens: int = 2048, total_num_pages: int | None = None,
                  seed: int = 0, device: str = "cuda:0", poison_freed_pages: bool = False, use_graphs: bool = True,
-                 _model=None):
+                 library_gemm_min_rows: int | None = None, _model=None):
         from ..kernels import lib
 
         lib.load()  # fails here, loudly, if the kernel library is missing and cannot be built
+        if library_gemm_min_rows is not None:  # before the weights are laid out: they keep a second form for it
+            from ..kernels import ops
+
+            ops.set_library_gemm_min_rows(library_gemm_min_rows)
         dtype = EngineConfig(activation_dtype=activation_dtype).dtype
         if _model is not None:       # a model that is already on the device (several engines over one set of weights)
             self.model, self.model_config = _model, config

@@ -229,6 +229,21 @@ def _workspace(device) -> torch.Tensor:
     return _scratch[key]
 
 
+# Plain products (no epilogue) of at least this many rows go to the library (hipBLASLt through torch.matmul) when
+# the weight has kept its row-major form; 0: never.  The gated and soft-capped products and everything with fewer
+# rows run on this package's kernels.
+_library_gemm_min_rows = 256
+
+
+def set_library_gemm_min_rows(rows: int) -> None:
+    global _library_gemm_min_rows
+    _library_gemm_min_rows = max(0, int(rows))
+
+
+def library_gemm_min_rows() -> int:
+    return _library_gemm_min_rows
+
+
 def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
          soft_cap: float | None = None, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
          algo: int = ALGO_AUTO, shape: int = 0) -> torch.Tensor:
@@ -268,6 +283,9 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
     if tuple(out.shape) != (M, N):
         raise KernelError("gemm: bad output shape")
     ldc = _rows(out, "gemm: out")
+    if (algo == ALGO_AUTO and packed and w.row_major is not None and epi == EPILOGUE_NONE and out.dtype == a.dtype
+            and 0 < _library_gemm_min_rows <= M):
+        return torch.matmul(a, w.row_major.t(), out=out)
     ws = _workspace(a.device)
     _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(wd), _ptr(w2d), _code(wd), _ptr(out), _code(out), ldc, M, N, K, epi,
               cap, algo, int(packed), int(shape), _ptr(ws), ws.numel(), _stream())

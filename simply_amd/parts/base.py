@@ -61,14 +61,22 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
-def as_product_weight(t: torch.Tensor, shared: bool = False):
+def as_product_weight(t: torch.Tensor, shared: bool = False, many_rows: bool = False):
     """A matrix in the form that the matrix-product kernels read fastest: bfloat16 matrices on the GPU are
     re-laid in tiles (simply_amd/kernels/packing.py), anything else stays row-major.  `shared`: parts that are
-    handed the same tensor during one load (a tied table and head) get the same re-laid copy."""
+    handed the same tensor during one load (a tied table and head) get the same re-laid copy.  `many_rows`: the
+    weight of a plain product that portions of prompts go through; it also keeps its row-major form, which the
+    library product for many rows reads (unless that is switched off: ops.set_library_gemm_min_rows(0))."""
+    import dataclasses as dc
+
+    from ..kernels import ops
     from ..kernels.packing import pack_tiles
 
     if t.dtype == torch.bfloat16 and t.is_cuda and t.dim() == 2:
-        return pack_tiles(t, cached=shared)
+        tiled = pack_tiles(t, cached=shared)
+        if many_rows and ops.library_gemm_min_rows() > 0:
+            tiled = dc.replace(tiled, row_major=t.contiguous())
+        return tiled
     return t
 
 
