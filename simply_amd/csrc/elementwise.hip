@@ -122,6 +122,75 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
   }
 }
 
+// The same for many rows (portions of prompts): one wave per row, the row in registers as 4-element pieces, wave
+// reductions only.  NCH: 256-element pieces of a row at most; D % 4 == 0 and 16-byte aligned rows.
+template <typename YT, typename OT, int NCH>
+__global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(
+    const YT* __restrict__ y, const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_one_post,
+    float* __restrict__ residual, const void* __restrict__ w_next, int w_next_dtype, float eps_next, float plus_one_next,
+    OT* __restrict__ out, int T, int D) {
+  const int lane = threadIdx.x % kWave;
+  const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= T) return;
+  const size_t rb = static_cast<size_t>(row) * D;
+  float4 hv[NCH], yv[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int d = c * 256 + lane * 4;
+    hv[c] = d < D ? *reinterpret_cast<const float4*>(residual + rb + d) : float4{0.f, 0.f, 0.f, 0.f};
+    yv[c] = float4{0.f, 0.f, 0.f, 0.f};
+    if (d < D) {
+      if constexpr (sizeof(YT) == 4) {
+        yv[c] = *reinterpret_cast<const float4*>(y + rb + d);
+      } else {
+        const uint2 raw = *reinterpret_cast<const uint2*>(y + rb + d);
+        yv[c] = float4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                       __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
+      }
+    }
+  }
+  float r = 1.f;
+  if (w_post != nullptr) {
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) ss += yv[c].x * yv[c].x + yv[c].y * yv[c].y + yv[c].z * yv[c].z + yv[c].w * yv[c].w;
+    r = rsqrtf(wave_sum(ss) / static_cast<float>(D) + eps_post);
+  }
+  float ss2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int d = c * 256 + lane * 4;
+    if (d >= D) continue;
+    float* h = reinterpret_cast<float*>(&hv[c]);
+    const float* v = reinterpret_cast<const float*>(&yv[c]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      h[e] += w_post != nullptr ? v[e] * r * (load_f(w_post, w_post_dtype, d + e) + plus_one_post) : v[e];
+      ss2 += h[e] * h[e];
+    }
+    *reinterpret_cast<float4*>(residual + rb + d) = hv[c];
+  }
+  if (w_next == nullptr) return;
+  const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(D) + eps_next);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int d = c * 256 + lane * 4;
+    if (d >= D) continue;
+    const float* h = reinterpret_cast<const float*>(&hv[c]);
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = h[e] * r2 * (load_f(w_next, w_next_dtype, d + e) + plus_one_next);
+    if constexpr (sizeof(OT) == 4) {
+      *reinterpret_cast<float4*>(out + rb + d) = float4{o[0], o[1], o[2], o[3]};
+    } else {
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(float_to_bf16(o[0]).bits) | (static_cast<uint32_t>(float_to_bf16(o[1]).bits) << 16);
+      packed.y = static_cast<uint32_t>(float_to_bf16(o[2]).bits) | (static_cast<uint32_t>(float_to_bf16(o[3]).bits) << 16);
+      *reinterpret_cast<uint2*>(out + rb + d) = packed;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ rotary + cache write
 // One block per (token, head) of a fused [T, (H + 2K) * hd] projection.
 //   q heads: rotate, divide by query_scale, write back in place.
@@ -185,6 +254,51 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
     T* dst = v_pages + (page * K + (head - H - K)) * page_size * hd + off;
     for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[static_cast<size_t>(i) * page_size] = src[i];
   }
+}
+
+// The same for many tokens: one block per token, which works out the sines and cosines of the token's angles once
+// for all heads (hd / 2 <= kMaxHalf).
+constexpr int kMaxHalf = 512;
+template <typename T>
+__global__ __launch_bounds__(256) void rope_cache_write_rows_kernel(
+    T* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ timescale,
+    float inv_scale_factor, float q_div, const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int H, int K, int hd, int page_size) {
+  __shared__ float sn[kMaxHalf], cs[kMaxHalf];
+  const int t = blockIdx.x, half = hd / 2;
+  const float pos = static_cast<float>(positions[t]);
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float s = 0.f, c = 1.f;
+    if (timescale != nullptr) sincosf(pos / timescale[i] * inv_scale_factor, &s, &c);
+    sn[i] = s;
+    cs[i] = c;
+  }
+  __syncthreads();
+  T* row = qkv + static_cast<size_t>(t) * row_stride;
+  const int64_t slot = slot_mapping != nullptr ? slot_mapping[t] : -1;
+  const bool write = k_pages != nullptr && slot >= 0;
+  const int64_t page = write ? slot / page_size : 0;
+  const int koff = write ? static_cast<int>(slot % page_size) : 0;
+  const bool tiled = keys_tiled(page_size, hd);
+  for (int idx = threadIdx.x; idx < (H + K) * half; idx += blockDim.x) {
+    const int head = idx / half, i = idx % half;
+    T* src = row + static_cast<size_t>(head) * hd;
+    const float x1 = to_float(src[i]), x2 = to_float(src[i + half]);
+    const float o1 = x1 * cs[i] - x2 * sn[i], o2 = x2 * cs[i] + x1 * sn[i];
+    if (head < H) {
+      src[i] = from_float<T>(o1 / q_div);
+      src[i + half] = from_float<T>(o2 / q_div);
+    } else if (write) {
+      T* dst = k_pages + (page * K + (head - H)) * page_size * hd;
+      dst[key_index(tiled, page_size, hd, koff, i)] = from_float<T>(o1);
+      dst[key_index(tiled, page_size, hd, koff, i + half)] = from_float<T>(o2);
+    }
+  }
+  if (!write) return;
+  // value pages are [page, head, hd, page_size]: the keys of a page are contiguous for each dimension
+  const T* vsrc = row + static_cast<size_t>(H + K) * hd;
+  T* vdst = v_pages + page * K * page_size * hd + koff;
+  for (int idx = threadIdx.x; idx < K * hd; idx += blockDim.x) vdst[static_cast<size_t>(idx) * page_size] = vsrc[idx];
 }
 
 // Rotation alone, in place, on [T, n_heads, hd] rows of stride row_stride.
@@ -256,6 +370,29 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
   if (T == 0) return 0;
   SA_REQUIRE(T > 0 && D > 0, "add_rmsnorm: bad sizes T=%d D=%d", T, D);
   SA_REQUIRE(w_next == nullptr || out != nullptr, "add_rmsnorm: a next norm needs an output");
+  // many rows: a wave per row
+  const auto aligned16 = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  const int o_dtype = out != nullptr ? out_dtype : y_dtype;
+  if (T >= 32 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out)) {
+    const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
+    const int blocks = (T + 3) / 4;
+#define SA_ROWS(YT, OT, NCH)                                                                                      \
+  add_rmsnorm_rows_kernel<YT, OT, NCH><<<blocks, 256, 0, stream>>>(static_cast<const YT*>(y), w_post, w_post_dtype, \
+                                                                   eps_post, pp, residual, w_next, w_next_dtype,    \
+                                                                   eps_next, pn, static_cast<OT*>(out), T, D)
+#define SA_ROWS_N(YT, OT)     \
+  do {                        \
+    if (D <= 2560) SA_ROWS(YT, OT, 10); \
+    else SA_ROWS(YT, OT, 20); \
+  } while (0)
+    if (y_dtype == kBF16 && o_dtype == kBF16) SA_ROWS_N(bf16, bf16);
+    else if (y_dtype == kBF16) SA_ROWS_N(bf16, float);
+    else if (o_dtype == kBF16) SA_ROWS_N(float, bf16);
+    else SA_ROWS_N(float, float);
+#undef SA_ROWS_N
+#undef SA_ROWS
+    return check_launch("add_rmsnorm");
+  }
   add_rmsnorm_kernel<<<T, row_threads(D), 0, stream>>>(y, y_dtype, w_post, w_post_dtype, eps_post,
                                                        plus_one_post ? 1.f : 0.f, residual, w_next, w_next_dtype,
                                                        eps_next, plus_one_next ? 1.f : 0.f, out, out_dtype, D);
@@ -274,6 +411,21 @@ extern "C" int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, con
   SA_REQUIRE(page_size > 0 && scale_factor > 0.f && q_div > 0.f, "rope_cache_write: bad page size, scale factor or query scale");
   SA_REQUIRE((k_pages == nullptr) == (v_pages == nullptr) && (k_pages == nullptr || slot_mapping != nullptr),
              "rope_cache_write: key pages, value pages and slots come together");
+  if (T >= 32 && hd / 2 <= kMaxHalf) {  // many tokens: a block per token
+    if (dtype == kF32)
+      rope_cache_write_rows_kernel<float><<<T, 256, 0, stream>>>(static_cast<float*>(qkv), row_stride, positions,
+                                                                 timescale, 1.f / scale_factor, q_div, slot_mapping,
+                                                                 static_cast<float*>(k_pages),
+                                                                 static_cast<float*>(v_pages), H, K, hd, page_size);
+    else if (dtype == kBF16)
+      rope_cache_write_rows_kernel<bf16><<<T, 256, 0, stream>>>(static_cast<bf16*>(qkv), row_stride, positions,
+                                                                timescale, 1.f / scale_factor, q_div, slot_mapping,
+                                                                static_cast<bf16*>(k_pages),
+                                                                static_cast<bf16*>(v_pages), H, K, hd, page_size);
+    else
+      SA_REQUIRE(false, "rope_cache_write: unknown dtype %d", dtype);
+    return check_launch("rope_cache_write");
+  }
   const dim3 grid(T, H + 2 * K);
   const int threads = hd / 2 >= 128 ? 128 : 64;
   if (dtype == kF32)

@@ -50,7 +50,7 @@ def test_rmsnorm(dtype, T, D):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304)])
+@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304), (40, 2304), (33, 100), (35, 5000), (32, 6000), (37, 50)])
 def test_add_rmsnorm(dtype, T, D):
     from simply_amd.kernels import ops
     y = rand((T, D), dtype, 3, 2.0)
@@ -71,11 +71,12 @@ def test_add_rmsnorm(dtype, T, D):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("H,K,hd,P", [(4, 2, 16, 4), (6, 1, 32, 3), (8, 4, 256, 16), (3, 3, 48, 5)])
-def test_rope_cache_write(dtype, H, K, hd, P):
+@pytest.mark.parametrize("T", [11, 44])   # few tokens: a block per (token, head); many: a block per token
+def test_rope_cache_write(dtype, H, K, hd, P, T):
     from simply_amd.kernels import ops
-    T, pages = 11, 9
+    pages = -(-T // P) + 6
     qkv = rand((T, (H + 2 * K) * hd), dtype, 7)
-    positions = torch.tensor([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7], dtype=torch.int32).cuda()
+    positions = torch.tensor(([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7] * 4)[:T], dtype=torch.int32).cuda()
     ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda()
     slots = torch.randperm(pages * P)[:T].to(torch.int64).cuda()
     kp, vp = torch.zeros((pages, K, P, hd), dtype=dtype).cuda(), torch.zeros((pages, K, hd, P), dtype=dtype).cuda()
