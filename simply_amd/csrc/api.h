@@ -61,6 +61,17 @@ int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* 
 // h_out = h_in + y), a = norm(h_out; w_next), C = epilogue(a . W^T) with W tiled (paired tiles for epilogue 1).
 // h_in, h_out: float32 [M, K], different buffers; y: bfloat16 [M, K]; norm weights float32 or bfloat16 [K].
 int sa_gemm_normed_takes(int M, int N, int K);
+
+// The fused q/k/v projection with the norms of sa_gemm_normed in front and the rotation, query scale and cache write
+// of sa_rope_cache_write behind: C receives the queries [M, H * hd] (rows of ldc elements), keys and values go into
+// the pages.  W has (H + 2 Kh) * hd rows, hd a multiple of 32.  timescale null: no rotation; slot_mapping null: no
+// cache write.
+int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype,
+                          float eps_post, int plus_one_post, const void* w_next, int w_next_dtype, float eps_next,
+                          int plus_one_next, const void* W, void* C, int c_dtype, int64_t ldc, int M, int K,
+                          const int* positions, const float* timescale, float scale_factor, float q_div,
+                          const int64_t* slot_mapping, void* k_pages, void* v_pages, int H, int Kh, int hd,
+                          int page_size, hipStream_t stream);
 int sa_gemm_normed(const void* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype, float eps_post,
                    int plus_one_post, const void* w_next, int w_next_dtype, float eps_next, int plus_one_next,
                    const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap,

@@ -370,10 +370,10 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
   if (T == 0) return 0;
   SA_REQUIRE(T > 0 && D > 0, "add_rmsnorm: bad sizes T=%d D=%d", T, D);
   SA_REQUIRE(w_next == nullptr || out != nullptr, "add_rmsnorm: a next norm needs an output");
-  // many rows: a wave per row
+  // many rows (enough for two workgroups of four rows per compute unit): a wave per row
   const auto aligned16 = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   const int o_dtype = out != nullptr ? out_dtype : y_dtype;
-  if (T >= 32 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out)) {
+  if (T >= 512 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out)) {
     const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
     const int blocks = (T + 3) / 4;
 #define SA_ROWS(YT, OT, NCH)                                                                                      \
@@ -411,7 +411,7 @@ extern "C" int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, con
   SA_REQUIRE(page_size > 0 && scale_factor > 0.f && q_div > 0.f, "rope_cache_write: bad page size, scale factor or query scale");
   SA_REQUIRE((k_pages == nullptr) == (v_pages == nullptr) && (k_pages == nullptr || slot_mapping != nullptr),
              "rope_cache_write: key pages, value pages and slots come together");
-  if (T >= 32 && hd / 2 <= kMaxHalf) {  // many tokens: a block per token
+  if (T >= 256 && hd / 2 <= kMaxHalf) {  // many tokens (a block for every compute unit): a block per token
     if (dtype == kF32)
       rope_cache_write_rows_kernel<float><<<T, 256, 0, stream>>>(static_cast<float*>(qkv), row_stride, positions,
                                                                  timescale, 1.f / scale_factor, q_div, slot_mapping,

@@ -31,14 +31,30 @@ __device__ inline float gelu_tanh_f(float x) {
 }
 __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
+// What the rotary epilogue (EPI 3) needs: the product is the fused q/k/v projection of an attention layer, columns
+// [H query heads | Kh key heads | Kh value heads] of hd each.  Query and key heads are rotated by the token's
+// position (pairs (i, i + hd / 2), angle position / timescale[i] / scale_factor), queries divided by q_div and
+// written to C, keys and values written into the cache pages at slot_mapping[row] (as the separate rotary kernel
+// does, from the product rounded to bfloat16 as that kernel reads it).
+struct RotaryArgs {
+  const int* positions;
+  const float* timescale;       // [hd / 2], or null: no rotation
+  float inv_scale_factor, q_div;
+  const int64_t* slot_mapping;  // null: nothing is written into the cache
+  bf16* k_pages;
+  bf16* v_pages;
+  int H, Kh, hd, page_size;
+};
+
 // NCH: 256-element pieces of a row (K <= 256 * NCH)
 template <int EPI, int NCH>
 __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     const bf16* __restrict__ y, const float* __restrict__ h_in, float* __restrict__ h_out,
     const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_post,
     const void* __restrict__ w_next, int w_next_dtype, float eps_next, float plus_next, const bf16* __restrict__ W,
-    void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N, int K, int chunks, int act_rows, float cap) {
-  constexpr int NP = EPI == 1 ? 2 : 1;
+    void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N, int K, int chunks, int act_rows, float cap,
+    RotaryArgs rot) {
+  constexpr int NP = (EPI == 1 || EPI == 3) ? 2 : 1;  // tiles of W that a workgroup multiplies side by side
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int pitch = K + 8;                               // elements per row of activations in LDS
   bf16* act = reinterpret_cast<bf16*>(smem);             // [act_rows][pitch]
@@ -51,12 +67,20 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
   // ---- set-up of the product: a workgroup takes the 16-row tiles of W (pairs of tiles for the gated epilogue)
   // blockIdx.x, blockIdx.x + gridDim.x, ...; K is cut over the waves.  The first fragments of W are asked for
   // before the norms, so that their way from HBM overlaps the norms' trips to L2.
-  const int ntiles = (N + 15) / 16;
+  // work items: 16-row tiles of W; pairs (2 i, 2 i + 1) for the gated epilogue; for the rotary epilogue pairs
+  // (t, t + hd / 32) of a head's tiles, which hold the two dimensions of every rotated pair
+  const int half_tiles = EPI == 3 ? rot.hd / 32 : 1;
+  const int ntiles = EPI == 3 ? (rot.H + 2 * rot.Kh) * half_tiles : (N + 15) / 16;
   const int c0 = static_cast<int>(static_cast<int64_t>(chunks) * wave / kWaves);
   const int c1 = static_cast<int>(static_cast<int64_t>(chunks) * (wave + 1) / kWaves);
   const size_t tile_elems = static_cast<size_t>(chunks) * 512;
-  const bf16* wrow = W + (EPI == 1 ? 2 : 1) * static_cast<size_t>(blockIdx.x) * tile_elems + lane * 8;
-  const bf16* w2row = wrow + tile_elems;
+  const size_t pair_off = (EPI == 3 ? half_tiles : 1) * tile_elems;  // from the first tile of an item to its second
+  auto tile_ptr = [&](int item) {
+    const int first = EPI == 1 ? 2 * item : EPI == 3 ? (item / half_tiles) * 2 * half_tiles + item % half_tiles : item;
+    return W + static_cast<size_t>(first) * tile_elems + lane * 8;
+  };
+  const bf16* wrow = tile_ptr(blockIdx.x);
+  const bf16* w2row = wrow + pair_off;
   const bf16* arow = act + static_cast<size_t>(r) * pitch + kq * 8;
   const bool a_ok = r < act_rows;
   const bf16x8 zero = {};
@@ -68,7 +92,7 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     for (int u = 0; u < kUnroll; ++u) {
       const bool ok = c + u < c1;
       a[set][u] = ok ? load_frag(wrow + static_cast<size_t>(c + u) * 512) : zero;
-      if (EPI == 1) a2[set][u] = ok ? load_frag(w2row + static_cast<size_t>(c + u) * 512) : zero;
+      if (NP == 2) a2[set][u] = ok ? load_frag(w2row + static_cast<size_t>(c + u) * 512) : zero;
     }
   };
   auto mul_set = [&](int set, int c) {
@@ -78,10 +102,14 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
       const int k = (c + u < c1 ? c + u : c0) * 32;
       const bf16x8 b = a_ok ? load_frag(arow + k) : zero;
       acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[set][u], b, acc[0], 0, 0, 0);
-      if (EPI == 1) acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[set][u], b, acc[1], 0, 0, 0);
+      if (NP == 2) acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[set][u], b, acc[1], 0, 0, 0);
     }
   };
+  // both sets of fragments are asked for before the norms: a wave's share of a tile is two or three sets, so most
+  // of the first tile is on its way while the norms are computed
+  const int nseg = (c1 - c0 + kUnroll - 1) / kUnroll;  // sets of fragments per tile for this wave
   load_set(0, c0);
+  if (nseg >= 2) load_set(1, c0 + kUnroll);
 
   // ---- the two norms, one wave per row.  A lane holds 4 consecutive elements of each 256-element piece of the
   // row; all loads of a row are issued before the first use, so a row costs one trip to L2.
@@ -150,23 +178,31 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
 #pragma unroll
     for (int p = 0; p < NP; ++p) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bool more = tile + static_cast<int>(gridDim.x) < ntiles;
-    const size_t step = (EPI == 1 ? 2 : 1) * static_cast<size_t>(gridDim.x) * tile_elems;
-    for (int c = c0; c < c1; c += 2 * kUnroll) {
-      load_set(1, c + kUnroll);
-      mul_set(0, c);
-      if (c + 2 * kUnroll < c1) {
-        load_set(0, c + 2 * kUnroll);
-      } else if (more) {  // the next tile's first fragments
-        wrow += step;
-        w2row += step;
-        load_set(0, c0);
-        wrow -= step;
-        w2row -= step;
+    const bf16* const here = wrow;
+    const bf16* const next = tile_ptr(tile + gridDim.x);
+    // at the start of a tile set 0 holds its first fragments and set 1 its second ones; each set is asked for
+    // again as soon as it has been used: for two sets further on in this tile, or for the next tile's start
+    auto refill = [&](int set, int seg) {
+      if (seg < nseg) {
+        load_set(set, c0 + seg * kUnroll);
+      } else if (more && set < nseg) {  // set 0 takes the next tile's first fragments, set 1 its second ones
+        wrow = next;
+        w2row = next + pair_off;
+        load_set(set, c0 + set * kUnroll);
+        wrow = here;
+        w2row = here + pair_off;
       }
-      mul_set(1, c + kUnroll);
+    };
+    for (int seg = 0; seg < nseg; seg += 2) {
+      mul_set(0, c0 + seg * kUnroll);
+      refill(0, seg + 2);
+      if (seg + 1 < nseg) {
+        mul_set(1, c0 + (seg + 1) * kUnroll);
+        refill(1, seg + 3);
+      }
     }
-    wrow += step;
-    w2row += step;
+    wrow = next;
+    w2row = next + pair_off;
 
     // ---- lane holds D[n = 4 * kq + v][m = r]; the waves' tiles are added up through LDS, in wave order
     __syncthreads();  // the previous tile's sums have been read
@@ -175,7 +211,45 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) red[(wave * NP + p) * (16 * 17) + (4 * kq + v) * 17 + r] = acc[p][v];
     __syncthreads();
-    if (tid < 256) {
+    if (EPI == 3) {
+      const int ml = tid / 16, nl = tid % 16;
+      if (tid < 256 && ml < M) {
+        float x[2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          float t = 0.f;
+          for (int w = 0; w < kWaves; ++w) t += red[(w * NP + p) * (16 * 17) + nl * 17 + ml];
+          x[p] = to_float(float_to_bf16(t));
+        }
+        const int head = tile / half_tiles, i = (tile % half_tiles) * 16 + nl, half = rot.hd / 2;
+        float o1 = x[0], o2 = x[1];
+        if (head < rot.H + rot.Kh && rot.timescale != nullptr) {
+          float sn, cs;
+          sincosf(static_cast<float>(rot.positions[ml]) / rot.timescale[i] * rot.inv_scale_factor, &sn, &cs);
+          o1 = x[0] * cs - x[1] * sn;
+          o2 = x[1] * cs + x[0] * sn;
+        }
+        if (head < rot.H) {
+          const size_t at = static_cast<size_t>(ml) * ldc + static_cast<size_t>(head) * rot.hd + i;
+          store_f(C, c_dtype, at, o1 / rot.q_div);
+          store_f(C, c_dtype, at + half, o2 / rot.q_div);
+        } else if (rot.slot_mapping != nullptr && rot.slot_mapping[ml] >= 0) {
+          const int64_t slot = rot.slot_mapping[ml];
+          const int64_t page = slot / rot.page_size;
+          const int koff = static_cast<int>(slot % rot.page_size);
+          if (head < rot.H + rot.Kh) {
+            bf16* dst = rot.k_pages + (page * rot.Kh + (head - rot.H)) * rot.page_size * rot.hd;
+            const bool tiled = keys_tiled(rot.page_size, rot.hd);
+            dst[key_index(tiled, rot.page_size, rot.hd, koff, i)] = float_to_bf16(o1);
+            dst[key_index(tiled, rot.page_size, rot.hd, koff, i + half)] = float_to_bf16(o2);
+          } else {  // value pages are [page, head, hd, page_size]
+            bf16* dst = rot.v_pages + (page * rot.Kh + (head - rot.H - rot.Kh)) * rot.page_size * rot.hd + koff;
+            dst[static_cast<size_t>(i) * rot.page_size] = float_to_bf16(x[0]);
+            dst[static_cast<size_t>(i + half) * rot.page_size] = float_to_bf16(x[1]);
+          }
+        }
+      }
+    } else if (tid < 256) {
       const int ml = tid / 16, nl = tid % 16, n = tile * 16 + nl;
       if (ml < M && n < N) {
         float sum[NP];
@@ -197,10 +271,11 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
 template <int EPI, int NCH>
 static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype, float eps_post,
                   float plus_post, const void* w_next, int w_next_dtype, float eps_next, float plus_next, const bf16* W,
-                  void* C, int c_dtype, int64_t ldc, int M, int N, int K, float cap, hipStream_t stream) {
+                  void* C, int c_dtype, int64_t ldc, int M, int N, int K, float cap, const RotaryArgs& rot,
+                  hipStream_t stream) {
   const int act_rows = M <= 8 ? 8 : 16;
   const size_t lds = static_cast<size_t>(act_rows) * (K + 8) * sizeof(bf16) +
-                     static_cast<size_t>(kWaves) * (EPI == 1 ? 2 : 1) * 16 * 17 * sizeof(float);
+                     static_cast<size_t>(kWaves) * ((EPI == 1 || EPI == 3) ? 2 : 1) * 16 * 17 * sizeof(float);
   auto kernel = gemm_normed_kernel<EPI, NCH>;
   if (lds > 64 * 1024) {
     static bool raised = false;  // per instantiation
@@ -214,11 +289,11 @@ static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_
       raised = true;
     }
   }
-  const int ntiles = (N + 15) / 16;
+  const int ntiles = EPI == 3 ? (rot.H + 2 * rot.Kh) * (rot.hd / 32) : (N + 15) / 16;
   const int grid = (ntiles + (ntiles + kMaxGroups - 1) / kMaxGroups - 1) / ((ntiles + kMaxGroups - 1) / kMaxGroups);
   kernel<<<grid, kWaves * kWave, lds, stream>>>(y, h_in, h_out, w_post, w_post_dtype, eps_post, plus_post, w_next,
                                                          w_next_dtype, eps_next, plus_next, W, C, c_dtype, ldc, M, N, K,
-                                                         (K + 31) / 32, act_rows, cap);
+                                                         (K + 31) / 32, act_rows, cap, rot);
   return check_launch("gemm_normed");
 }
 
@@ -249,9 +324,41 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
   const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
 #define SA_NORMED(EPI, NCH)                                                                                      \
   return normed::launch<EPI, NCH>(yb, h_in, h_out, w_post, w_post_dtype, eps_post, pp, w_next, w_next_dtype, eps_next, \
-                                  pn, w, C, c_dtype, ldc, M, N, K, cap, stream)
+                                  pn, w, C, c_dtype, ldc, M, N, K, cap, normed::RotaryArgs{}, stream)
   if (epilogue == 0) SA_NORMED(0, 10);
   if (epilogue == 1) SA_NORMED(1, 10);
   SA_NORMED(2, 10);
 #undef SA_NORMED
+}
+
+// The fused q/k/v projection of an attention layer with the norms in front (as sa_gemm_normed) and, behind it, the
+// rotation of queries and keys, the query scale and the write of keys and values into the cache pages (as
+// sa_rope_cache_write): C receives the queries only, [M, >= H * hd] with rows of ldc elements.  W has (H + 2 Kh) * hd
+// rows; hd is a multiple of 32.  timescale null: no rotation; slot_mapping null: nothing is written into the cache.
+extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype,
+                                     float eps_post, int plus_one_post, const void* w_next, int w_next_dtype,
+                                     float eps_next, int plus_one_next, const void* W, void* C, int c_dtype, int64_t ldc,
+                                     int M, int K, const int* positions, const float* timescale, float scale_factor,
+                                     float q_div, const int64_t* slot_mapping, void* k_pages, void* v_pages, int H,
+                                     int Kh, int hd, int page_size, hipStream_t stream) {
+  SA_REQUIRE(H >= 0 && Kh >= 0 && H + 2 * Kh > 0 && hd > 0 && hd % 32 == 0,
+             "gemm_normed_rotary: bad head counts, or a head size that is no multiple of 32 (H=%d K=%d hd=%d)", H, Kh, hd);
+  const int N = (H + 2 * Kh) * hd;
+  SA_REQUIRE(sa_gemm_normed_takes(M, N, K),
+             "gemm_normed takes 1..16 rows and a width that is a multiple of 32, at most 2560, and fits in LDS; got M=%d K=%d", M, K);
+  SA_REQUIRE(ldc >= static_cast<int64_t>(H) * hd && w_next != nullptr && h_in != nullptr && W != nullptr && C != nullptr &&
+                 positions != nullptr,
+             "gemm_normed_rotary: bad arguments");
+  SA_REQUIRE(w_next_dtype == kBF16 && (w_post == nullptr || w_post_dtype == kBF16),
+             "gemm_normed: the norm weights must be bfloat16");
+  SA_REQUIRE(y == nullptr || (h_out != nullptr && h_out != h_in),
+             "gemm_normed: with y the updated residual goes to a buffer other than the input");
+  SA_REQUIRE(page_size > 0 && scale_factor > 0.f && q_div > 0.f, "gemm_normed_rotary: bad page size, scale factor or query scale");
+  SA_REQUIRE(slot_mapping == nullptr || (k_pages != nullptr && v_pages != nullptr),
+             "gemm_normed_rotary: slots come with key and value pages");
+  normed::RotaryArgs rot{positions, timescale, 1.f / scale_factor, q_div, slot_mapping, static_cast<bf16*>(k_pages),
+                         static_cast<bf16*>(v_pages), H, Kh, hd, page_size};
+  return normed::launch<3, 10>(static_cast<const bf16*>(y), h_in, h_out, w_post, w_post_dtype, eps_post,
+                               plus_one_post ? 1.f : 0.f, w_next, w_next_dtype, eps_next, plus_one_next ? 1.f : 0.f,
+                               static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, 0.f, rot, stream);
 }

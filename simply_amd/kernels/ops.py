@@ -331,6 +331,53 @@ def gemm_normed(y: torch.Tensor | None, h_in: torch.Tensor, h_out: torch.Tensor 
     return out
 
 
+def gemm_normed_rotary(y: torch.Tensor | None, h_in: torch.Tensor, h_out: torch.Tensor | None, w: TiledWeight, *,
+                       post_weight: torch.Tensor | None, post_eps: float, post_plus_one: bool,
+                       next_weight: torch.Tensor, next_eps: float, next_plus_one: bool, positions: torch.Tensor,
+                       timescale: torch.Tensor | None, scale_factor: float, query_scale: float, num_heads: int,
+                       num_kv_heads: int, head_dim: int, slot_mapping: torch.Tensor | None = None,
+                       k_pages: torch.Tensor | None = None, v_pages: torch.Tensor | None = None) -> torch.Tensor:
+    """`gemm_normed` for the fused q/k/v projection (w has (H + 2 K) * hd rows) followed by `rope_cache_write` in
+    the same kernel.  Returns [M, (H + 2 K) * hd] of which only the query columns are written."""
+    _dev(y, h_in, h_out, post_weight, next_weight, w.data, positions, timescale, slot_mapping, k_pages, v_pages)
+    M, K = h_in.shape
+    H, Kh, hd = num_heads, num_kv_heads, head_dim
+    if w.paired or w.rows != (H + 2 * Kh) * hd or w.cols != K:
+        raise KernelError("gemm_normed_rotary: the weight must have (H + 2 K) * hd rows of the residual's width")
+    if h_in.dtype != torch.float32 or not h_in.is_contiguous():
+        raise KernelError("gemm_normed_rotary: the residual must be contiguous float32 [M, K]")
+    if y is not None:
+        if y.dtype != torch.bfloat16 or tuple(y.shape) != (M, K) or not y.is_contiguous():
+            raise KernelError("gemm_normed_rotary: y must be contiguous bfloat16 [M, K]")
+        if h_out is None or h_out.dtype != torch.float32 or tuple(h_out.shape) != (M, K) or not h_out.is_contiguous() \
+                or h_out.data_ptr() == h_in.data_ptr():
+            raise KernelError("gemm_normed_rotary: the updated residual needs its own contiguous float32 [M, K] buffer")
+    for t in (post_weight, next_weight):
+        if t is not None and (t.numel() != K or not t.is_contiguous()):
+            raise KernelError("gemm_normed_rotary: a norm weight does not match the width")
+    _i32(positions, "gemm_normed_rotary: positions", M)
+    if timescale is not None and (timescale.dtype != torch.float32 or timescale.numel() != hd // 2):
+        raise KernelError("gemm_normed_rotary: timescale must be float32 [hd / 2]")
+    page_size = 1
+    if slot_mapping is not None:
+        if k_pages is None or v_pages is None:
+            raise KernelError("gemm_normed_rotary: slots come with key and value pages")
+        _check_pages(k_pages, v_pages, torch.bfloat16, "gemm_normed_rotary")
+        if k_pages.shape[1] != Kh or k_pages.shape[3] != hd:
+            raise KernelError("gemm_normed_rotary: the pages do not match the heads")
+        page_size = k_pages.shape[2]
+        if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < M or not slot_mapping.is_contiguous():
+            raise KernelError("gemm_normed_rotary: slot_mapping must be contiguous int64 with one entry per row")
+    out = torch.empty((M, w.rows), dtype=torch.bfloat16, device=h_in.device)
+    _lib.call("sa_gemm_normed_rotary", _ptr(y), _ptr(h_in), _ptr(h_out), _ptr(post_weight),
+              _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one),
+              _ptr(next_weight), _code(next_weight), float(next_eps), int(next_plus_one), _ptr(w.data), _ptr(out),
+              _code(out), out.stride(0), M, K, _ptr(positions), _ptr(timescale), float(scale_factor),
+              float(query_scale), _ptr(slot_mapping), _ptr(k_pages) if slot_mapping is not None else None,
+              _ptr(v_pages) if slot_mapping is not None else None, H, Kh, hd, int(page_size), _stream())
+    return out
+
+
 # --------------------------------------------------------------------------- attention
 
 

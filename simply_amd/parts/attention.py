@@ -6,12 +6,14 @@ q / query_scale (:1987-2020), attention over the cache with soft-cap and window
 """
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from ..config.spec import PartSpec
 from ..kernels import ops
 from ..registry import MIXERS, POSITION_ENCODINGS
-from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight, project
+from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight, pending_fits_product, pending_product, project
 
 
 @MIXERS.register("paged_attention")
@@ -54,22 +56,29 @@ class PagedAttention(Mixer):
     def forward(self, x, ctx, cache):
         H, K, hd = self.num_heads, self.num_kv_heads, self.head_dim
         group = ctx.groups[cache.group_id]
-        qkv = project(x, self.qkv_proj)
         pe = self.position_encoding
         rotary = pe.rotary_table() if pe is not None else None
         write = cache.write
-        if pe is None or rotary is not None:
+        pages = dict(slot_mapping=group.slot_mapping if write else None, k_pages=cache.k_pages if write else None,
+                     v_pages=cache.v_pages if write else None)
+        if (pe is None or rotary is not None) and hd % 32 == 0 and pending_fits_product(x, self.qkv_proj) \
+                and cache.k_pages.dtype == torch.bfloat16:
+            # a few tokens: the norms in front of the projection and the rotation, query scale and cache write
+            # behind it run in the projection's kernel
             table, sf = rotary if rotary is not None else (None, 1.0)
-            ops.rope_cache_write(qkv, ctx.positions, table, sf, self.query_scale, H, K, hd,
-                                 slot_mapping=group.slot_mapping if write else None,
-                                 k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+            qkv = pending_product(x, functools.partial(
+                ops.gemm_normed_rotary, w=self.qkv_proj, positions=ctx.positions, timescale=table, scale_factor=sf,
+                query_scale=self.query_scale, num_heads=H, num_kv_heads=K, head_dim=hd, **pages))
         else:
-            # another position encoding: applied by the part itself, then the plain scale-and-write kernel
-            pe.apply(qkv, ctx.positions, H, hd, 1.0)
-            pe.apply(qkv[:, H * hd:], ctx.positions, K, hd, 1.0)
-            ops.rope_cache_write(qkv, ctx.positions, None, 1.0, self.query_scale, H, K, hd,
-                                 slot_mapping=group.slot_mapping if write else None,
-                                 k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+            qkv = project(x, self.qkv_proj)
+            if pe is None or rotary is not None:
+                table, sf = rotary if rotary is not None else (None, 1.0)
+                ops.rope_cache_write(qkv, ctx.positions, table, sf, self.query_scale, H, K, hd, **pages)
+            else:
+                # another position encoding: applied by the part itself, then the plain scale-and-write kernel
+                pe.apply(qkv, ctx.positions, H, hd, 1.0)
+                pe.apply(qkv[:, H * hd:], ctx.positions, K, hd, 1.0)
+                ops.rope_cache_write(qkv, ctx.positions, None, 1.0, self.query_scale, H, K, hd, **pages)
         o = torch.empty((qkv.shape[0], H * hd), dtype=qkv.dtype, device=qkv.device)
         if ops.decode_attention_takes(qkv, cache.k_pages, H, 1):
             # the MFMA kernels take up to 16 query rows (tokens x heads per key head) as a unit: a decoding request

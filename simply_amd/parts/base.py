@@ -115,32 +115,48 @@ class PendingNorm:
         return self.next_norm.forward(self.settle(), self.dtype)
 
 
-def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """x . w^T (gated if w is a paired tiled weight) for activations x or a `PendingNorm`.  A pending norm is done
-    inside the product's kernel when that kernel takes the sizes (bfloat16, up to 16 rows, tiled weight, RMSNorms);
-    otherwise it is materialized first."""
+def pending_fits_product(x, w) -> bool:
+    """Whether the product kernel with the norms in front takes the pending norm `x` against the weight `w`
+    (bfloat16, up to 16 rows, a tiled weight, RMSNorms with bfloat16 scales)."""
     from ..kernels import ops
     from ..kernels.packing import TiledWeight
 
+    if not isinstance(x, PendingNorm):
+        return False
+    pn, nn = x.post_norm, x.next_norm
+    return (x.dtype == torch.bfloat16 and nn is not None and getattr(nn, "fusable_rms", False)
+            and nn.scale.dtype == torch.bfloat16
+            and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
+            and isinstance(w, TiledWeight) and w.rows <= 16 * 2048   # every workgroup redoes the norms
+            and ops.gemm_normed_takes(x.residual.shape[0], w)
+            and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
+
+
+def pending_product(x: PendingNorm, run) -> torch.Tensor:
+    """Runs `run(y, h_in, h_out, **norm arguments)` (ops.gemm_normed or a relative of it) for a pending norm that
+    `pending_fits_product`, and settles `x` with the residual that the kernel wrote."""
+    pn, nn = x.post_norm, x.next_norm
+    h_out = torch.empty_like(x.residual) if x.y is not None else None
+    out = run(x.y, x.residual, h_out,
+              post_weight=pn.scale if (pn is not None and x.y is not None) else None,
+              post_eps=pn.eps if pn is not None else 0.0, post_plus_one=pn.scale_plus_one if pn is not None else True,
+              next_weight=nn.scale, next_eps=nn.eps, next_plus_one=nn.scale_plus_one)
+    if x.y is not None:
+        x.residual, x.y = h_out, None
+    return out
+
+
+def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x . w^T (gated if w is a paired tiled weight) for activations x or a `PendingNorm`.  A pending norm is done
+    inside the product's kernel when that kernel takes the sizes; otherwise it is materialized first."""
+    import functools
+
+    from ..kernels import ops
+
     if isinstance(x, PendingNorm):
-        pn, nn = x.post_norm, x.next_norm
-        fusable = (x.dtype == torch.bfloat16 and nn is not None and getattr(nn, "fusable_rms", False)
-                   and nn.scale.dtype == torch.bfloat16
-                   and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
-                   and isinstance(w, TiledWeight) and w.rows <= 16 * 2048   # every workgroup redoes the norms
-                   and ops.gemm_normed_takes(x.residual.shape[0], w)
-                   and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
-        if fusable:
-            h_out = torch.empty_like(x.residual) if x.y is not None else None
-            out = ops.gemm_normed(
-                x.y, x.residual, h_out, w,
-                post_weight=pn.scale if (pn is not None and x.y is not None) else None,
-                post_eps=pn.eps if pn is not None else 0.0, post_plus_one=pn.scale_plus_one if pn is not None else True,
-                next_weight=nn.scale, next_eps=nn.eps, next_plus_one=nn.scale_plus_one, soft_cap=soft_cap,
-                out_dtype=out_dtype or x.dtype)
-            if x.y is not None:
-                x.residual, x.y = h_out, None
-            return out
+        if pending_fits_product(x, w):
+            return pending_product(x, functools.partial(ops.gemm_normed, w=w, soft_cap=soft_cap,
+                                                        out_dtype=out_dtype or x.dtype))
         x = x.materialize()
     return ops.gemm(x, w, soft_cap=soft_cap, out_dtype=out_dtype)
 

@@ -50,7 +50,7 @@ def test_rmsnorm(dtype, T, D):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304), (40, 2304), (33, 100), (35, 5000), (32, 6000), (37, 50)])
+@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304), (600, 2304), (513, 100), (515, 5000), (512, 6000), (517, 50)])
 def test_add_rmsnorm(dtype, T, D):
     from simply_amd.kernels import ops
     y = rand((T, D), dtype, 3, 2.0)
@@ -71,12 +71,12 @@ def test_add_rmsnorm(dtype, T, D):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("H,K,hd,P", [(4, 2, 16, 4), (6, 1, 32, 3), (8, 4, 256, 16), (3, 3, 48, 5)])
-@pytest.mark.parametrize("T", [11, 44])   # few tokens: a block per (token, head); many: a block per token
+@pytest.mark.parametrize("T", [11, 300])   # few tokens: a block per (token, head); many: a block per token
 def test_rope_cache_write(dtype, H, K, hd, P, T):
     from simply_amd.kernels import ops
     pages = -(-T // P) + 6
     qkv = rand((T, (H + 2 * K) * hd), dtype, 7)
-    positions = torch.tensor(([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7] * 4)[:T], dtype=torch.int32).cuda()
+    positions = torch.tensor(([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7] * 28)[:T], dtype=torch.int32).cuda()
     ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda()
     slots = torch.randperm(pages * P)[:T].to(torch.int64).cuda()
     kp, vp = torch.zeros((pages, K, P, hd), dtype=dtype).cuda(), torch.zeros((pages, K, hd, P), dtype=dtype).cuda()
@@ -551,3 +551,40 @@ def test_bfloat16_rounding_of_the_kernels():
     nan = torch.isnan(x)
     assert torch.equal(torch.isnan(got.float()), nan)
     assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan])
+
+
+@pytest.mark.parametrize("M", [1, 8, 13])
+@pytest.mark.parametrize("H,Kh,hd,P,K", [(8, 4, 256, 16, 2304), (4, 2, 64, 16, 128), (3, 1, 32, 48, 96), (2, 2, 128, 32, 2560)])
+@pytest.mark.parametrize("rotate", [True, False])
+def test_gemm_normed_rotary(M, H, Kh, hd, P, K, rotate):
+    """Norms, q/k/v projection, rotation, query scale and cache write in one kernel against the same from the
+    separate kernels (residual sum and norms in the projection, then the rotary kernel)."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_tiles
+    N = (H + 2 * Kh) * hd
+    y, h = rand((M, K), torch.bfloat16, 110, 2.0), rand((M, K), torch.float32, 111, 4.0)
+    wp, wn = rand((K,), torch.bfloat16, 112, 0.3), rand((K,), torch.bfloat16, 113, 0.3)
+    tw = pack_tiles(rand((N, K), torch.bfloat16, 114, 0.05))
+    positions = torch.tensor([0, 1, 5, 100, 8000, 33, 7, 2, 4095, 4096, 9, 10, 11][:M], dtype=torch.int32).cuda()
+    ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda() if rotate else None
+    pages = 5
+    slots = torch.randperm(pages * P)[:M].to(torch.int64).cuda()
+    norm = dict(post_weight=wp, post_eps=1e-6, post_plus_one=True, next_weight=wn, next_eps=1e-5, next_plus_one=True)
+    for with_y in (True, False):
+        kp, vp = torch.zeros((pages, Kh, P, hd), dtype=torch.bfloat16).cuda(), torch.zeros((pages, Kh, hd, P), dtype=torch.bfloat16).cuda()
+        kp2, vp2 = kp.clone(), vp.clone()
+        h_out, h_out2 = torch.full_like(h, 7.0), torch.full_like(h, 7.0)
+        got = ops.gemm_normed_rotary(y if with_y else None, h, h_out if with_y else None, tw, **norm, positions=positions,
+                                     timescale=ts, scale_factor=1.0, query_scale=12.0, num_heads=H, num_kv_heads=Kh,
+                                     head_dim=hd, slot_mapping=slots, k_pages=kp, v_pages=vp)
+        want = ops.gemm_normed(y if with_y else None, h, h_out2 if with_y else None, tw, **norm)
+        ops.rope_cache_write(want, positions, ts, 1.0, 12.0, H, Kh, hd, slots, kp2, vp2)
+        t = dict(rtol=1e-2, atol=1e-3)   # the same sums; the rotation's products may round one bfloat16 step apart
+        torch.testing.assert_close(got[:, :H * hd].float(), want[:, :H * hd].float(), **t)
+        torch.testing.assert_close(kp.float(), kp2.float(), **t)
+        assert torch.equal(vp, vp2)
+        assert torch.equal(h_out, h_out2)
+    # without pages only the queries are produced
+    got = ops.gemm_normed_rotary(None, h, None, tw, **norm, positions=positions, timescale=ts, scale_factor=1.0,
+                                 query_scale=12.0, num_heads=H, num_kv_heads=Kh, head_dim=hd)
+    torch.testing.assert_close(got[:, :H * hd].float(), want[:, :H * hd].float(), rtol=1e-2, atol=1e-3)
