@@ -25,10 +25,6 @@ constexpr int kWaves = 8;
 constexpr int kUnroll = 4;
 constexpr int kMaxGroups = 256;  // one workgroup per compute unit; each takes the same number of tiles, or one fewer
 
-__device__ inline float gelu_tanh_f(float x) {
-  const float k = 0.7978845608028654f;
-  return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
-}
 __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
 // What the rotary epilogue (EPI 3) needs: the product is the fused q/k/v projection of an attention layer, columns
@@ -260,7 +256,7 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
           sum[p] = t;
         }
         float v = sum[0];
-        if (EPI == 1) v = gelu_tanh_f(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
+        if (EPI == 1) v = gelu_tanh_fast(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
         else if (EPI == 2) v = cap * tanhf(v / cap);
         store_f(C, c_dtype, static_cast<size_t>(ml) * ldc + n, v);
       }

@@ -21,11 +21,6 @@ namespace sa {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
-__device__ inline float gelu_tanh_f(float x) {
-  const float k = 0.7978845608028654f;
-  return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
-}
-
 __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
 constexpr int kUnroll = 4;
@@ -128,7 +123,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
     float v = sum[0];
     if (EPI == 1) {
       // both products are rounded to bfloat16 first, as separate matrix products would be
-      v = gelu_tanh_f(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
+      v = gelu_tanh_fast(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
     } else if (EPI == 2) {
       v = cap * tanhf(v / cap);
     }

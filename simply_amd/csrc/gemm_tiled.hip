@@ -26,11 +26,6 @@ namespace tiled {
 constexpr int BK = 64;          // columns of A per LDS slab
 constexpr int PITCH = BK + 8;   // elements per LDS row: 144 bytes
 
-__device__ inline float gelu_tanh_f(float x) {
-  const float k = 0.7978845608028654f;
-  return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
-}
-
 // WAVES_N: 2 = waves as 2 x 2 (BM = 2 * WM * 16 rows, 128 columns of W tiles); 4 = waves as 1 x 4 (BM = WM * 16 rows,
 // 256 columns: for few rows, every W fragment is loaded by one wave only).  gridDim.z > 1 cuts K over workgroups:
 // each writes its float32 partial tile to `partials` [z][M][NW] and gemm_reduce_kernel adds them up.
@@ -39,7 +34,8 @@ __device__ inline float gelu_tanh_f(float x) {
 // rows 16 i .. of the gate, tile 2 i + 1: the same rows of the other factor; pack_gate_up in the Python package):
 // a wave's four tiles are two output tiles, and gate and factor meet in the same lane's registers.  NW is the
 // number of weight rows (2 N for the gated epilogue, else N).
-template <int WM, int EPI, int WAVES_N>
+// TAIL: K is no multiple of the slab, so the loads carry tests against K.
+template <int WM, int EPI, int WAVES_N, bool TAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __restrict__ W, void* __restrict__ C,
                        int c_dtype, int64_t ldc, int M, int N, int K, int chunks, float cap,
@@ -67,16 +63,22 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
     for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // ---- A: global -> registers -> LDS.  Piece q of this thread: row (tid / 8) + 32 q, columns (tid % 8) * 8 .. + 8.
+  // Rows beyond M read row M - 1 instead (their products are never stored), so that the loop carries no row test;
+  // what depends on the thread alone (row offsets) is computed once, the slab's offset is the same for all.
   const int a_row = tid / 8, a_kg = tid % 8;
   bf16x8 areg[APT];
   const bf16x8 zero = {};
-  auto load_a = [&](int stage) {
-    const int k = stage * BK + a_kg * 8;
+  uint32_t a_off[APT];  // elements; the host checks that M * lda fits
 #pragma unroll
-    for (int q = 0; q < APT; ++q) {
-      const int m = m_base + a_row + 32 * q;
-      areg[q] = (m < M && k < K) ? *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(m) * lda + k) : zero;
-    }
+  for (int q = 0; q < APT; ++q) {
+    const int m = m_base + a_row + 32 * q;
+    a_off[q] = static_cast<uint32_t>(m < M ? m : M - 1) * static_cast<uint32_t>(lda) + a_kg * 8;
+  }
+  auto load_a = [&](int stage) {
+    const bf16* slab = A + static_cast<size_t>(stage) * BK;  // the same for the whole workgroup
+    const bool in_k = !TAIL || stage * BK + a_kg * 8 < K;
+#pragma unroll
+    for (int q = 0; q < APT; ++q) areg[q] = in_k ? *reinterpret_cast<const bf16x8*>(slab + a_off[q]) : zero;
   };
   auto store_a = [&](int buf) {
 #pragma unroll
@@ -85,18 +87,25 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
   };
 
   // ---- W fragments of a whole slab (two steps of 32): tile nt, chunk c is the KiB at ((nt * chunks + c) * 512)
-  // elements, this lane's 16 bytes at lane * 8.  They are requested one slab ahead.
+  // elements, this lane's 16 bytes at lane * 8.  They are requested one slab ahead.  Tiles beyond the last read the
+  // last tile instead (their products are never stored).
   bf16x8 wreg[2][2][4];
+  const bf16* wtile[4];  // the same for the whole wave
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int nt = __builtin_amdgcn_readfirstlane(nt0 + j < ntiles ? nt0 + j : ntiles - 1);
+    wtile[j] = W + static_cast<size_t>(nt) * chunks * 512;
+  }
   auto load_w = [&](int buf, int stage) {
 #pragma unroll
-    for (int kc = 0; kc < 2; ++kc)
+    for (int kc = 0; kc < 2; ++kc) {
+      const int chunk = stage * 2 + kc;
+      const bool in_k = !TAIL || chunk < chunks;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int nt = nt0 + j, chunk = stage * 2 + kc;
-        const bool ok = nt < ntiles && chunk < chunks;
-        const size_t off = (static_cast<size_t>(ok ? nt : 0) * chunks + (ok ? chunk : 0)) * 512 + lane * 8;
-        wreg[buf][kc][j] = ok ? *reinterpret_cast<const bf16x8*>(W + off) : zero;
-      }
+      for (int j = 0; j < 4; ++j)
+        wreg[buf][kc][j] =
+            in_k ? *reinterpret_cast<const bf16x8*>(wtile[j] + static_cast<size_t>(chunk) * 512 + lane * 8) : zero;
+    }
   };
   auto multiply = [&](int wbuf, int abuf) {
 #pragma unroll
@@ -129,14 +138,14 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
   for (int s = s0; s < s1; s += 2) {
     // slab s: LDS buffer 0, W registers 0
     if (s + 2 < s1) load_a(s + 2);
-    load_w(1, s + 1);
+    if (s + 1 < s1) load_w(1, s + 1);
     multiply(0, 0);
     __syncthreads();                       // all waves are done with LDS buffer 0
     if (s + 2 < s1) store_a(0);
     if (s + 1 >= s1) break;
     // slab s + 1: LDS buffer 1, W registers 1
     if (s + 3 < s1) load_a(s + 3);
-    load_w(0, s + 2);
+    if (s + 2 < s1) load_w(0, s + 2);
     multiply(1, 1);
     __syncthreads();                       // all waves are done with LDS buffer 1; buffer 0 is complete
     if (s + 3 < s1) store_a(1);
@@ -170,7 +179,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
         const int n = EPI == 1 ? (nt0 / 2 + j) * 16 + r : (nt0 + j) * 16 + r;
         if (n >= N) continue;
         float x;
-        if (EPI == 1) x = gelu_tanh_f(to_float(float_to_bf16(acc[i][2 * j][v]))) * to_float(float_to_bf16(acc[i][2 * j + 1][v]));
+        if (EPI == 1) x = gelu_tanh_fast(to_float(float_to_bf16(acc[i][2 * j][v]))) * to_float(float_to_bf16(acc[i][2 * j + 1][v]));
         else if (EPI == 2) x = cap * tanhf(acc[i][j][v] / cap);
         else x = acc[i][j][v];
         store_f(C, c_dtype, static_cast<size_t>(m) * ldc + n, x);
@@ -194,7 +203,7 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partials, int KS, v
       x += partials[z * plane + m * NW + col];
       if (EPI == 1) y += partials[z * plane + m * NW + col + 16];
     }
-    if (EPI == 1) x = gelu_tanh_f(to_float(float_to_bf16(x))) * to_float(float_to_bf16(y));
+    if (EPI == 1) x = gelu_tanh_fast(to_float(float_to_bf16(x))) * to_float(float_to_bf16(y));
     else if (EPI == 2) x = cap * tanhf(x / cap);
     store_f(C, c_dtype, m * ldc + n, x);
   }
@@ -206,8 +215,12 @@ static void launch(const bf16* A, int64_t lda, const bf16* W, void* C, int c_dty
   constexpr int BM = (4 / WAVES_N) * WM * 16, BNW = WAVES_N * 64;
   const int NW = EPI == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM, ks);
-  gemm_tiled_kernel<WM, EPI, WAVES_N><<<grid, 256, 0, stream>>>(A, lda, W, C, c_dtype, ldc, M, N, K, (K + 31) / 32, cap,
-                                                                partials);
+  if (K % BK == 0)
+    gemm_tiled_kernel<WM, EPI, WAVES_N, false><<<grid, 256, 0, stream>>>(A, lda, W, C, c_dtype, ldc, M, N, K, (K + 31) / 32,
+                                                                         cap, partials);
+  else
+    gemm_tiled_kernel<WM, EPI, WAVES_N, true><<<grid, 256, 0, stream>>>(A, lda, W, C, c_dtype, ldc, M, N, K, (K + 31) / 32,
+                                                                        cap, partials);
   if (ks > 1) {
     const size_t total = static_cast<size_t>(M) * N;
     const int blocks = static_cast<int>((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
@@ -219,7 +232,8 @@ static void launch(const bf16* A, int64_t lda, const bf16* W, void* C, int c_dty
 
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed) {
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-  return packed && W2 == nullptr && M >= 1 && K % 8 == 0 && lda % 8 == 0 && aligned(A) && aligned(W);
+  return packed && W2 == nullptr && M >= 1 && K % 8 == 0 && lda % 8 == 0 && aligned(A) && aligned(W) &&
+         static_cast<int64_t>(M) * lda < (int64_t{1} << 32);  // row offsets are kept in 32 bits
 }
 
 // ksplit > 0 fixes the number of cuts of K.
