@@ -284,7 +284,8 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
         raise KernelError("gemm: bad output shape")
     ldc = _rows(out, "gemm: out")
     if (algo == ALGO_AUTO and packed and w.row_major is not None and epi == EPILOGUE_NONE and out.dtype == a.dtype
-            and 0 < _library_gemm_min_rows <= M):
+            and 0 < _library_gemm_min_rows <= M and not torch.cuda.is_current_stream_capturing()):
+        # (not while a graph is recorded: the library may allocate a workspace)
         return torch.matmul(a, w.row_major.t(), out=out)
     ws = _workspace(a.device)
     _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(wd), _ptr(w2d), _code(wd), _ptr(out), _code(out), ldc, M, N, K, epi,

@@ -47,3 +47,39 @@ def test_real_layer_shapes(tmp_path, gpu_lib, shape, dtype, tol):
         assert torch.isfinite(got).all()
         err = (got - want).abs().max().item() / scale
         assert err <= tol, (cuts, err)
+
+
+@pytest.mark.parametrize("library_rows", [256, 0])
+def test_long_portions(tmp_path, gpu_lib, library_rows):
+    """Portions of several hundred tokens at the 2B layer sizes: the kernels for many rows (the library's or the
+    tiled product, the residual/norm and rotary kernels with a wave per row and a block per token, attention with
+    64 query rows per workgroup over a history and a window), against the plain implementation."""
+    from simply_amd.kernels import ops
+    d = dict(architectures=["Gemma2ForCausalLM"], num_hidden_layers=2, vocab_size=2000, rms_norm_eps=1e-6,
+             rope_theta=10000.0, sliding_window=200, attn_logit_softcapping=50.0, final_logit_softcapping=30.0,
+             max_position_embeddings=8192, initializer_range=0.02, **SHAPES["2b"])
+    folder = write_random_model(config_from_dict(d), str(tmp_path / "m"), 6, torch.bfloat16, norm_std=0.1)
+    w, cfg = plain.load(folder)
+    tokens = tiny.random_tokens(700, 2000, 12)
+    want = plain.forward(w, cfg, tokens, torch.float64)
+    ecfg = EngineConfig(activation_dtype="bfloat16", page_size=16, batch_size=2, max_seq_len=704, max_num_issue_tokens=704,
+                        total_num_pages=48, device="cuda:0", use_graphs=False, poison_freed_pages=True)
+    before = ops.library_gemm_min_rows()
+    ops.set_library_gemm_min_rows(library_rows)
+    try:
+        model, _ = load_model(folder, ecfg.dtype, "cuda:0")
+        ex = Executor(model, ecfg)
+        scale = want.abs().max().item()
+        for cuts in ([700], [600, 98, 2]):
+            ex.add_request("r")
+            out, i = [], 0
+            for c in cuts:
+                out.append(ex.step([StepEntry("r", tokens[i:i + c], list(range(c)))]).cpu())
+                i += c
+            ex.finish_request("r")
+            got = torch.cat(out).double()
+            assert torch.isfinite(got).all()
+            err = (got - want).abs().max().item() / scale
+            assert err <= 3e-2, (cuts, err)
+    finally:
+        ops.set_library_gemm_min_rows(before)
