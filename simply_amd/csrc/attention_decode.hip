@@ -357,11 +357,58 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   return 0;
 }
 
+// The same for units with many rows (portions of prompts): one workgroup per (unit, head) takes all 16 rows, 16
+// threads per row, each with its share of the output dimensions in pieces of four.
+__global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const float* __restrict__ workspace, int KS,
+                                                                         int HD, const SeqMeta* __restrict__ seq_meta,
+                                                                         int seq_begin, bf16* __restrict__ out,
+                                                                         int64_t out_stride, int Kh, int G) {
+  const int tid = threadIdx.x, kh = blockIdx.x, z = blockIdx.y;
+  const SeqMeta sm = seq_meta[seq_begin + z];
+  const int orow = tid / 16, part = tid % 16;
+  if (orow >= G * sm.q_len) return;
+  const size_t row_words = HD + 2;
+  const size_t unit = static_cast<size_t>(z) * Kh + kh;
+  const float* base = workspace + (unit * KS * 16 + orow) * row_words;
+  const size_t stride = 16 * row_words;
+  float Mg = -INFINITY;
+  for (int y = 0; y < KS; ++y) Mg = fmaxf(Mg, base[y * stride + HD]);
+  float Lg = 0.f;
+  for (int y = 0; y < KS; ++y) {
+    const float my = base[y * stride + HD];
+    Lg += my == -INFINITY ? 0.f : base[y * stride + HD + 1] * __expf(my - Mg);
+  }
+  const float inv = 1.f / Lg;
+  const int oq = orow / G, og = orow % G;
+  bf16* op = out + static_cast<size_t>(sm.q_start + oq) * out_stride + static_cast<size_t>(kh * G + og) * HD;
+  for (int d = part * 4; d < HD; d += 64) {
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int y = 0; y < KS; ++y) {
+      const float my = base[y * stride + HD];
+      const float wy = my == -INFINITY ? 0.f : __expf(my - Mg);
+      // rows are HD + 2 words long: a piece of four is 8-byte aligned
+      const float2 lo = *reinterpret_cast<const float2*>(base + y * stride + d);
+      const float2 hi = *reinterpret_cast<const float2*>(base + y * stride + d + 2);
+      o[0] += lo.x * wy;
+      o[1] += lo.y * wy;
+      o[2] += hi.x * wy;
+      o[3] += hi.y * wy;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) op[d + e] = float_to_bf16(o[e] * inv);
+  }
+}
+
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
                            int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
                            hipStream_t stream) {
-  // one workgroup per row: rows beyond the longest unit's are not launched
   const int max_rows = G * max_q_len < 16 ? G * max_q_len : 16;
+  if (max_rows > 4 && num_ranges <= 4) {
+    paged_attention_merge_rows_kernel<<<dim3(Kh, unit_count), 256, 0, stream>>>(workspace, num_ranges, hd, units,
+                                                                               unit_begin, out, out_stride, Kh, G);
+    return check_launch("paged_attention_merge_rows");
+  }
+  // one workgroup per row: rows beyond the longest unit's are not launched
   paged_attention_merge_kernel<<<dim3(Kh, unit_count, max_rows), 256, 0, stream>>>(workspace, num_ranges, hd, units, unit_begin,
                                                                             out, out_stride, Kh, G);
   return check_launch("paged_attention_merge");
