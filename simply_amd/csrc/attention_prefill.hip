@@ -131,29 +131,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const float c1 = CAP ? 2.f * kLog2e / soft_cap : kLog2e;
   const float c2 = soft_cap * kLog2e;
 
-  // Chunk c = wave + 4 * i of a tile's keys is the KiB (sub-tile t = c / NDC, dimensions 32 * (c % NDC) ..): 64 lanes
-  // x 16 bytes, contiguous in the page and in LDS.  Chunk c of its values is dimensions 32 * (c % NDC) .. + 31 of
-  // sub-tile t, 32 bytes (16 keys) each: a lane takes 8 keys of one dimension.  A wave's chunks lie in at most
-  // NT sub-tiles (one if the head has 64 dimensions, else both); what depends on the lane is computed once.
-  constexpr int NT = CPW < 2 ? 1 : 2;      // sub-tiles this wave reads from
-  constexpr int CPT = CPW / NT;            // chunks per sub-tile
-  uint32_t k_off[CPW], v_off[CPW], lds_off[CPW];  // in elements
+  // How a tile of 32 keys lies in LDS.  The two score products of a tile do not take keys 0..15 and 16..31 but
+  //     product t, row i of its A operand  <->  key 8 * (i / 4) + 4 * t + i % 4   of the tile,
+  // so that a lane's eight scores (rows 4 * grp + v of both products) belong to the eight consecutive keys 8 * grp ..
+  // 8 * grp + 7: the value operand of the second product is then one 16-byte piece of a value page per lane.  Both
+  // operands lie in LDS in blocks of 64 lanes x 16 bytes in the order of the lanes that read them (no bank
+  // conflicts); it is the load into LDS that picks, lane by lane, the matching 16 bytes of the pages:
+  //   key block (t, dc), lane (kgrp, i):    sub-tile i / 8 of the tile, its key 8 * ((i / 4) % 2) + 4 * t + i % 4,
+  //                                         dimensions 32 * dc + 8 * kgrp .. + 7
+  //   value block db, lane (grp, r):        sub-tile grp / 2, keys 8 * (grp % 2) .. + 7 of dimension 16 * db + r
+  // A wave loads blocks c = wave + 4 * i of the keys' 2 * NDC blocks and of the values' 2 * NDC blocks.
+  uint32_t k_off[CPW], v_off[CPW], lds_off[CPW];  // in elements; what depends on the lane is computed once
+  const int k_sub = (lane % 16) / 8, v_sub = lane / 32;  // the sub-tile (page) that this lane's pieces come from
 #pragma unroll
   for (int i = 0; i < CPW; ++i) {
     const int c = wave + kWaves * i;
-    k_off[i] = (c % NDC) * 512 + lane * 8;
-    // lane -> (block of 16 dimensions lane / 32, keys 8h .. 8h + 7 with h = lane % 32 / 16, dimension lane % 16 of
-    // the block): in LDS a block is [h][dimension][8 keys], which the operand reads below take without bank conflicts
-    v_off[i] = ((c % NDC) * 32 + (lane / 32) * 16 + lane % 16) * page_size + ((lane % 32) / 16) * 8;
+    const int t = c / NDC, dc = c % NDC, row = lane % 16;
+    k_off[i] = dc * 512 + ((lane / 16) * 16 + 8 * ((row / 4) % 2) + 4 * t + row % 4) * 8;
+    v_off[i] = (c * 16 + lane % 16) * page_size + ((lane / 16) % 2) * 8;
     lds_off[i] = __builtin_amdgcn_readfirstlane(c * 512);
   }
-  const int t_first = __builtin_amdgcn_readfirstlane(wave / NDC);  // sub-tile of chunk 0 (1 only for waves 2, 3 of NDC 2)
-  // Where sub-tile n of this wave lies for the tile asked for next: block blk[n] of the table, key off[n] of its
+  // Where the tile's two sub-tiles lie for the tile asked for next: block blk[n] of the table, key off[n] of its
   // page; kept by stepping, without divisions.  All of it is the same for the whole wave: scalar registers.
-  int blk[NT], off[NT];
+  int blk[2], off[2];
 #pragma unroll
-  for (int n = 0; n < NT; ++n) {
-    const int sk0 = tb * kTile + (t_first + n) * 16;
+  for (int n = 0; n < 2; ++n) {
+    const int sk0 = tb * kTile + n * 16;
     blk[n] = __builtin_amdgcn_readfirstlane(sk0 / page_size);
     off[n] = __builtin_amdgcn_readfirstlane(sk0 % page_size);
   }
@@ -162,24 +165,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const bf16* const v_head = v_pages + static_cast<int64_t>(kh) * page_size * HD;
   // sub-tiles (of 16 keys) with a page that this workgroup may read: [sub_lo, sub_hi)
   const int sub_lo = lo_g / 16, sub_hi = min((hi_g + 15) / 16, te * 2);
-  // Asks for this wave's chunks of `tile` (called for consecutive tiles) into a buffer.  A sub-tile without a page
+  // Asks for this wave's blocks of `tile` (called for consecutive tiles) into a buffer.  A sub-tile without a page
   // (beyond the keys, or given back by a windowed layer) reads page 0; its values are dropped when they are used.
   auto request = [&](int tile, __bf16* stage) __attribute__((always_inline)) {
+    const bf16* kb[2];
+    const bf16* vb[2];
 #pragma unroll
-    for (int n = 0; n < NT; ++n) {
-      const int sub = tile * 2 + t_first + n;
+    for (int n = 0; n < 2; ++n) {
+      const int sub = tile * 2 + n;
       const uint32_t page = (sub >= sub_lo && sub < sub_hi) ? static_cast<uint32_t>(table[blk[n]]) : 0u;
       const uint64_t at = static_cast<uint64_t>(page) * page_stride;
-      const bf16* const kb = k_head + at + static_cast<uint32_t>(off[n] >> 4) * (NDC * 512);
-      const bf16* const vb = v_head + at + static_cast<uint32_t>(off[n]);
-#pragma unroll
-      for (int m = 0; m < CPT; ++m) {
-        const int i = n * CPT + m;
-        __bf16* const k_to = stage + lds_off[i];
-        __bf16* const v_to = k_to + HALF;
-        load_to_lds(kb + k_off[i], k_to);
-        load_to_lds(vb + v_off[i], v_to);
-      }
+      kb[n] = k_head + at + static_cast<uint32_t>(off[n] >> 4) * (NDC * 512);
+      vb[n] = v_head + at + static_cast<uint32_t>(off[n]);
       off[n] += kTile;
 #pragma unroll
       for (int twice = 0; twice < 2; ++twice)
@@ -187,6 +184,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
           off[n] -= page_size;
           ++blk[n];
         }
+    }
+    const bf16* const k_from = k_sub ? kb[1] : kb[0];
+    const bf16* const v_from = v_sub ? vb[1] : vb[0];
+#pragma unroll
+    for (int i = 0; i < CPW; ++i) {
+      __bf16* const k_to = stage + lds_off[i];
+      __bf16* const v_to = k_to + HALF;
+      load_to_lds(k_from + k_off[i], k_to);
+      load_to_lds(v_from + v_off[i], v_to);
     }
   };
 
@@ -242,7 +248,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            const int key = key0 + t * 16 + grp * 4 + v;
+            const int key = key0 + grp * 8 + t * 4 + v;
             y[t][v] = (row_ok[j] && key <= pos_r[j] && key >= lo_r[j]) ? y[t][v] : -INFINITY;
           }
       }
@@ -277,7 +283,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[j][db][v] *= alpha[j];
     }
-    // Lane (d = r, grp) of the value operand holds V^T[db * 16 + r][keys 4 * grp .. + 3 of each sub-tile].  Values of
+    // Lane (d = r, grp) of the value operand holds V^T[db * 16 + r][keys 8 * grp .. + 7 of the tile].  Values of
     // keys that no row may use (unwritten, given back, another request's) count as 0; their scores are masked
     // anyway.  That concerns the last tile of the keys and tiles at a window's lower edge.
     constexpr int VB = 4;  // output blocks per batch of value operands
@@ -286,18 +292,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     for (int db0 = 0; db0 < NDB; db0 += VB) {
       bf16x8 vf[VB];
 #pragma unroll
-      for (int b = 0; b < VB; ++b) {
-        const int at = (db0 + b) * 256 + (grp / 2) * 128 + r * 8 + (grp % 2) * 4;
-        const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(v_s + at);
-        const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(v_s + HD * 16 + at);
-        vf[b] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-      }
+      for (int b = 0; b < VB; ++b) vf[b] = *reinterpret_cast<const bf16x8*>(v_s + ((db0 + b) * 64 + lane) * 8);
       if (fix) {
 #pragma unroll
         for (int b = 0; b < VB; ++b)
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            const int key = key0 + (e / 4) * 16 + grp * 4 + (e % 4);
+            const int key = key0 + grp * 8 + e;
             if (key >= hi_g || key < lo_g) vf[b][e] = to_bf16_raw(0.f);
           }
       }
