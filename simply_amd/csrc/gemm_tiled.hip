@@ -199,9 +199,20 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partials, int KS, v
     const size_t m = e / N, n = e % N;
     const size_t col = EPI == 1 ? 32 * (n / 16) + n % 16 : n;
     float x = 0.f, y = 0.f;
-    for (int z = 0; z < KS; ++z) {
-      x += partials[z * plane + m * NW + col];
-      if (EPI == 1) y += partials[z * plane + m * NW + col + 16];
+    // eight planes at a time: their loads are in flight together, the sums keep the order of the planes
+    for (int z0 = 0; z0 < KS; z0 += 8) {
+      float px[8], py[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool ok = z0 + j < KS;
+        px[j] = ok ? partials[(z0 + j) * plane + m * NW + col] : 0.f;
+        py[j] = (EPI == 1 && ok) ? partials[(z0 + j) * plane + m * NW + col + 16] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        x += px[j];
+        y += py[j];
+      }
     }
     if (EPI == 1) x = gelu_tanh_fast(to_float(float_to_bf16(x))) * to_float(float_to_bf16(y));
     else if (EPI == 2) x = cap * tanhf(x / cap);
@@ -251,9 +262,11 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
   } else if (few) {
     // few rows: the product is bound by streaming W, so it needs a workgroup or two per CU even when N is small:
     // waves side by side (64 rows x 256 weight rows per workgroup), K cut over workgroups
+    // (measured at 64 rows: about 200 workgroups of at least four slabs each; more cuts cost more in the sum of
+    // the partial tiles than they gain)
     const int tiles = (NW + 255) / 256;
-    ks = (512 + tiles - 1) / tiles;
-    if (ks > stages / 2) ks = stages / 2;
+    ks = (200 + tiles / 2) / tiles;
+    if (ks > stages / 4) ks = stages / 4;
   }
   if (ks > stages) ks = stages;
   if (ks < 1) ks = 1;
