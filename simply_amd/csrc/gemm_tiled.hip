@@ -51,10 +51,31 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int r = lane % 16, grp = lane / 16;
-  const int m_base = blockIdx.y * BM;
+  // Which tile this workgroup takes.  Workgroups are handed to the eight XCDs in turn, each with an L2 of its own:
+  // the numbering is turned round so that an XCD gets a contiguous share of the tiles, and within it tiles go in
+  // columns eight wide, rows first: the 32 workgroups that an XCD runs at a time are a 4 x 8 patch that shares its
+  // rows of A and of W through that L2.
+  int bx = blockIdx.x, by = blockIdx.y;
+  {
+    const int nx = gridDim.x, ny = gridDim.y, total = nx * ny;
+    int l = bx + nx * by;
+    if (total % 8 == 0) l = (l % 8) * (total / 8) + l / 8;
+    constexpr int GX = 8;
+    const int full = nx / GX;
+    if (l < full * GX * ny) {
+      const int col = l / (GX * ny), rem = l % (GX * ny);
+      by = rem / GX;
+      bx = col * GX + rem % GX;
+    } else {
+      const int rem = l - full * GX * ny, width = nx % GX;
+      by = rem / width;
+      bx = full * GX + rem % width;
+    }
+  }
+  const int m_base = by * BM;
   const int NW = EPI == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const int ntiles = (NW + 15) / 16;
-  const int nt0 = blockIdx.x * (BNW / 16) + wn * 4;  // this wave's first 16-row tile of W
+  const int nt0 = bx * (BNW / 16) + wn * 4;  // this wave's first 16-row tile of W
 
   floatx4 acc[WM][4];
 #pragma unroll
