@@ -156,6 +156,22 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(
     for (int c = 0; c < NCH; ++c) ss += yv[c].x * yv[c].x + yv[c].y * yv[c].y + yv[c].z * yv[c].z + yv[c].w * yv[c].w;
     r = rsqrtf(wave_sum(ss) / static_cast<float>(D) + eps_post);
   }
+  // four scale factors at a time (one 8-byte load when they are bfloat16)
+  auto scales = [&](const void* w, int dtype, float plus, int d, float* out4) {
+    if (dtype == kBF16) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const bf16*>(w) + d);
+      out4[0] = __uint_as_float(raw.x << 16) + plus;
+      out4[1] = __uint_as_float(raw.x & 0xffff0000u) + plus;
+      out4[2] = __uint_as_float(raw.y << 16) + plus;
+      out4[3] = __uint_as_float(raw.y & 0xffff0000u) + plus;
+    } else {
+      const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(w) + d);
+      out4[0] = raw.x + plus;
+      out4[1] = raw.y + plus;
+      out4[2] = raw.z + plus;
+      out4[3] = raw.w + plus;
+    }
+  };
   float ss2 = 0.f;
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
@@ -163,9 +179,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(
     if (d >= D) continue;
     float* h = reinterpret_cast<float*>(&hv[c]);
     const float* v = reinterpret_cast<const float*>(&yv[c]);
+    float w4[4] = {1.f, 1.f, 1.f, 1.f};
+    if (w_post != nullptr) scales(w_post, w_post_dtype, plus_one_post, d, w4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      h[e] += w_post != nullptr ? v[e] * r * (load_f(w_post, w_post_dtype, d + e) + plus_one_post) : v[e];
+      h[e] += w_post != nullptr ? v[e] * r * w4[e] : v[e];
       ss2 += h[e] * h[e];
     }
     *reinterpret_cast<float4*>(residual + rb + d) = hv[c];
@@ -177,9 +195,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(
     const int d = c * 256 + lane * 4;
     if (d >= D) continue;
     const float* h = reinterpret_cast<const float*>(&hv[c]);
-    float o[4];
+    float w4[4], o[4];
+    scales(w_next, w_next_dtype, plus_one_next, d, w4);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = h[e] * r2 * (load_f(w_next, w_next_dtype, d + e) + plus_one_next);
+    for (int e = 0; e < 4; ++e) o[e] = h[e] * r2 * w4[e];
     if constexpr (sizeof(OT) == 4) {
       *reinterpret_cast<float4*>(out + rb + d) = float4{o[0], o[1], o[2], o[3]};
     } else {
@@ -373,7 +392,8 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
   // many rows (enough for two workgroups of four rows per compute unit): a wave per row
   const auto aligned16 = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   const int o_dtype = out != nullptr ? out_dtype : y_dtype;
-  if (T >= 512 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out)) {
+  if (T >= 512 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out) &&
+      aligned16(w_post) && aligned16(w_next)) {
     const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
     const int blocks = (T + 3) / 4;
 #define SA_ROWS(YT, OT, NCH)                                                                                      \
