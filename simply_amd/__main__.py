@@ -6,7 +6,7 @@ random     write a model folder with random weights from a config.json and a see
 
 Options of `generate` carry the names of simply/serving/common_flags.py:19-132 where the reference
 has the option (--batch_size, --activation_dtype, --max_seq_len, --max_decode_steps, --page_size,
---temperature, --top_k, --top_p, --max_num_issue_tokens, --ckpt_dir) and of
+--temperature, --top_k, --top_p, --max_num_issue_tokens, --intermediate_steps, --ckpt_dir) and of
 simply/eval/page_decode_eval.py (--seed); dashes are accepted for underscores.
 """
 from __future__ import annotations
@@ -56,6 +56,8 @@ def cmd_generate(argv) -> int:
     _flag(ap, "top_k", type=int, default=-1)
     _flag(ap, "top_p", type=float, default=1.0)
     _flag(ap, "max_num_issue_tokens", type=int, default=2048)
+    _flag(ap, "intermediate_steps", type=int, default=8,
+          help="decode steps that may run in a row on the device before the host looks at the tokens")
     _flag(ap, "seed", type=int, default=0)
     _flag(ap, "ignore_eos", action="store_true")
     args = ap.parse_args(argv)
@@ -64,7 +66,7 @@ def cmd_generate(argv) -> int:
 
     kw = dict(activation_dtype=args.activation_dtype, batch_size=args.batch_size, max_seq_len=args.max_seq_len,
               page_size=args.page_size, max_num_issue_tokens=args.max_num_issue_tokens,
-              total_num_pages=args.total_num_pages, seed=args.seed)
+              total_num_pages=args.total_num_pages, seed=args.seed, intermediate_steps=args.intermediate_steps)
     if args.ckpt_dir:
         lm = LMInterface(args.ckpt_dir, **kw)
     elif args.config and args.random_weights is not None:

@@ -42,6 +42,17 @@ int sa_gather_rows(const void* x, int x_dtype, const int* index, void* out, int 
 
 int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t stream);
 
+// Between two decode steps that run without the host in between (every request brings one token): records the tokens
+// and log-probabilities just drawn as row *step_counter of out_tokens / out_logprobs [max_steps, B], makes them the
+// next step's input tokens, adds one to every token's position, to every request's first position (seq_meta
+// [B, 4], column 3) and draw counter, and to *step_counter.  B <= 1024.
+int sa_decode_advance(int B, int* step_counter, const int* sampled_tokens, const float* sampled_logprobs,
+                      int* tokens_in, int* positions, int* seq_meta, int* draw_counters, int* out_tokens,
+                      float* out_logprobs, int max_steps, hipStream_t stream);
+// slot_mapping[b] = block_table[token_seq[b], positions[b] / page_size] * page_size + positions[b] % page_size
+int sa_decode_slots(int B, const int* positions, const int* token_seq, const int* block_table, int table_stride,
+                    int page_size, int64_t* slot_mapping, hipStream_t stream);
+
 // C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1: gelu_tanh(A.W^T) * (A.W2^T);
 // 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
 // few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel (2 and 3 refuse what they do not take).

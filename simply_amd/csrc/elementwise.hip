@@ -351,6 +351,42 @@ __global__ void fill_u32_kernel(uint32_t* __restrict__ p, uint32_t value, int64_
     p[i] = value;
 }
 
+// ------------------------------------------------------------------ decoding several steps without the host
+// After a decode step and its sampling: records what was drawn as step *step_counter of this run, makes the drawn
+// tokens the next step's input, and moves every request on by one position (its token's position, its
+// descriptor's first position, its draw counter).  One block; B <= 1024.
+__global__ void decode_advance_kernel(int B, int* __restrict__ step_counter, const int* __restrict__ sampled_tokens,
+                                      const float* __restrict__ sampled_logprobs, int* __restrict__ tokens_in,
+                                      int* __restrict__ positions, int* __restrict__ seq_meta,
+                                      int* __restrict__ draw_counters, int* __restrict__ out_tokens,
+                                      float* __restrict__ out_logprobs, int max_steps) {
+  const int b = threadIdx.x;
+  const int k = *step_counter;
+  __syncthreads();
+  if (b < B) {
+    if (k < max_steps) {
+      out_tokens[static_cast<size_t>(k) * B + b] = sampled_tokens[b];
+      out_logprobs[static_cast<size_t>(k) * B + b] = sampled_logprobs[b];
+    }
+    tokens_in[b] = sampled_tokens[b];
+    positions[b] += 1;
+    seq_meta[4 * b + 3] += 1;
+    draw_counters[b] += 1;
+  }
+  if (b == 0) *step_counter = k + 1;
+}
+
+// slot_mapping[b] = where the key of token b goes: page (from its request's block-table row) * page_size + offset
+__global__ void decode_slots_kernel(int B, const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                    const int* __restrict__ block_table, int table_stride, int page_size,
+                                    int64_t* __restrict__ slot_mapping) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  const int pos = positions[b];
+  const int page = block_table[static_cast<size_t>(token_seq[b]) * table_stride + pos / page_size];
+  slot_mapping[b] = static_cast<int64_t>(page) * page_size + pos % page_size;
+}
+
 static int row_threads(int D) {
   int t = 64;
   while (t < 1024 && t * 4 < D) t *= 2;
@@ -494,4 +530,26 @@ extern "C" int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t strea
   fill_u32_kernel<<<static_cast<int>(blocks > 4096 ? 4096 : blocks), 256, 0, stream>>>(static_cast<uint32_t*>(p),
                                                                                       value, n);
   return check_launch("fill_u32");
+}
+
+extern "C" int sa_decode_advance(int B, int* step_counter, const int* sampled_tokens, const float* sampled_logprobs,
+                                 int* tokens_in, int* positions, int* seq_meta, int* draw_counters, int* out_tokens,
+                                 float* out_logprobs, int max_steps, hipStream_t stream) {
+  if (B == 0) return 0;
+  SA_REQUIRE(B > 0 && B <= 1024 && max_steps > 0, "decode_advance: 1..1024 requests and a positive number of steps");
+  int threads = 64;
+  while (threads < B) threads *= 2;
+  decode_advance_kernel<<<1, threads, 0, stream>>>(B, step_counter, sampled_tokens, sampled_logprobs, tokens_in,
+                                                   positions, seq_meta, draw_counters, out_tokens, out_logprobs,
+                                                   max_steps);
+  return check_launch("decode_advance");
+}
+
+extern "C" int sa_decode_slots(int B, const int* positions, const int* token_seq, const int* block_table,
+                               int table_stride, int page_size, int64_t* slot_mapping, hipStream_t stream) {
+  if (B == 0) return 0;
+  SA_REQUIRE(B > 0 && table_stride > 0 && page_size > 0, "decode_slots: bad sizes");
+  decode_slots_kernel<<<(B + 63) / 64, 64, 0, stream>>>(B, positions, token_seq, block_table, table_stride, page_size,
+                                                        slot_mapping);
+  return check_launch("decode_slots");
 }

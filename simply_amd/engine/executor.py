@@ -54,9 +54,12 @@ class Executor:
         self._host = torch.empty(self._words, dtype=torch.int32, pin_memory=self._on_gpu)
         self._dev = torch.empty(self._words, dtype=torch.int32, device=self.device)
         self._copied = torch.cuda.Event() if self._on_gpu else None
-        # decode-only steps (one token per request) are captured once per number of requests and replayed
-        self._graphs: dict[int, tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        # decode-only steps (one token per request) are captured once per number of requests and order of magnitude
+        # of the context (the attention kernels choose their cut of the keys when they are recorded) and replayed
+        self._graphs: dict[tuple, tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._graph_pool = None
+        # several decode steps in a row without the host (decode_many): what was drawn in each, and the step count
+        self._records: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid: Hashable) -> int:
@@ -85,7 +88,8 @@ class Executor:
         with the same number of requests (tokens, positions, slots, block tables) lies in buffers at fixed
         addresses that the kernels read, so the launches can be recorded once.  The returned logits are
         overwritten by the next replay with as many requests."""
-        entry = self._graphs.get(T)
+        key = (T, self._context_bucket(ctx))
+        entry = self._graphs.get(key)
         if entry is None:
             # once eagerly (kernels compile their plans, scratch buffers get allocated; the step's writes to the
             # cache are the same when repeated), then record
@@ -97,14 +101,106 @@ class Executor:
             with torch.cuda.graph(graph, pool=self._graph_pool):
                 logits = self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
             entry = (graph, logits)
-            self._graphs[T] = entry
+            self._graphs[key] = entry
         entry[0].replay()
         return entry[1]
+
+    @staticmethod
+    def _context_bucket(ctx: StepContext) -> int:
+        return max(ctx.max_kv_len - 1, 0).bit_length()
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
         """Runs the entries as one batch.  Returns float32 logits [wanted, vocab] in the order of the
         entries and of their `want`, or None if nothing is wanted."""
+        prepared = self._prepare(entries)
+        if prepared is None:
+            return None
+        T, R, ctx, logit_rows, wants, num_entries = prepared
+        decode_only = (self._on_gpu and self.config.use_graphs and all(q == 1 for q in ctx.q_lens)
+                       and R == num_entries)
+        if decode_only:
+            logits = self._replay(T, ctx, logit_rows)
+        else:
+            logits = self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
+        for rid, start, q in wants:
+            self.num_computed[rid] = (self.cache.admission[rid], start + q)
+        return logits
+
+    def decode_many(self, entries: Sequence[StepEntry], num_steps: int, sampler) -> tuple[list[list[int]], list[list[float]]]:
+        """`num_steps` decode steps in a row for requests that bring one token each (after
+        `SamplingState.continue_decode`, simply/utils/ragged_paged_attention.py, which loops on the device for up
+        to `intermediate_steps`): every step's drawn tokens are the next step's input, on the device; the host
+        comes back in once, at the end.  `sampler` has been staged (`Sampler.stage`) with one row per entry, in
+        the entries' order.  Pages for all the steps are reserved first (`OutOfPages` if they do not fit).
+        Returns (tokens, log-probabilities), each [num_steps][entry]."""
+        entries = list(entries)
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            raise ValueError("decode_many: every request brings one token whose logits are wanted")
+        B = len(entries)
+        if not (self._on_gpu and self.config.use_graphs) or num_steps == 1:
+            # step by step through the host (no graphs: the CPU stand-in of the tests, or a single step)
+            tokens, logprobs = [], []
+            for k in range(num_steps):
+                logits = self.step(entries)
+                toks, lps = sampler.launch(logits)
+                tokens.append(toks[:B].tolist())
+                logprobs.append(lps[:B].tolist())
+                sampler.draw_counters[:B] += 1
+                entries = [StepEntry(e.request_id, [t], [0]) for e, t in zip(entries, tokens[-1])]
+            return tokens, logprobs
+        prepared = self._prepare(entries, reserve_ahead=num_steps)
+        T, R, ctx, logit_rows, wants, _ = prepared
+        assert T == B == R and ctx.request_ids == [e.request_id for e in entries]  # rows, tokens and entries line up
+        cap, dev = self._cap, self._dev
+        if self._records is None or self._records[0].numel() < num_steps * cap:
+            room = max(num_steps, 64)   # recorded graphs hold these addresses: made once for any usual run
+            self._records = (torch.empty(room * cap, dtype=torch.int32, device=self.device),
+                             torch.empty(room * cap, dtype=torch.float32, device=self.device),
+                             torch.zeros(1, dtype=torch.int32, device=self.device))
+            self._graphs = {k: v for k, v in self._graphs.items() if k[0] != "many"}  # they hold the old addresses
+        rec_tok, rec_lp, counter = self._records
+        max_steps = rec_tok.numel() // cap
+        out_tok, out_lp = rec_tok[:max_steps * B].view(max_steps, B), rec_lp[:max_steps * B].view(max_steps, B)
+        from ..kernels import ops
+
+        def one_step():
+            logits = self.model.forward(dev[:T], ctx, self.cache.views, logit_rows)
+            toks, lps = sampler.launch(logits)
+            ops.decode_advance(counter, toks, lps, dev[:T], dev[cap:cap + T], ctx.seq_meta, sampler.draw_counters,
+                               out_tok, out_lp)
+            for g in self.cache.groups:
+                ops.decode_slots(dev[cap:cap + T], dev[2 * cap:2 * cap + T], ctx.groups[g.group_id].block_table,
+                                 self.cache.page_size, ctx.groups[g.group_id].slot_mapping)
+
+        ops.fill_(counter, 0)
+        key = ("many", B, self._context_bucket(ctx), max_steps, id(sampler))
+        entry = self._graphs.get(key)
+        done = 0
+        if entry is None:
+            one_step()   # once eagerly (it counts as the first step), then recorded
+            done = 1
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                one_step()
+            entry = (graph, None)
+            self._graphs[key] = entry
+        for _ in range(done, num_steps):
+            entry[0].replay()
+        tokens = out_tok[:num_steps].tolist()      # waits for the steps
+        logprobs = out_lp[:num_steps].tolist()
+        for rid, start, _ in wants:
+            self.num_computed[rid] = (self.cache.admission[rid], start + num_steps)
+        return tokens, logprobs
+
+    def _prepare(self, entries: Sequence[StepEntry], reserve_ahead: int = 1):
+        """Checks the entries, reserves their pages (for `reserve_ahead` tokens where an entry brings one token
+        and more steps follow without the host), lays the step out in the staging buffer and copies it to the
+        device.  Returns (tokens, wanted rows, context, wanted-row indices on the device, [(request, start,
+        tokens reserved)], number of entries), or None for an empty step."""
         entries = [e for e in entries if len(e.tokens) > 0]
         T = sum(len(e.tokens) for e in entries)
         if T == 0:
@@ -119,8 +215,6 @@ class Executor:
             if e.request_id not in self.cache.requests:
                 raise KeyError(f"request {e.request_id!r} has not been admitted to the cache")
         cache, cap = self.cache, self._cap
-        # make room for every entry first: a failure leaves earlier steps' state untouched only if nothing
-        # has been reserved, so check all of them together before changing anything
         # forget what is known of requests that have left the cache since (finished or preempted elsewhere)
         for rid in [r for r in self.num_computed if r not in self.cache.requests]:
             del self.num_computed[rid]
@@ -129,7 +223,8 @@ class Executor:
         order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens))
         if len(entries) > self.config.batch_size:
             raise ValueError(f"{len(entries)} requests in one step, batch_size is {self.config.batch_size}")
-        wants = [(e.request_id, self._start_of(e), len(e.tokens)) for e in entries]
+        # make room for every entry first: nothing is reserved unless all of it fits
+        wants = [(e.request_id, self._start_of(e), max(len(e.tokens), reserve_ahead)) for e in entries]
         if not cache.can_reserve(wants):
             from ..cache import OutOfPages
 
@@ -148,7 +243,8 @@ class Executor:
         first_token = [0] * len(entries)
         t0 = 0
         for j, i in enumerate(order):
-            e, (rid, start, q) = entries[i], wants[i]
+            e, (rid, start, reserved) = entries[i], wants[i]
+            q = len(e.tokens)
             ids = np.asarray(e.tokens, dtype=np.int64)
             if ids.min() < 0 or ids.max() >= self.vocab_size:
                 raise ValueError(f"request {rid!r}: token id outside [0, {self.vocab_size})")
@@ -159,7 +255,7 @@ class Executor:
             meta[j] = (slot, t0, q, start)
             for g in cache.groups:
                 slot_maps[g.group_id][t0:t0 + q] = cache.slot_mapping(g.group_id, rid, start, q)
-                cache.check_readable(g.group_id, rid, start, q)
+                cache.check_readable(g.group_id, rid, start, reserved)
             first_token[i] = t0
             ctx_ids.append(rid); ctx_slots.append(slot); ctx_starts.append(start); ctx_q.append(q)
             t0 += q
@@ -185,11 +281,5 @@ class Executor:
                           groups=groups, request_ids=ctx_ids, seq_slots=ctx_slots, seq_starts=ctx_starts, q_lens=ctx_q,
                           cu_q_lens=cu)
         logit_rows = dev[3 * cap:3 * cap + R] if R else None
-        decode_only = self._on_gpu and self.config.use_graphs and all(q == 1 for q in ctx_q) and R == len(entries)
-        if decode_only:
-            logits = self._replay(T, ctx, logit_rows)
-        else:
-            logits = self.model.forward(dev[:T], ctx, cache.views, logit_rows)
-        for rid, start, q in wants:
-            self.num_computed[rid] = (cache.admission[rid], start + q)
-        return logits
+        return T, R, ctx, logit_rows, [(rid, start, len(e.tokens)) for (rid, start, _), e in zip(wants, entries)], \
+            len(entries)

@@ -16,7 +16,7 @@ from ..config import EngineConfig, load_config
 from ..sampling import Sampler, SamplingParams, request_seed
 from .executor import Executor, StepEntry
 from .loading import load_model, random_model
-from .scheduler import Request, Scheduler
+from .scheduler import Request, Scheduled, Scheduler, Status
 
 
 @dataclasses.dataclass(frozen=True)
@@ -54,7 +54,7 @@ class LMInterface:
                  activation_dtype: str = "bfloat16", batch_size: int = 8, max_seq_len: int | None = None,
                  page_size: int = 16, max_num_issue_tokens: int = 2048, total_num_pages: int | None = None,
                  seed: int = 0, device: str = "cuda:0", poison_freed_pages: bool = False, use_graphs: bool = True,
-                 library_gemm_min_rows: int | None = None, _model=None):
+                 library_gemm_min_rows: int | None = None, intermediate_steps: int = 8, _model=None):
         from ..kernels import lib
 
         lib.load()  # fails here, loudly, if the kernel library is missing and cannot be built
@@ -82,6 +82,9 @@ class LMInterface:
         self.scheduler = Scheduler(self.executor.cache, max_num_issue_tokens=self.engine_config.issue_budget,
                                    max_seq_len=max_seq_len)
         self.sampler = Sampler(device, max(batch_size, 1))
+        # decode steps that may run in a row on the device before the host looks at the tokens
+        # (simply/serving/common_flags.py:84 --intermediate_steps)
+        self.intermediate_steps = max(1, int(intermediate_steps))
         self.seed = int(seed)
         self._num_requests = 0
         self.stats = {"steps": 0, "tokens": 0, "preemptions": 0, "seconds": 0.0}
@@ -99,8 +102,10 @@ class LMInterface:
         self.scheduler.add(r)
         return r
 
-    def step(self) -> list[Request]:
-        """One scheduling decision and one run of the step function.  Returns the requests that finished."""
+    def step(self, max_decode_steps: int | None = None) -> list[Request]:
+        """One scheduling decision and one run of the step function; when every scheduled request is decoding and
+        nothing waits for admission, up to `intermediate_steps` (and `max_decode_steps`) decode steps in a row
+        without the host in between.  Returns the requests that finished."""
         out = self.scheduler.schedule()
         self.stats["preemptions"] += len(out.preempted)
         finished = list(out.finished)
@@ -110,6 +115,24 @@ class LMInterface:
         for s in out.scheduled:
             toks = s.request.all_token_ids[s.start:s.start + s.num_tokens]
             entries.append(StepEntry(s.request.request_id, toks, [s.num_tokens - 1] if s.samples else [], s.start))
+        n = self._decode_steps_ahead(out.scheduled, max_decode_steps)
+        if n > 1:
+            reqs = [s.request for s in out.scheduled]
+            self.sampler.stage([r.params for r in reqs], [r.seed for r in reqs], [len(r.output_token_ids) for r in reqs])
+            step_tokens, step_logprobs = self.executor.decode_many(entries, n, self.sampler)
+            live = list(out.scheduled)
+            for k in range(n):
+                index = {id(s): i for i, s in enumerate(out.scheduled)}
+                now = [Scheduled(s.request, s.start + k, 1, True) for s in live]
+                done = self.scheduler.update(now, [step_tokens[k][index[id(s)]] for s in live],
+                                             [step_logprobs[k][index[id(s)]] for s in live])
+                finished += done
+                live = [s for s in live if s.request.status is Status.RUNNING]
+                self.stats["steps"] += 1
+                self.stats["tokens"] += len(now)
+                if not live:
+                    break
+            return finished
         logits = self.executor.step(entries)
         tokens: list = [None] * len(entries)
         logprobs: list = [None] * len(entries)
@@ -124,6 +147,21 @@ class LMInterface:
         self.stats["steps"] += 1
         self.stats["tokens"] += out.num_tokens
         return finished
+
+    def _decode_steps_ahead(self, scheduled, max_decode_steps: int | None) -> int:
+        """How many decode steps may run in a row now: more than one only if every scheduled request decodes, nothing
+        waits, none of them would pass its own limits, and the free pages hold all of it."""
+        n = self.intermediate_steps if max_decode_steps is None else min(self.intermediate_steps, max_decode_steps)
+        if n <= 1 or self.scheduler.waiting or any(s.num_tokens != 1 or not s.samples for s in scheduled):
+            return 1
+        if len(scheduled) != len(self.scheduler.running):
+            return 1   # someone is still in its prompt
+        for s in scheduled:
+            r = s.request
+            n = min(n, r.params.max_decode_steps - len(r.output_token_ids), self.scheduler._limit(r) - r.num_tokens)
+        while n > 1 and not self.executor.cache.can_reserve([(s.request.request_id, s.start, n) for s in scheduled]):
+            n //= 2
+        return max(n, 1)
 
     # ------------------------------------------------------------------ generate
     def generate(self, input_token_ids: Sequence[int] | Sequence[Sequence[int]], prng_key: int | None = None,

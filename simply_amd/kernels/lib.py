@@ -30,6 +30,8 @@ _SIGNATURES = {
     "sa_rope": [_P, _I, _L, _P, _P, _F, _F, _I, _I, _I, _P],
     "sa_gather_rows": [_P, _I, _P, _P, _I, _I, _I, _P],
     "sa_fill_u32": [_P, c_uint32, _L, _P],
+    "sa_decode_advance": [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P],
+    "sa_decode_slots": [_I, _P, _P, _P, _I, _I, _P, _P],
     "sa_gemm": [_P, _I, _L, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P],
     "sa_paged_attention": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "sa_paged_attention_decode": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L,

@@ -212,6 +212,48 @@ def fill_(t: torch.Tensor, value_bits: int = 0) -> None:
     _lib.call("sa_fill_u32", _ptr(t), value_bits & 0xFFFFFFFF, nbytes // 4, _stream())
 
 
+def decode_advance(step_counter: torch.Tensor, sampled_tokens: torch.Tensor, sampled_logprobs: torch.Tensor,
+                   tokens_in: torch.Tensor, positions: torch.Tensor, seq_meta: torch.Tensor,
+                   draw_counters: torch.Tensor, out_tokens: torch.Tensor, out_logprobs: torch.Tensor) -> None:
+    """Between two decode steps that the host does not see: what was drawn is recorded as row step_counter[0] of
+    out_tokens / out_logprobs [max_steps, B] and becomes the next step's input; positions, the requests' first
+    positions (seq_meta[:, 3]), their draw counters and the step counter go up by one."""
+    _dev(step_counter, sampled_tokens, sampled_logprobs, tokens_in, positions, seq_meta, draw_counters, out_tokens,
+         out_logprobs)
+    B = tokens_in.numel()
+    for t, name in ((step_counter, "step_counter"), (sampled_tokens, "sampled_tokens"), (tokens_in, "tokens_in"),
+                    (positions, "positions"), (seq_meta, "seq_meta"), (draw_counters, "draw_counters"),
+                    (out_tokens, "out_tokens")):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise KernelError(f"decode_advance: {name} must be contiguous int32")
+    for t, name in ((sampled_logprobs, "sampled_logprobs"), (out_logprobs, "out_logprobs")):
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise KernelError(f"decode_advance: {name} must be contiguous float32")
+    if out_tokens.dim() != 2 or out_tokens.shape[1] != B or tuple(out_logprobs.shape) != tuple(out_tokens.shape):
+        raise KernelError("decode_advance: the records are [max_steps, B]")
+    if min(sampled_tokens.numel(), sampled_logprobs.numel(), positions.numel(), draw_counters.numel()) < B \
+            or seq_meta.numel() < 4 * B or step_counter.numel() < 1:
+        raise KernelError("decode_advance: an array is shorter than the number of requests")
+    _lib.call("sa_decode_advance", B, _ptr(step_counter), _ptr(sampled_tokens), _ptr(sampled_logprobs), _ptr(tokens_in),
+              _ptr(positions), _ptr(seq_meta), _ptr(draw_counters), _ptr(out_tokens), _ptr(out_logprobs),
+              out_tokens.shape[0], _stream())
+
+
+def decode_slots(positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor, page_size: int,
+                 slot_mapping: torch.Tensor) -> None:
+    """slot_mapping[b] = block_table[token_seq[b], positions[b] // page_size] * page_size + positions[b] % page_size."""
+    _dev(positions, token_seq, block_table, slot_mapping)
+    B = positions.numel()
+    _i32(positions, "decode_slots: positions", B)
+    _i32(token_seq, "decode_slots: token_seq", B)
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("decode_slots: block_table must be int32 [sequences, blocks]")
+    if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < B or not slot_mapping.is_contiguous():
+        raise KernelError("decode_slots: slot_mapping must be contiguous int64 with one entry per token")
+    _lib.call("sa_decode_slots", B, _ptr(positions), _ptr(token_seq), _ptr(block_table), block_table.stride(0),
+              int(page_size), _ptr(slot_mapping), _stream())
+
+
 # --------------------------------------------------------------------------- matrix products
 
 EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2

@@ -37,11 +37,10 @@ class Sampler:
         self._tokens = torch.empty(max_rows, dtype=torch.int32, device=self.device)
         self._logprobs = torch.empty(max_rows, dtype=torch.float32, device=self.device)
 
-    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
-               counters: Sequence[int]) -> tuple[list[int], list[float]]:
-        """logits float32 [R, V]; one SamplingParams, seed and draw counter per row."""
-        R = logits.shape[0]
-        if not (len(params) == len(seeds) == len(counters) == R):
+    def stage(self, params: Sequence[SamplingParams], seeds: Sequence[int], counters: Sequence[int]) -> None:
+        """Puts the rows' parameters, seeds and draw counters where `launch` reads them (fixed device buffers)."""
+        R = len(params)
+        if not (len(seeds) == len(counters) == R):
             raise ValueError("sample: one params, seed and counter per row of logits")
         if R > self.max_rows:
             raise ValueError(f"sample: {R} rows, room for {self.max_rows}")
@@ -55,7 +54,26 @@ class Sampler:
         self._f_dev.copy_(self._f_host, non_blocking=True)
         self._i_dev.copy_(self._i_host, non_blocking=True)
         self._s_dev.copy_(self._s_host, non_blocking=True)
-        tokens, logprobs = ops.sample(logits, self._f_dev[:n], self._i_dev[:n], self._f_dev[n:], self._s_dev,
-                                      self._i_dev[n:], self._tokens, self._logprobs)
+
+    @property
+    def draw_counters(self) -> torch.Tensor:
+        """The rows' draw counters on the device (int32 [max_rows]); `launch` reads them."""
+        return self._i_dev[self.max_rows:]
+
+    def launch(self, logits: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        """The sampling kernel on what `stage` left: returns the device buffers (tokens int32, log-probabilities
+        float32, [max_rows], the same every time) without waiting for it."""
+        n = self.max_rows
+        return ops.sample(logits, self._f_dev[:n], self._i_dev[:n], self._f_dev[n:], self._s_dev, self._i_dev[n:],
+                          self._tokens, self._logprobs)
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+               counters: Sequence[int]) -> tuple[list[int], list[float]]:
+        """logits float32 [R, V]; one SamplingParams, seed and draw counter per row."""
+        R = logits.shape[0]
+        if len(params) != R:
+            raise ValueError("sample: one params, seed and counter per row of logits")
+        self.stage(params, seeds, counters)
+        tokens, logprobs = self.launch(logits)
         # one synchronising copy back: the scheduler needs the tokens to go on
         return tokens[:R].tolist(), logprobs[:R].tolist()

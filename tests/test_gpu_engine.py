@@ -110,7 +110,7 @@ def test_graph_replays_match_eager(tmp_path, dtype):
                 ex.finish_request(r)
                 live.remove(r)
         if graphs:
-            assert sorted(ex._graphs) == [1, 2, 3]
+            assert sorted({k[0] for k in ex._graphs}) == [1, 2, 3]   # recorded per number of requests (and context scale)
         outs[graphs] = {r: torch.cat(v) for r, v in got.items()}
     for r in reqs:
         assert torch.equal(outs[False][r], outs[True][r]), r

@@ -1,4 +1,5 @@
 """Greedy and sampled generation through the entry point and the command line, on the GPU."""
+import dataclasses
 import json
 import os
 import subprocess
@@ -67,3 +68,36 @@ def test_command_line(tmp_path, gpu_lib):
     assert r.returncode == 0, r.stderr
     rec = json.loads(r.stdout.strip().splitlines()[-1])
     assert rec["tokens"] == plain.greedy(w, cfg, prompt, 5, torch.float64) and rec["finish_reason"] == "length"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_in_a_row_on_the_device(tmp_path, gpu_lib, dtype):
+    """Decoding several steps without the host in between (drawn tokens fed on the device, positions, slots and
+    draw counters advanced by a kernel) gives what step-by-step decoding gives: greedy and sampled, across page
+    edges and a window, with requests that end at different times, an end-of-sequence token among them."""
+    d = tiny.write_model("D", str(tmp_path / "D"), dtype=torch.bfloat16, std=0.3)
+    _, cfg = plain.load(d)
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 90 + n) for n in (3, 14, 31, 18)]
+    plist = [SamplingParams(temperature=0.0, max_decode_steps=37), SamplingParams(temperature=0.8, max_decode_steps=21, seed=5),
+             SamplingParams(temperature=1.1, top_k=20, max_decode_steps=40, seed=6),
+             SamplingParams(temperature=0.0, max_decode_steps=9)]
+    kw = dict(activation_dtype=dtype, batch_size=4, max_seq_len=96, page_size=16, max_num_issue_tokens=64)
+    one = LMInterface(d, intermediate_steps=1, **kw).generate(prompts, sampling_params=plist)
+    for steps in (2, 8, 64):
+        lm_many = LMInterface(d, intermediate_steps=steps, **kw)
+        many = lm_many.generate(prompts, sampling_params=plist)
+        assert [o.output_token_ids for o in many] == [o.output_token_ids for o in one], steps
+        for a, b in zip(many, one):
+            torch.testing.assert_close(torch.tensor(a.output_token_logprobs), torch.tensor(b.output_token_logprobs),
+                                       rtol=1e-5, atol=1e-5)
+        lm_many.executor.cache.check()
+        # a second call goes through the recorded graph from its first step
+        again = lm_many.generate(prompts, sampling_params=plist)
+        assert [o.output_token_ids for o in again] == [o.output_token_ids for o in one], steps
+    # an end-of-sequence token in the middle of a run of steps ends that request there
+    eos = one[0].output_token_ids[5]
+    lm_eos = LMInterface(d, intermediate_steps=8, **kw)
+    lm_eos.model.spec = dataclasses.replace(lm_eos.model.spec, eos_token_ids=(eos,))
+    out = lm_eos.generate([prompts[0]], sampling_params=[SamplingParams(temperature=0.0, max_decode_steps=37)])[0]
+    assert out.output_token_ids == one[0].output_token_ids[:one[0].output_token_ids.index(eos) + 1]
+    assert out.finish_reason == "eos"
