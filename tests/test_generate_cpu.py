@@ -62,3 +62,21 @@ def test_eos_stops(tmp_path, cpu_ops):
     out = lm(d).generate(prompt, sampling_params=SamplingParams(temperature=0.0, max_decode_steps=6))[0]
     stop = free_run.index(free_run[2]) + 1
     assert out.output_token_ids == free_run[:stop] and out.finish_reason == "eos" and not out.is_truncated
+
+
+def test_steps_in_a_row_change_nothing(tmp_path, cpu_ops):
+    """The entry point's bookkeeping for several decode steps per scheduling decision (here through the host,
+    step by step): the same tokens as one step at a time, also when requests end inside a run of steps and when
+    the pages are so few that runs shrink."""
+    d = tiny.write_model("B", str(tmp_path / "B"), std=0.1)
+    _, cfg = plain.load(d)
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 80 + n) for n in (2, 9, 13)]
+    plist = [SamplingParams(temperature=0.7, max_decode_steps=n, seed=50 + n) for n in (5, 12, 9)]
+    one = lm(d, intermediate_steps=1).generate(prompts, sampling_params=plist)
+    for steps, pages in ((4, None), (16, None), (16, 9)):
+        many = lm(d, intermediate_steps=steps, total_num_pages=pages)
+        outs = many.generate(prompts, sampling_params=plist)
+        assert [o.output_token_ids for o in outs] == [o.output_token_ids for o in one], (steps, pages)
+        assert [o.finish_reason for o in outs] == [o.finish_reason for o in one]
+        many.executor.cache.check()
+        assert many.stats["steps"] >= max(len(o.output_token_ids) for o in one)
