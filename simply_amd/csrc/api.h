@@ -55,14 +55,16 @@ int sa_decode_slots(int B, const int* positions, const int* token_seq, const int
 
 // C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1: gelu_tanh(A.W^T) * (A.W2^T);
 // 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
-// few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel (2 and 3 refuse what they do not take).
+// few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel; 4: the wide-tile bfloat16 MFMA kernel for very
+// many rows (2, 3 and 4 refuse what they do not take).
 // packed: W (and W2) are tiled instead of row-major: [ceil(N / 16)][ceil(K / 32)][64][8] bfloat16, block (i, j)
 // holding rows 16 i .. 16 i + 15 and columns 32 j .. 32 j + 31 as element [(k % 32) / 8 * 16 + n % 16][k % 8],
 // zero beyond N and K (one MFMA operand per block, in register order).  With epilogue 1 a packed W holds both
 // matrices, their row blocks in turn (block row 2 i: rows 16 i .. of the gate, 2 i + 1: of the other factor), and
 // W2 is null.
 // shape > 0 fixes how a kernel cuts its work: for the few-rows kernel rows of W per workgroup (4, 8 or 16) * 100 +
-// waves, for the tiled kernel the number of cuts of K.  workspace (bytes): scratch memory for partial results
+// waves, for the tiled kernel the number of cuts of K, for the wide kernel (algo 4 only) stages * 1000000 + rows *
+// 1000 + weight rows of a workgroup's tile.  workspace (bytes): scratch memory for partial results
 // when K is cut over workgroups.
 int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C, int c_dtype,
             int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, int packed, int shape,
@@ -149,6 +151,10 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
                             hipStream_t stream);
+bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
+                     const void* C, int c_dtype, int epi, int packed);
+int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
+              hipStream_t stream);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
                int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream);

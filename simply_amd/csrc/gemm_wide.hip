@@ -1,0 +1,301 @@
+// C[M, N] = epilogue(A[M, K] . W[N, K]^T) in bfloat16 for very many rows (whole prompts), on tiles wide enough
+// that the vector memory path is no longer the bound: the 128 x 128 tiles of the tiled kernel pull 96 KiB per
+// slab of 64 columns through a CU's 64 bytes a clock, which caps it at about a third of the MFMA rate.
+//
+// A workgroup of eight waves (one per CU) owns 256 x 192, 256 x 128 or 128 x 256 outputs and takes both operands
+// through LDS, in slabs of 64 columns of K that go round two or three buffers, with loads that go from global
+// memory straight into LDS (no registers in between).
+//   * Layout in LDS: W as KiB blocks in MFMA operand order (16 rows x 32 columns, lane l holds row l % 16,
+//     columns 8 (l / 16) ..), which is how it lies in global memory, so a block is a copy.  A as rows of 128 bytes
+//     (eight lanes load a row: whole lines) whose eight 16-byte pieces are permuted by the row's number, so that
+//     the 16 rows of a fragment read fall into different banks.  All fragment reads are ds_read_b128 without bank
+//     conflicts (measured).
+//   * Schedule of a wave: the fragments of the two halves of a slab have registers of their own; the products of
+//     the second half are held back until after the next barrier, where they cover the fragment reads of the next
+//     slab's first half, and the reads of the second half are covered by the products of the first: between two
+//     barriers the MFMA unit always has products to do.  The loads of the slab one or two ahead are spread over
+//     the products, one after each row of them: issued together after the barrier, the eight waves queue up at
+//     the memory pipeline (16 cycles a load) while the MFMA unit idles.
+//   * The products are taken transposed (W fragment as the first operand), so that a lane holds four neighbouring
+//     columns of one row of C and stores them as one 8-byte piece.
+//
+// Epilogues: none; gated (C = gelu_tanh(A.Wg^T) * (A.Wu^T), both rounded to bfloat16 first, from one weight whose
+// 16-row tiles alternate between Wg and Wu).  K must be a multiple of 64, N and ldc of 4.
+#include "api.h"
+#include "common.h"
+
+namespace sa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+namespace wide {
+
+constexpr int kWaves = 8;
+constexpr int BK = 64;
+constexpr int kCUs = 256;  // compute units of an MI355X
+
+// s_waitcnt for "at most n vector-memory loads outstanding" and nothing else (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8)
+constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+// The workgroup barrier alone; the empty statements keep the compiler from moving memory accesses across it.
+__device__ inline void bare_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// 16 bytes per lane from global memory (base + offset bytes, base the same for the whole wave) into LDS at byte
+// address lds + 16 * lane (the same for the whole wave).  Written as an instruction: the compiler counts a load
+// into LDS that it knows of as a pending LDS access for as long as the load is under way, and then makes every
+// wait for a fragment read a wait for all of them.  It does not know of these loads: the kernel waits for them
+// itself (vmcnt) before the barrier that precedes the first read of what they bring.
+__device__ __forceinline__ void load_to_lds(const bf16* base, uint32_t offset, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(offset), "s"(base), "s"(lds)
+               : "memory");
+}
+
+// WM x WN: 16 x 16 tiles of a wave (rows of A x rows of W); WAVES_M x (8 / WAVES_M) waves.
+template <int WM, int WN, int WAVES_M, int EPI, int NSTAGE>
+__global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__ A, int64_t lda,
+                                                        const bf16* __restrict__ W, bf16* __restrict__ C, int64_t ldc,
+                                                        int M, int N, int K, int chunks) {
+  constexpr int WAVES_N = kWaves / WAVES_M;
+  constexpr int MT = WAVES_M * WM, NT = WAVES_N * WN;  // 16-row tiles of A and of W per workgroup
+  constexpr int BM = MT * 16;
+  constexpr int A_BLOCKS = MT * 2, W_BLOCKS = NT * 2;  // KiB blocks of a slab
+  static_assert(A_BLOCKS % kWaves == 0 && W_BLOCKS % kWaves == 0, "every wave copies the same number of blocks");
+  static_assert(EPI != 1 || WN % 2 == 0, "gate and factor tiles come in pairs");
+  constexpr int APW = A_BLOCKS / kWaves, WPW = W_BLOCKS / kWaves;
+  constexpr int STAGE = (A_BLOCKS + W_BLOCKS) * 512;  // elements
+  __shared__ __attribute__((aligned(16))) __bf16 stages[NSTAGE * STAGE];
+  const uint32_t lds_base = static_cast<uint32_t>(
+      reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) __bf16*)stages));
+
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  // Which tile: workgroups go to the eight XCDs in turn, each with an L2 of its own; the numbering is turned round
+  // so that an XCD gets a contiguous share of the tiles, and within it tiles go in columns eight wide, rows first.
+  int bx = blockIdx.x, by = blockIdx.y;
+  {
+    const int nx = gridDim.x, ny = gridDim.y, total = nx * ny;
+    int l = bx + nx * by;
+    if (total % 8 == 0) l = (l % 8) * (total / 8) + l / 8;
+    constexpr int GX = 8;
+    const int full = nx / GX;
+    if (l < full * GX * ny) {
+      const int col = l / (GX * ny), rem = l % (GX * ny);
+      by = rem / GX;
+      bx = col * GX + rem % GX;
+    } else {
+      const int rem = l - full * GX * ny, width = nx % GX;
+      by = rem / width;
+      bx = full * GX + rem % width;
+    }
+  }
+  const int m_base = by * BM;
+  const int NW = EPI == 1 ? 2 * ((N + 15) / 16) * 16 : N;
+  const int ntiles = (NW + 15) / 16;
+  const int nt_base = bx * NT;
+
+  // ---- what this wave copies of every slab: KiB blocks wave + 8 i of A and of W.
+  // A block b is rows 8 (b % 2) .. + 8 of tile b / 2, all 64 columns of the slab: eight lanes per row read its 128
+  // bytes, so a load is eight whole lines.  In LDS a row's eight 16-byte pieces are permuted (piece p of row r of
+  // the tile lies at p ^ (r / 2)), which makes the fragment reads below (16 rows, one piece each) hit all banks.
+  // W block b is tile b / 2, columns 32 (b % 2) .. of the slab: a KiB as it lies in global memory.
+  // Rows beyond M read row M - 1, tiles beyond the last the last one (their products are never stored).
+  const int half_mine = wave % 2, tile_mine = wave / 2;
+  uint32_t a_off[APW];  // bytes; the host checks that M * lda fits
+#pragma unroll
+  for (int i = 0; i < APW; ++i) {
+    const int r = half_mine * 8 + lane / 8;  // row of the tile
+    const int m = m_base + (tile_mine + 4 * i) * 16 + r;
+    a_off[i] = (static_cast<uint32_t>(m < M ? m : M - 1) * static_cast<uint32_t>(lda) + ((lane % 8) ^ (r / 2)) * 8) * 2;
+  }
+  const bf16* w_from[WPW];  // the same for the whole wave
+#pragma unroll
+  for (int i = 0; i < WPW; ++i) {
+    const int nt = nt_base + tile_mine + 4 * i;
+    const int clamped = __builtin_amdgcn_readfirstlane(nt < ntiles ? nt : ntiles - 1);
+    w_from[i] = W + (static_cast<size_t>(clamped) * chunks + half_mine) * 512;
+  }
+  // load n (of LOADS) of slab `slab` into buffer `buf`
+  constexpr int LOADS = APW + WPW;
+  auto request_one = [&](int n, int slab, int buf) __attribute__((always_inline)) {
+    const uint32_t to = lds_base + static_cast<uint32_t>(buf) * (STAGE * 2);
+    if (n < APW)
+      load_to_lds(A + static_cast<size_t>(slab) * BK, a_off[n], to + ((tile_mine + 4 * n) * 2 + half_mine) * 1024);
+    else
+      load_to_lds(w_from[n - APW] + static_cast<size_t>(slab) * 1024, lane * 16,
+                  to + (A_BLOCKS + (tile_mine + 4 * (n - APW)) * 2 + half_mine) * 1024);
+  };
+
+  floatx4 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // this lane's piece of an A fragment (row lane % 16, columns 32 kc + 8 (lane / 16) ..) within its tile, elements
+  int a_frag[2];
+#pragma unroll
+  for (int kc = 0; kc < 2; ++kc) {
+    const int r = lane % 16;
+    a_frag[kc] = r * 64 + ((kc * 4 + lane / 16) ^ (r / 2)) * 8;
+  }
+  const int slabs = K / BK;
+  // Fragments of the two halves of a slab (columns 0 .. 31 and 32 .. 63) in registers of their own.  The products
+  // of the second half are held back until after the next barrier, where they cover the time that the fragment
+  // reads of the next slab's first half take; the reads of the second half are covered by the products of the
+  // first.  So the MFMA unit always has products to do while LDS reads are under way.
+  bf16x8 fa[2][WM], fw[2][WN];
+  auto read = [&](const __bf16* stage, int kc) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+      fa[kc][i] = *reinterpret_cast<const bf16x8*>(stage + (wm * WM + i) * 1024 + a_frag[kc]);
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+      fw[kc][j] = *reinterpret_cast<const bf16x8*>(stage + ((A_BLOCKS + (wn * WN + j) * 2 + kc) * 64 + lane) * 8);
+  };
+  static_assert(LOADS <= 2 * WM, "a load after each row of products");
+  // The products of half kc; after row i of them load first + i of slab `slab` is asked for (if there is one): the
+  // loads of a slab are spread over its products, so that the waves do not queue up at the memory pipeline
+  // (which takes 16 cycles for each) while the MFMA unit idles.
+  auto multiply = [&](int kc, int first, int slab, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kc][j], fa[kc][i], acc[i][j], 0, 0, 0);
+      if (first >= 0 && first + i < LOADS) {
+        __builtin_amdgcn_sched_barrier(0);
+        request_one(first + i, slab, buf);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  // The slabs go round NSTAGE buffers.  Before the barrier of slab s this wave's loads of slab s have arrived (those
+  // of the NSTAGE - 2 slabs after it may be under way) and its fragment reads of slab s - 1 are done; after it
+  // everyone's, so that the loads of slab s + NSTAGE - 1 may go into the buffer of slab s - 1.  Past the last slab
+  // the last one is loaded again (no branch).
+#pragma unroll
+  for (int p = 0; p < NSTAGE; ++p)
+#pragma unroll
+    for (int n = 0; n < LOADS; ++n) request_one(n, p < slabs ? p : slabs - 1, p);
+  // slab 0: nothing held back yet, and its loads for later are already asked for
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm((NSTAGE - 1) * LOADS));
+  bare_barrier();
+  read(stages, 0);
+  read(stages, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(0, -1, 0, 0);
+  int cur = 1, target = 0;
+  for (int s = 1; s < slabs; ++s) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((NSTAGE - 2) * LOADS) & ~(15 << 8));
+    bare_barrier();
+    const int ahead = s + NSTAGE - 1 < slabs ? s + NSTAGE - 1 : slabs - 1;
+    const __bf16* stage = stages + cur * STAGE;
+    read(stage, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1, 0, ahead, target);
+    __builtin_amdgcn_sched_barrier(0);  // (reads moved up among these products would need registers of their own)
+    read(stage, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(0, WM, ahead, target);
+    target = cur;
+    cur = cur + 1 == NSTAGE ? 0 : cur + 1;
+  }
+  multiply(1, -1, 0, 0);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the loads asked for beyond the last slab
+
+  // ---- epilogue.  acc[i][j][v] is the product at row (tile i, lane % 16) of A and row (tile j, 4 (lane / 16) + v)
+  // of W.
+  const int row = lane % 16, quad = lane / 16;
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int m = m_base + (wm * WM + i) * 16 + row;
+    if (m >= M) continue;
+    bf16* c_row = C + static_cast<size_t>(m) * ldc;
+    constexpr int OUT = EPI == 1 ? WN / 2 : WN;
+#pragma unroll
+    for (int j = 0; j < OUT; ++j) {
+      const int tile = EPI == 1 ? (nt_base + wn * WN) / 2 + j : nt_base + wn * WN + j;
+      const int n = tile * 16 + quad * 4;
+      if (n >= N) continue;
+      float x[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        if (EPI == 1)
+          x[v] = gelu_tanh_fast(to_float(float_to_bf16(acc[i][2 * j][v]))) * to_float(float_to_bf16(acc[i][2 * j + 1][v]));
+        else
+          x[v] = acc[i][j][v];
+      }
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(float_to_bf16(x[0]).bits) | (static_cast<uint32_t>(float_to_bf16(x[1]).bits) << 16);
+      packed.y = static_cast<uint32_t>(float_to_bf16(x[2]).bits) | (static_cast<uint32_t>(float_to_bf16(x[3]).bits) << 16);
+      *reinterpret_cast<uint2*>(c_row + n) = packed;
+    }
+  }
+}
+
+template <int WM, int WN, int WAVES_M, int NSTAGE>
+static void launch(const bf16* A, int64_t lda, const bf16* W, bf16* C, int64_t ldc, int M, int N, int K, int epi,
+                   hipStream_t stream) {
+  constexpr int BM = WAVES_M * WM * 16, BNW = (kWaves / WAVES_M) * WN * 16;
+  const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
+  const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM);
+  if (epi == 1)
+    gemm_wide_kernel<WM, WN, WAVES_M, 1, NSTAGE><<<grid, 512, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
+  else
+    gemm_wide_kernel<WM, WN, WAVES_M, 0, NSTAGE><<<grid, 512, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
+}
+
+}  // namespace wide
+
+bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
+                     const void* C, int c_dtype, int epi, int packed) {
+  auto aligned = [](const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+  return packed && W2 == nullptr && (epi == 0 || epi == 1) && c_dtype == kBF16 && M >= 1 && K % wide::BK == 0 &&
+         N % 4 == 0 && lda % 8 == 0 && ldc % 4 == 0 && aligned(A, 16) && aligned(W, 16) && aligned(C, 8) &&
+         static_cast<int64_t>(M) * lda < (int64_t{1} << 31);  // byte offsets of rows are kept in 32 bits
+}
+
+// shape: 0: chosen here; else stages * 1000000 + rows * 1000 + weight rows of a workgroup's tile (2256192, 3256128,
+// 3128256).
+int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
+              hipStream_t stream) {
+  const bf16* a = static_cast<const bf16*>(A);
+  const bf16* w = static_cast<const bf16*>(W);
+  bf16* c = static_cast<bf16*>(C);
+  if (shape == 0) {
+    // one workgroup per CU at a time: the cost of a shape is its rounds over the CUs times the size of its tile;
+    // of equals the first (256 x 192 has the least traffic per product)
+    const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
+    const int shapes[3][3] = {{2256192, 256, 192}, {3256128, 256, 128}, {3128256, 128, 256}};
+    int64_t best = -1;
+    for (const auto& sh : shapes) {
+      const int64_t tiles = static_cast<int64_t>((M + sh[1] - 1) / sh[1]) * ((NW + sh[2] - 1) / sh[2]);
+      const int64_t cost = ((tiles + wide::kCUs - 1) / wide::kCUs) * sh[1] * sh[2];
+      if (best < 0 || cost < best) {
+        best = cost;
+        shape = sh[0];
+      }
+    }
+  }
+  switch (shape) {
+    case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
+    case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
+    case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
+    default:
+      set_error("gemm: unknown wide tile %d", shape);
+      return 1;
+  }
+  return check_launch("gemm_wide");
+}
+
+}  // namespace sa

@@ -43,7 +43,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(epilogue != 1 || (W2 != nullptr) != (packed != 0),
              "gemm: the gated epilogue takes two row-major weights, or one tiled weight that holds both");
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
-  SA_REQUIRE(algo >= 0 && algo <= 3, "gemm: unknown algorithm %d", algo);
+  SA_REQUIRE(algo >= 0 && algo <= 4, "gemm: unknown algorithm %d", algo);
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
   // up to 16 rows, and up to 32 for products without the gated epilogue (measured: the few-rows kernel, whose waves
   // read the activations from L2, beats the tiled one with K cut over workgroups there)
@@ -54,6 +54,15 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "operands; got M=%d K=%d lda=%lld", M, K, (long long)lda);
     if (takes)
       return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, shape, stream);
+  }
+  // from 256 rows on, the wide tiles (both operands through LDS)
+  if (algo == 4 || (algo == 0 && bf16_in && packed && M >= 256)) {
+    const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
+    SA_REQUIRE(takes || algo == 0,
+               "gemm: the wide MFMA kernel takes bfloat16 in and out with tiled weights, no soft-cap, K a multiple of "
+               "64, N and ldc of 4, lda of 8; got N=%d K=%d lda=%lld ldc=%lld tiled=%d", N, K, (long long)lda,
+               (long long)ldc, packed);
+    if (takes) return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, algo == 4 ? shape : 0, stream);
   }
   if (algo == 3 || (algo == 0 && bf16_in && packed && M > 16)) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);

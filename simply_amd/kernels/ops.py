@@ -17,7 +17,7 @@ from .packing import TiledWeight
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
-ALGO_AUTO, ALGO_GENERIC, ALGO_SKINNY, ALGO_TILED = 0, 1, 2, 3
+ALGO_AUTO, ALGO_GENERIC, ALGO_SKINNY, ALGO_TILED, ALGO_WIDE = 0, 1, 2, 3, 4
 
 
 def _code(t: torch.Tensor) -> int:
@@ -272,9 +272,9 @@ def _workspace(device) -> torch.Tensor:
 
 
 # Plain products (no epilogue) of at least this many rows go to the library (hipBLASLt through torch.matmul) when
-# the weight has kept its row-major form; 0: never.  The gated and soft-capped products and everything with fewer
-# rows run on this package's kernels.
-_library_gemm_min_rows = 256
+# the weight has kept its row-major form; 0 (the default): never, everything runs on this package's kernels.  Set
+# before the weights are loaded: they keep the second form only while this is on.
+_library_gemm_min_rows = 0
 
 
 def set_library_gemm_min_rows(rows: int) -> None:

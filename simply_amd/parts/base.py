@@ -65,8 +65,8 @@ def as_product_weight(t: torch.Tensor, shared: bool = False, many_rows: bool = F
     """A matrix in the form that the matrix-product kernels read fastest: bfloat16 matrices on the GPU are
     re-laid in tiles (simply_amd/kernels/packing.py), anything else stays row-major.  `shared`: parts that are
     handed the same tensor during one load (a tied table and head) get the same re-laid copy.  `many_rows`: the
-    weight of a plain product that portions of prompts go through; it also keeps its row-major form, which the
-    library product for many rows reads (unless that is switched off: ops.set_library_gemm_min_rows(0))."""
+    weight of a plain product that portions of prompts go through; it also keeps its row-major form when the
+    library product for many rows is switched on (ops.set_library_gemm_min_rows), which reads that form."""
     import dataclasses as dc
 
     from ..kernels import ops

@@ -382,6 +382,46 @@ def test_gemm_tiled(M, N, K):
         ops.gemm(a, w, **kw)     # row-major weights are refused
 
 
+@pytest.mark.parametrize("M,N,K", [(257, 1000, 192), (300, 200, 128), (1, 16, 64), (700, 100, 64), (2048, 2304, 2048),
+                                   (513, 4096, 2304), (1000, 388, 1088)])
+def test_gemm_wide(M, N, K):
+    """The wide-tile MFMA kernel for very many rows: its three tile shapes and its own choice, plain and gated,
+    edges in M and N, odd numbers of slabs, strided rows in and out; and what it refuses."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.lib import KernelError
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles
+    a, w, w2 = rand((M, K), torch.bfloat16, 90), rand((N, K), torch.bfloat16, 91, 0.05), rand((N, K), torch.bfloat16, 92, 0.05)
+    tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
+    t = dict(rtol=2e-2, atol=2e-2)
+    want, want_gated = ref.gemm(a, w).float(), ref.gemm(a, w, w2=w2).float()
+    for shape in (0, 2256192, 3256128, 3128256):
+        kw = dict(algo=ops.ALGO_WIDE, shape=shape)
+        torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), want, **t)
+        torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), want_gated, **t)
+    # the same rows whatever the tile and whoever else is in the batch, to the bit: every sum runs along K in order
+    one = ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=2256192)
+    assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=3128256))
+    assert torch.equal(one[: M // 2 + 1], ops.gemm(a[: M // 2 + 1], tw, algo=ops.ALGO_WIDE))
+    assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_TILED))
+    # rows inside wider rows, in and out
+    kw = dict(algo=ops.ALGO_WIDE)
+    big = rand((M, K + 16), torch.bfloat16, 93)
+    out = torch.full((M, N + 12), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.gemm(big[:, 8:8 + K], tw, out=out[:, 4:4 + N], **kw)
+    torch.testing.assert_close(out[:, 4:4 + N].float(), ref.gemm(big[:, 8:8 + K], w).float(), **t)
+    assert (out[:, :4] == 7.0).all() and (out[:, 4 + N:] == 7.0).all()
+    with pytest.raises(KernelError, match="wide"):
+        ops.gemm(a, w, **kw)                                     # row-major weights
+    with pytest.raises(KernelError, match="wide"):
+        ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw)   # the soft-cap epilogue
+    with pytest.raises(KernelError, match="wide"):
+        ops.gemm(a[:, :K - 32], pack_tiles(w[:, :K - 32].contiguous()), **kw)   # K that is no multiple of 64
+    with pytest.raises(KernelError, match="wide"):
+        ops.gemm(a, pack_tiles(w[:N - 2].contiguous()), **kw)  # N that is no multiple of 4
+    # from 256 rows on it is what the library chooses by itself; below, and for what it refuses, the tiled kernel
+    torch.testing.assert_close(ops.gemm(a, pack_tiles(w[:N - 2].contiguous())).float(), want[:, :N - 2], **t)
+
+
 def test_add_rmsnorm_wide_rows():
     """Rows wider than the kernel keeps in registers take its second code path."""
     from simply_amd.kernels import ops
