@@ -2,9 +2,9 @@
 // that the vector memory path is no longer the bound: the 128 x 128 tiles of the tiled kernel pull 96 KiB per
 // slab of 64 columns through a CU's 64 bytes a clock, which caps it at about a third of the MFMA rate.
 //
-// A workgroup of eight waves (one per CU) owns 256 x 192, 256 x 128 or 128 x 256 outputs and takes both operands
-// through LDS, in slabs of 64 columns of K that go round two or three buffers, with loads that go from global
-// memory straight into LDS (no registers in between).
+// A workgroup of eight waves (one per CU) owns 256 x 192, 256 x 128, 128 x 256 or 192 x 128 outputs and takes both
+// operands through LDS, in slabs of 64 columns of K that go round two or three buffers, with loads that go from
+// global memory straight into LDS (no registers in between).
 //   * Layout in LDS: W as KiB blocks in MFMA operand order (16 rows x 32 columns, lane l holds row l % 16,
 //     columns 8 (l / 16) ..), which is how it lies in global memory, so a block is a copy.  A as rows of 128 bytes
 //     (eight lanes load a row: whole lines) whose eight 16-byte pieces are permuted by the row's number, so that
@@ -266,7 +266,7 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
 }
 
 // shape: 0: chosen here; else stages * 1000000 + rows * 1000 + weight rows of a workgroup's tile (2256192, 3256128,
-// 3128256).
+// 3128256, 3192128).
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
               hipStream_t stream) {
   const bf16* a = static_cast<const bf16*>(A);
@@ -276,7 +276,7 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     // one workgroup per CU at a time: the cost of a shape is its rounds over the CUs times the size of its tile;
     // of equals the first (256 x 192 has the least traffic per product)
     const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-    const int shapes[3][3] = {{2256192, 256, 192}, {3256128, 256, 128}, {3128256, 128, 256}};
+    const int shapes[4][3] = {{2256192, 256, 192}, {3256128, 256, 128}, {3128256, 128, 256}, {3192128, 192, 128}};
     int64_t best = -1;
     for (const auto& sh : shapes) {
       const int64_t tiles = static_cast<int64_t>((M + sh[1] - 1) / sh[1]) * ((NW + sh[2] - 1) / sh[2]);
@@ -291,6 +291,7 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
     case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
     case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
+    case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
     default:
       set_error("gemm: unknown wide tile %d", shape);
       return 1;
