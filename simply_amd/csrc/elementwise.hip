@@ -320,6 +320,122 @@ __global__ __launch_bounds__(256) void rope_cache_write_rows_kernel(
   for (int idx = threadIdx.x; idx < K * hd; idx += blockDim.x) vdst[static_cast<size_t>(idx) * page_size] = vsrc[idx];
 }
 
+// The same for many tokens in bfloat16 with 16-byte accesses (hd a multiple of 16, 16-byte aligned rows and pages).
+// The first rot_blocks blocks rotate the q and k heads of kRotTokens tokens each: sines and cosines once per token
+// in LDS, then eight dimensions (and the eight that pair with them) per thread and step; keys go into the pages as
+// 16-byte pieces (eight neighbouring dimensions of a key are neighbours in both page layouts).  The other blocks
+// copy the v heads of kValTokens tokens each into the transposed value pages: a thread holds eight dimensions of
+// all 16 tokens and, when their slots are one run inside a page that starts at a multiple of eight (a prompt's
+// portion that starts at a page's edge), writes each dimension's 16 keys as two 16-byte pieces instead of 16
+// scattered 2-byte ones.
+constexpr int kRotTokens = 8, kValTokens = 16, kWideMaxHalf = 256;
+__global__ __launch_bounds__(256) void rope_cache_write_wide_kernel(
+    bf16* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ timescale,
+    float inv_scale_factor, float q_div, const int64_t* __restrict__ slot_mapping, bf16* __restrict__ k_pages,
+    bf16* __restrict__ v_pages, int T, int H, int K, int hd, int page_size, int rot_blocks) {
+  __shared__ float sn[kRotTokens * kWideMaxHalf], cs[kRotTokens * kWideMaxHalf];
+  const int tid = threadIdx.x, half = hd / 2;
+  if (static_cast<int>(blockIdx.x) < rot_blocks) {
+    const int t0 = blockIdx.x * kRotTokens;
+    const int nt = T - t0 < kRotTokens ? T - t0 : kRotTokens;
+    for (int idx = tid; idx < nt * half; idx += blockDim.x) {
+      float s = 0.f, c = 1.f;
+      if (timescale != nullptr)
+        sincosf(static_cast<float>(positions[t0 + idx / half]) / timescale[idx % half] * inv_scale_factor, &s, &c);
+      sn[idx] = s;
+      cs[idx] = c;
+    }
+    __syncthreads();
+    const int groups = half / 8, per_token = (H + K) * groups;
+    const bool tiled = keys_tiled(page_size, hd);
+    for (int item = tid; item < nt * per_token; item += blockDim.x) {
+      const int j = item / per_token, head = (item % per_token) / groups, i = (item % groups) * 8;
+      bf16* src = qkv + static_cast<size_t>(t0 + j) * row_stride + static_cast<size_t>(head) * hd + i;
+      bf16* to1 = src;
+      bf16* to2 = src + half;
+      if (head >= H) {
+        const int64_t slot = k_pages != nullptr ? slot_mapping[t0 + j] : -1;
+        if (slot < 0) continue;
+        const int koff = static_cast<int>(slot % page_size);
+        bf16* page = k_pages + ((slot / page_size) * K + (head - H)) * page_size * hd;
+        to1 = page + key_index(tiled, page_size, hd, koff, i);
+        to2 = page + key_index(tiled, page_size, hd, koff, i + half);
+      }
+      const uint4 a = *reinterpret_cast<const uint4*>(src), b = *reinterpret_cast<const uint4*>(src + half);
+      const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+      uint32_t o1[4], o2[4];
+      const float* sj = sn + j * half + i;
+      const float* cj = cs + j * half + i;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float r1[2], r2[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const float x1 = __uint_as_float(e ? aw[w] & 0xffff0000u : aw[w] << 16);
+          const float x2 = __uint_as_float(e ? bw[w] & 0xffff0000u : bw[w] << 16);
+          const float s = sj[2 * w + e], c = cj[2 * w + e];
+          r1[e] = x1 * c - x2 * s;
+          r2[e] = x2 * c + x1 * s;
+          if (head < H) {
+            r1[e] = r1[e] / q_div;
+            r2[e] = r2[e] / q_div;
+          }
+        }
+        o1[w] = static_cast<uint32_t>(float_to_bf16(r1[0]).bits) | (static_cast<uint32_t>(float_to_bf16(r1[1]).bits) << 16);
+        o2[w] = static_cast<uint32_t>(float_to_bf16(r2[0]).bits) | (static_cast<uint32_t>(float_to_bf16(r2[1]).bits) << 16);
+      }
+      *reinterpret_cast<uint4*>(to1) = uint4{o1[0], o1[1], o1[2], o1[3]};
+      *reinterpret_cast<uint4*>(to2) = uint4{o2[0], o2[1], o2[2], o2[3]};
+    }
+    return;
+  }
+  if (v_pages == nullptr) return;
+  const int t0 = (blockIdx.x - rot_blocks) * kValTokens;
+  const int nt = T - t0 < kValTokens ? T - t0 : kValTokens;
+  const int64_t slot0 = slot_mapping[t0];
+  bool run = nt == kValTokens && slot0 >= 0 && slot0 % 8 == 0 && slot0 % page_size + kValTokens <= page_size;
+  if (tid < nt && slot_mapping[t0 + tid] != slot0 + tid) run = false;
+  run = __syncthreads_and(run);
+  const int groups = hd / 8;
+  for (int item = tid; item < K * groups; item += blockDim.x) {
+    const int head = item / groups, d0 = (item % groups) * 8;
+    const bf16* src = qkv + static_cast<size_t>(t0) * row_stride + static_cast<size_t>(H + K + head) * hd + d0;
+    uint32_t x[kValTokens][4];
+#pragma unroll
+    for (int j = 0; j < kValTokens; ++j) {
+      const uint4 v = j < nt ? *reinterpret_cast<const uint4*>(src + static_cast<size_t>(j) * row_stride) : uint4{0, 0, 0, 0};
+      x[j][0] = v.x, x[j][1] = v.y, x[j][2] = v.z, x[j][3] = v.w;
+    }
+    if (run) {
+      bf16* dst = v_pages + (((slot0 / page_size) * K + head) * hd + d0) * page_size + slot0 % page_size;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        uint32_t o[kValTokens / 2];
+#pragma unroll
+        for (int w = 0; w < kValTokens / 2; ++w) {
+          const uint32_t lo = x[2 * w][e / 2], hi = x[2 * w + 1][e / 2];
+          o[w] = e % 2 ? (lo >> 16) | (hi & 0xffff0000u) : (lo & 0xffffu) | (hi << 16);
+        }
+        uint4* to = reinterpret_cast<uint4*>(dst + static_cast<size_t>(e) * page_size);
+        to[0] = uint4{o[0], o[1], o[2], o[3]};
+        to[1] = uint4{o[4], o[5], o[6], o[7]};
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kValTokens; ++j) {
+        if (j >= nt) continue;
+        const int64_t slot = slot_mapping[t0 + j];
+        if (slot < 0) continue;
+        uint16_t* dst = reinterpret_cast<uint16_t*>(v_pages) + (((slot / page_size) * K + head) * hd + d0) * page_size +
+                        slot % page_size;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          dst[static_cast<size_t>(e) * page_size] = static_cast<uint16_t>(e % 2 ? x[j][e / 2] >> 16 : x[j][e / 2] & 0xffffu);
+      }
+    }
+  }
+}
+
 // Rotation alone, in place, on [T, n_heads, hd] rows of stride row_stride.
 template <typename T>
 __global__ void rope_kernel(T* __restrict__ x, int64_t row_stride, const int* __restrict__ positions,
@@ -467,6 +583,16 @@ extern "C" int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, con
   SA_REQUIRE(page_size > 0 && scale_factor > 0.f && q_div > 0.f, "rope_cache_write: bad page size, scale factor or query scale");
   SA_REQUIRE((k_pages == nullptr) == (v_pages == nullptr) && (k_pages == nullptr || slot_mapping != nullptr),
              "rope_cache_write: key pages, value pages and slots come together");
+  auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  if (T >= 256 && dtype == kBF16 && hd % 16 == 0 && hd / 2 <= kWideMaxHalf && row_stride % 8 == 0 && aligned16(qkv) &&
+      aligned16(k_pages) && aligned16(v_pages)) {
+    const int rot_blocks = (T + kRotTokens - 1) / kRotTokens;
+    const int val_blocks = v_pages != nullptr && K > 0 ? (T + kValTokens - 1) / kValTokens : 0;
+    rope_cache_write_wide_kernel<<<rot_blocks + val_blocks, 256, 0, stream>>>(
+        static_cast<bf16*>(qkv), row_stride, positions, timescale, 1.f / scale_factor, q_div, slot_mapping,
+        static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), T, H, K, hd, page_size, rot_blocks);
+    return check_launch("rope_cache_write");
+  }
   if (T >= 256 && hd / 2 <= kMaxHalf) {  // many tokens (a block for every compute unit): a block per token
     if (dtype == kF32)
       rope_cache_write_rows_kernel<float><<<T, 256, 0, stream>>>(static_cast<float*>(qkv), row_stride, positions,

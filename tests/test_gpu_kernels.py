@@ -71,14 +71,26 @@ def test_add_rmsnorm(dtype, T, D):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("H,K,hd,P", [(4, 2, 16, 4), (6, 1, 32, 3), (8, 4, 256, 16), (3, 3, 48, 5)])
-@pytest.mark.parametrize("T", [11, 300])   # few tokens: a block per (token, head); many: a block per token
-def test_rope_cache_write(dtype, H, K, hd, P, T):
+@pytest.mark.parametrize("T,order", [(11, "random"), (300, "random"), (300, "run"), (300, "run from 5"), (333, "runs")])
+def test_rope_cache_write(dtype, H, K, hd, P, T, order):
+    """Few tokens: a block per (token, head); many: a block per token, or (bfloat16, head sizes in steps of 16)
+    blocks of 8 and 16 tokens with 16-byte accesses, which write the values of 16 tokens in one piece where their
+    slots are a run inside a page."""
     from simply_amd.kernels import ops
-    pages = -(-T // P) + 6
+    pages = 2 * -(-T // P) + 6
     qkv = rand((T, (H + 2 * K) * hd), dtype, 7)
-    positions = torch.tensor(([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7] * 28)[:T], dtype=torch.int32).cuda()
+    positions = torch.tensor(([0, 1, 2, 3, 100, 101, 7, 8000, 5, 6, 7] * 32)[:T], dtype=torch.int32).cuda()
     ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda()
-    slots = torch.randperm(pages * P)[:T].to(torch.int64).cuda()
+    if order == "random":
+        slots = torch.randperm(pages * P)[:T]
+    elif order == "run":
+        slots = torch.arange(T) + P          # one run from a page's edge
+    elif order == "run from 5":
+        slots = torch.arange(T) + 5          # one run that starts inside a page
+    else:                                    # runs of 40 slots at scattered places: some blocks of 16 are a run, some not
+        starts = torch.randperm(pages * P // 48)[: -(-T // 40)] * 48
+        slots = torch.cat([st + torch.arange(40) for st in starts])[:T]
+    slots = slots.to(torch.int64).cuda()
     kp, vp = torch.zeros((pages, K, P, hd), dtype=dtype).cuda(), torch.zeros((pages, K, hd, P), dtype=dtype).cuda()
     kp2, vp2, qkv2 = kp.clone(), vp.clone(), qkv.clone()
     ops.rope_cache_write(qkv, positions, ts, 1.0, 12.0, H, K, hd, slots, kp, vp)
