@@ -2,6 +2,8 @@
 // sum and the next norm), rotary encoding fused with the cache write, row gather.
 // All statistics, angles and the residual sum are in 32-bit whatever the
 // activation type is.
+#include <type_traits>
+
 #include "api.h"
 #include "common.h"
 
@@ -122,42 +124,35 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
   }
 }
 
-// The same for many rows (portions of prompts): one wave per row, the row in registers as 4-element pieces, wave
-// reductions only.  NCH: 256-element pieces of a row at most; D % 4 == 0 and 16-byte aligned rows.
+// The same for many rows (portions of prompts): a workgroup is one wave, which takes `rows_per_wave` rows in
+// turn, each row whole in registers as 4-element pieces (wave reductions only), and (rows of up to 2560 elements)
+// asks for the next row before it works on the one it has, so that stores and loads overlap a little.  NCH: 256-element pieces of a row at most; D % 4 == 0, 16-byte aligned.
 template <typename YT, typename OT, int NCH>
-__global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(
+__global__ __launch_bounds__(64) void add_rmsnorm_rows_kernel(
     const YT* __restrict__ y, const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_one_post,
     float* __restrict__ residual, const void* __restrict__ w_next, int w_next_dtype, float eps_next, float plus_one_next,
-    OT* __restrict__ out, int T, int D) {
-  const int lane = threadIdx.x % kWave;
-  const int row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (row >= T) return;
-  const size_t rb = static_cast<size_t>(row) * D;
-  float4 hv[NCH], yv[NCH];
+    OT* __restrict__ out, int T, int D, int rows_per_wave) {
+  const int lane = threadIdx.x;
+  const int row0 = blockIdx.x * rows_per_wave;
+  const int nrows = T - row0 < rows_per_wave ? T - row0 : rows_per_wave;
+  using RawY = typename std::conditional<sizeof(YT) == 4, float4, uint2>::type;
+  struct Row {
+    float4 h[NCH];
+    RawY y[NCH];
+  };
+  auto load = [&](int row, Row& b) __attribute__((always_inline)) {
+    const size_t rb = static_cast<size_t>(row) * D;
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) {
-    const int d = c * 256 + lane * 4;
-    hv[c] = d < D ? *reinterpret_cast<const float4*>(residual + rb + d) : float4{0.f, 0.f, 0.f, 0.f};
-    yv[c] = float4{0.f, 0.f, 0.f, 0.f};
-    if (d < D) {
-      if constexpr (sizeof(YT) == 4) {
-        yv[c] = *reinterpret_cast<const float4*>(y + rb + d);
-      } else {
-        const uint2 raw = *reinterpret_cast<const uint2*>(y + rb + d);
-        yv[c] = float4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
-                       __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
+    for (int c = 0; c < NCH; ++c) {
+      const int d = c * 256 + lane * 4;
+      if (d < D) {
+        b.h[c] = *reinterpret_cast<const float4*>(residual + rb + d);
+        b.y[c] = *reinterpret_cast<const RawY*>(y + rb + d);
       }
     }
-  }
-  float r = 1.f;
-  if (w_post != nullptr) {
-    float ss = 0.f;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) ss += yv[c].x * yv[c].x + yv[c].y * yv[c].y + yv[c].z * yv[c].z + yv[c].w * yv[c].w;
-    r = rsqrtf(wave_sum(ss) / static_cast<float>(D) + eps_post);
-  }
+  };
   // four scale factors at a time (one 8-byte load when they are bfloat16)
-  auto scales = [&](const void* w, int dtype, float plus, int d, float* out4) {
+  auto scales = [&](const void* w, int dtype, float plus, int d, float* out4) __attribute__((always_inline)) {
     if (dtype == kBF16) {
       const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const bf16*>(w) + d);
       out4[0] = __uint_as_float(raw.x << 16) + plus;
@@ -172,40 +167,79 @@ __global__ __launch_bounds__(256) void add_rmsnorm_rows_kernel(
       out4[3] = raw.w + plus;
     }
   };
-  float ss2 = 0.f;
+  auto process = [&](int row, Row& b) __attribute__((always_inline)) {
+    const size_t rb = static_cast<size_t>(row) * D;
+    float4 yv[NCH];
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) {
-    const int d = c * 256 + lane * 4;
-    if (d >= D) continue;
-    float* h = reinterpret_cast<float*>(&hv[c]);
-    const float* v = reinterpret_cast<const float*>(&yv[c]);
-    float w4[4] = {1.f, 1.f, 1.f, 1.f};
-    if (w_post != nullptr) scales(w_post, w_post_dtype, plus_one_post, d, w4);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      h[e] += w_post != nullptr ? v[e] * r * w4[e] : v[e];
-      ss2 += h[e] * h[e];
+    for (int c = 0; c < NCH; ++c) {
+      if (c * 256 + lane * 4 >= D) {
+        yv[c] = float4{0.f, 0.f, 0.f, 0.f};
+        b.h[c] = float4{0.f, 0.f, 0.f, 0.f};
+      } else if constexpr (sizeof(YT) == 4) {
+        yv[c] = b.y[c];
+      } else {
+        yv[c] = float4{__uint_as_float(b.y[c].x << 16), __uint_as_float(b.y[c].x & 0xffff0000u),
+                       __uint_as_float(b.y[c].y << 16), __uint_as_float(b.y[c].y & 0xffff0000u)};
+      }
     }
-    *reinterpret_cast<float4*>(residual + rb + d) = hv[c];
-  }
-  if (w_next == nullptr) return;
-  const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(D) + eps_next);
+    float r = 1.f;
+    if (w_post != nullptr) {
+      float ss = 0.f;
 #pragma unroll
-  for (int c = 0; c < NCH; ++c) {
-    const int d = c * 256 + lane * 4;
-    if (d >= D) continue;
-    const float* h = reinterpret_cast<const float*>(&hv[c]);
-    float w4[4], o[4];
-    scales(w_next, w_next_dtype, plus_one_next, d, w4);
+      for (int c = 0; c < NCH; ++c) ss += yv[c].x * yv[c].x + yv[c].y * yv[c].y + yv[c].z * yv[c].z + yv[c].w * yv[c].w;
+      r = rsqrtf(wave_sum(ss) / static_cast<float>(D) + eps_post);
+    }
+    float ss2 = 0.f;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = h[e] * r2 * w4[e];
-    if constexpr (sizeof(OT) == 4) {
-      *reinterpret_cast<float4*>(out + rb + d) = float4{o[0], o[1], o[2], o[3]};
-    } else {
-      uint2 packed;
-      packed.x = static_cast<uint32_t>(float_to_bf16(o[0]).bits) | (static_cast<uint32_t>(float_to_bf16(o[1]).bits) << 16);
-      packed.y = static_cast<uint32_t>(float_to_bf16(o[2]).bits) | (static_cast<uint32_t>(float_to_bf16(o[3]).bits) << 16);
-      *reinterpret_cast<uint2*>(out + rb + d) = packed;
+    for (int c = 0; c < NCH; ++c) {
+      const int d = c * 256 + lane * 4;
+      if (d >= D) continue;
+      float* h = reinterpret_cast<float*>(&b.h[c]);
+      const float* v = reinterpret_cast<const float*>(&yv[c]);
+      float w4[4] = {1.f, 1.f, 1.f, 1.f};
+      if (w_post != nullptr) scales(w_post, w_post_dtype, plus_one_post, d, w4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        h[e] += w_post != nullptr ? v[e] * r * w4[e] : v[e];
+        ss2 += h[e] * h[e];
+      }
+      *reinterpret_cast<float4*>(residual + rb + d) = b.h[c];
+    }
+    if (w_next == nullptr) return;
+    const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(D) + eps_next);
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int d = c * 256 + lane * 4;
+      if (d >= D) continue;
+      const float* h = reinterpret_cast<const float*>(&b.h[c]);
+      float w4[4], o[4];
+      scales(w_next, w_next_dtype, plus_one_next, d, w4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = h[e] * r2 * w4[e];
+      if constexpr (sizeof(OT) == 4) {
+        *reinterpret_cast<float4*>(out + rb + d) = float4{o[0], o[1], o[2], o[3]};
+      } else {
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(float_to_bf16(o[0]).bits) | (static_cast<uint32_t>(float_to_bf16(o[1]).bits) << 16);
+        packed.y = static_cast<uint32_t>(float_to_bf16(o[2]).bits) | (static_cast<uint32_t>(float_to_bf16(o[3]).bits) << 16);
+        *reinterpret_cast<uint2*>(out + rb + d) = packed;
+      }
+    }
+  };
+  Row b0;
+  load(row0, b0);
+  if constexpr (NCH <= 10) {
+    Row b1;
+    for (int i = 0; i < nrows; i += 2) {
+      if (i + 1 < nrows) load(row0 + i + 1, b1);
+      process(row0 + i, b0);
+      if (i + 2 < nrows) load(row0 + i + 2, b0);
+      if (i + 1 < nrows) process(row0 + i + 1, b1);
+    }
+  } else {
+    for (int i = 0; i < nrows; ++i) {
+      if (i > 0) load(row0 + i, b0);
+      process(row0 + i, b0);
     }
   }
 }
@@ -547,11 +581,16 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
   if (T >= 512 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out) &&
       aligned16(w_post) && aligned16(w_next)) {
     const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
-    const int blocks = (T + 3) / 4;
-#define SA_ROWS(YT, OT, NCH)                                                                                      \
-  add_rmsnorm_rows_kernel<YT, OT, NCH><<<blocks, 256, 0, stream>>>(static_cast<const YT*>(y), w_post, w_post_dtype, \
-                                                                   eps_post, pp, residual, w_next, w_next_dtype,    \
-                                                                   eps_next, pn, static_cast<OT*>(out), T, D)
+    // rows of a wave: enough waves for two per compute unit first, then up to four rows each
+    // two rows to a wave once that still leaves two waves for every SIMD (measured: more rows to a wave are slower,
+    // a wave takes about 5 us for a row); rows of more than 2560 elements do not fit twice into the registers
+    const int rows_per_wave = T >= 1024 && D <= 2560 ? 2 : 1;
+    const int blocks = (T + rows_per_wave - 1) / rows_per_wave;
+#define SA_ROWS(YT, OT, NCH)                                                                                     \
+  add_rmsnorm_rows_kernel<YT, OT, NCH><<<blocks, 64, 0, stream>>>(static_cast<const YT*>(y), w_post, w_post_dtype, \
+                                                                  eps_post, pp, residual, w_next, w_next_dtype,    \
+                                                                  eps_next, pn, static_cast<OT*>(out), T, D,       \
+                                                                  rows_per_wave)
 #define SA_ROWS_N(YT, OT)     \
   do {                        \
     if (D <= 2560) SA_ROWS(YT, OT, 10); \
