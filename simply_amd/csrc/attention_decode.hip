@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   if (wave == 0) take(0);
 
   const int KS = num_splits;
-  const size_t row_words = HD + 2;  // output, maximum, sum
+  const size_t row_words = HD + kRowExtra;  // output, maximum, sum
   const size_t unit = (static_cast<size_t>(blockIdx.z) * Kh + kh);
   if (wave == 0 && row_ok) {
     if (KS == 1) {
@@ -278,10 +278,11 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
                                                                     int G) {
   __shared__ float w_s[kMaxSplits];
   __shared__ float scratch[16];
+  __shared__ float4 part_s[256];
   const int tid = threadIdx.x, kh = blockIdx.x, z = blockIdx.y, orow = blockIdx.z;
   const SeqMeta sm = seq_meta[seq_begin + z];
   if (orow >= G * sm.q_len) return;
-  const size_t row_words = HD + 2;
+  const size_t row_words = HD + kRowExtra;
   const size_t unit = static_cast<size_t>(z) * Kh + kh;
   const float* base = workspace + (unit * KS * 16 + orow) * row_words;
   const size_t stride = 16 * row_words;
@@ -295,14 +296,38 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
   const float wy = my == -INFINITY ? 0.f : __expf(my - Mg);
   if (tid < KS) w_s[tid] = wy;
   const float Lg = block_sum(ly * wy, scratch + 4);  // has its own barriers; w_s is complete after them
+  // The threads are `parts` groups of HD / 4: group p adds up ranges p, p + parts, ... for four dimensions per
+  // thread (the loads of a thread do not depend on each other), then group 0 adds the groups up in order.
+  const int quarter = HD / 4, parts = 256 / quarter;
+  const int c = tid % quarter, part = tid / quarter;
+  float4 o = {0.f, 0.f, 0.f, 0.f};
+  if (part < parts) {
+    for (int y = part; y < KS; y += parts) {
+      const float4 v = *reinterpret_cast<const float4*>(base + y * stride + 4 * c);
+      const float w = w_s[y];
+      o.x += v.x * w;
+      o.y += v.y * w;
+      o.z += v.z * w;
+      o.w += v.w * w;
+    }
+    part_s[tid] = o;
+  }
+  __syncthreads();
+  if (part != 0) return;
+  for (int p = 1; p < parts; ++p) {
+    const float4 v = part_s[p * quarter + c];
+    o.x += v.x;
+    o.y += v.y;
+    o.z += v.z;
+    o.w += v.w;
+  }
   const int oq = orow / G, og = orow % G;
   bf16* op = out + static_cast<size_t>(sm.q_start + oq) * out_stride + static_cast<size_t>(kh * G + og) * HD;
   const float inv = 1.f / Lg;
-  for (int d = tid; d < HD; d += 256) {
-    float o = 0.f;
-    for (int y = 0; y < KS; ++y) o += base[y * stride + d] * w_s[y];
-    op[d] = float_to_bf16(o * inv);
-  }
+  op[4 * c] = float_to_bf16(o.x * inv);
+  op[4 * c + 1] = float_to_bf16(o.y * inv);
+  op[4 * c + 2] = float_to_bf16(o.z * inv);
+  op[4 * c + 3] = float_to_bf16(o.w * inv);
 }
 
 bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q) {
@@ -331,7 +356,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   if (KS > max_tiles) KS = max_tiles;
   if (KS > kMaxSplits) KS = kMaxSplits;
   if (KS < 1) KS = 1;
-  const size_t per_split = static_cast<size_t>(units) * 16 * (hd + 2) * sizeof(float);
+  const size_t per_split = static_cast<size_t>(units) * 16 * (hd + kRowExtra) * sizeof(float);
   while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
   const dim3 grid(KS, Kh, seq_count);
   const bf16* qp = static_cast<const bf16*>(q);
@@ -367,7 +392,7 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
   const SeqMeta sm = seq_meta[seq_begin + z];
   const int orow = tid / 16, part = tid % 16;
   if (orow >= G * sm.q_len) return;
-  const size_t row_words = HD + 2;
+  const size_t row_words = HD + kRowExtra;
   const size_t unit = static_cast<size_t>(z) * Kh + kh;
   const float* base = workspace + (unit * KS * 16 + orow) * row_words;
   const size_t stride = 16 * row_words;
@@ -386,13 +411,11 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
     for (int y = 0; y < KS; ++y) {
       const float my = base[y * stride + HD];
       const float wy = my == -INFINITY ? 0.f : __expf(my - Mg);
-      // rows are HD + 2 words long: a piece of four is 8-byte aligned
-      const float2 lo = *reinterpret_cast<const float2*>(base + y * stride + d);
-      const float2 hi = *reinterpret_cast<const float2*>(base + y * stride + d + 2);
-      o[0] += lo.x * wy;
-      o[1] += lo.y * wy;
-      o[2] += hi.x * wy;
-      o[3] += hi.y * wy;
+      const float4 v = *reinterpret_cast<const float4*>(base + y * stride + d);
+      o[0] += v.x * wy;
+      o[1] += v.y * wy;
+      o[2] += v.z * wy;
+      o[3] += v.w * wy;
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) op[d + e] = float_to_bf16(o[e] * inv);

@@ -345,7 +345,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
       }
     } else {
       // the merge kernel works with natural logarithms
-      const size_t row_words = HD + 2;
+      const size_t row_words = HD + kRowExtra;
       const size_t unit = static_cast<size_t>(group * GROUP + wave * R + j) * Kh + kh;
       float* wp = workspace + ((unit * num_splits + split) * 16 + r) * row_words;
 #pragma unroll
@@ -394,7 +394,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   if (KS > max_tiles) KS = max_tiles;
   if (KS > kMaxSplits) KS = kMaxSplits;
   if (KS < 1) KS = 1;
-  const size_t per_split = static_cast<size_t>(unit_count) * Kh * 16 * (hd + 2) * sizeof(float);
+  const size_t per_split = static_cast<size_t>(unit_count) * Kh * 16 * (hd + kRowExtra) * sizeof(float);
   while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
   const dim3 grid(KS, Kh, groups);
   const bf16* qp = static_cast<const bf16*>(q);

@@ -2,8 +2,8 @@
 // that the vector memory path is no longer the bound: the 128 x 128 tiles of the tiled kernel pull 96 KiB per
 // slab of 64 columns through a CU's 64 bytes a clock, which caps it at about a third of the MFMA rate.
 //
-// A workgroup of eight waves (one per CU) owns 256 x 192, 256 x 128, 128 x 256 or 192 x 128 outputs and takes both
-// operands through LDS, in slabs of 64 columns of K that go round two or three buffers, with loads that go from
+// A workgroup of eight waves (one per CU) owns 256 x 192, 256 x 128, 128 x 256 or 192 x 128 outputs (or one of four
+// waves, two per CU, 128 x 192) and takes both operands through LDS, in slabs of 64 columns of K that go round two or three buffers, with loads that go from
 // global memory straight into LDS (no registers in between).
 //   * Layout in LDS: W as KiB blocks in MFMA operand order (16 rows x 32 columns, lane l holds row l % 16,
 //     columns 8 (l / 16) ..), which is how it lies in global memory, so a block is a copy.  A as rows of 128 bytes
@@ -31,7 +31,6 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 namespace wide {
 
-constexpr int kWaves = 8;
 constexpr int BK = 64;
 constexpr int kCUs = 256;  // compute units of an MI355X
 
@@ -59,17 +58,17 @@ __device__ __forceinline__ void load_to_lds(const bf16* base, uint32_t offset, u
 }
 
 // WM x WN: 16 x 16 tiles of a wave (rows of A x rows of W); WAVES_M x (8 / WAVES_M) waves.
-template <int WM, int WN, int WAVES_M, int EPI, int NSTAGE>
-__global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__ A, int64_t lda,
+template <int WM, int WN, int WAVES_M, int EPI, int NSTAGE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __restrict__ A, int64_t lda,
                                                         const bf16* __restrict__ W, bf16* __restrict__ C, int64_t ldc,
                                                         int M, int N, int K, int chunks) {
-  constexpr int WAVES_N = kWaves / WAVES_M;
+  constexpr int WAVES_N = WAVES / WAVES_M;
   constexpr int MT = WAVES_M * WM, NT = WAVES_N * WN;  // 16-row tiles of A and of W per workgroup
   constexpr int BM = MT * 16;
   constexpr int A_BLOCKS = MT * 2, W_BLOCKS = NT * 2;  // KiB blocks of a slab
-  static_assert(A_BLOCKS % kWaves == 0 && W_BLOCKS % kWaves == 0, "every wave copies the same number of blocks");
+  static_assert(A_BLOCKS % WAVES == 0 && W_BLOCKS % WAVES == 0, "every wave copies the same number of blocks");
   static_assert(EPI != 1 || WN % 2 == 0, "gate and factor tiles come in pairs");
-  constexpr int APW = A_BLOCKS / kWaves, WPW = W_BLOCKS / kWaves;
+  constexpr int APW = A_BLOCKS / WAVES, WPW = W_BLOCKS / WAVES;
   constexpr int STAGE = (A_BLOCKS + W_BLOCKS) * 512;  // elements
   __shared__ __attribute__((aligned(16))) __bf16 stages[NSTAGE * STAGE];
   const uint32_t lds_base = static_cast<uint32_t>(
@@ -102,7 +101,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__
   const int ntiles = (NW + 15) / 16;
   const int nt_base = bx * NT;
 
-  // ---- what this wave copies of every slab: KiB blocks wave + 8 i of A and of W.
+  // ---- what this wave copies of every slab: KiB blocks wave + WAVES i of A and of W.
   // A block b is rows 8 (b % 2) .. + 8 of tile b / 2, all 64 columns of the slab: eight lanes per row read its 128
   // bytes, so a load is eight whole lines.  In LDS a row's eight 16-byte pieces are permuted (piece p of row r of
   // the tile lies at p ^ (r / 2)), which makes the fragment reads below (16 rows, one piece each) hit all banks.
@@ -113,13 +112,13 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__
 #pragma unroll
   for (int i = 0; i < APW; ++i) {
     const int r = half_mine * 8 + lane / 8;  // row of the tile
-    const int m = m_base + (tile_mine + 4 * i) * 16 + r;
+    const int m = m_base + (tile_mine + (WAVES / 2) * i) * 16 + r;
     a_off[i] = (static_cast<uint32_t>(m < M ? m : M - 1) * static_cast<uint32_t>(lda) + ((lane % 8) ^ (r / 2)) * 8) * 2;
   }
   const bf16* w_from[WPW];  // the same for the whole wave
 #pragma unroll
   for (int i = 0; i < WPW; ++i) {
-    const int nt = nt_base + tile_mine + 4 * i;
+    const int nt = nt_base + tile_mine + (WAVES / 2) * i;
     const int clamped = __builtin_amdgcn_readfirstlane(nt < ntiles ? nt : ntiles - 1);
     w_from[i] = W + (static_cast<size_t>(clamped) * chunks + half_mine) * 512;
   }
@@ -128,10 +127,10 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__
   auto request_one = [&](int n, int slab, int buf) __attribute__((always_inline)) {
     const uint32_t to = lds_base + static_cast<uint32_t>(buf) * (STAGE * 2);
     if (n < APW)
-      load_to_lds(A + static_cast<size_t>(slab) * BK, a_off[n], to + ((tile_mine + 4 * n) * 2 + half_mine) * 1024);
+      load_to_lds(A + static_cast<size_t>(slab) * BK, a_off[n], to + ((tile_mine + (WAVES / 2) * n) * 2 + half_mine) * 1024);
     else
       load_to_lds(w_from[n - APW] + static_cast<size_t>(slab) * 1024, lane * 16,
-                  to + (A_BLOCKS + (tile_mine + 4 * (n - APW)) * 2 + half_mine) * 1024);
+                  to + (A_BLOCKS + (tile_mine + (WAVES / 2) * (n - APW)) * 2 + half_mine) * 1024);
   };
 
   floatx4 acc[WM][WN];
@@ -161,20 +160,24 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__
     for (int j = 0; j < WN; ++j)
       fw[kc][j] = *reinterpret_cast<const bf16x8*>(stage + ((A_BLOCKS + (wn * WN + j) * 2 + kc) * 64 + lane) * 8);
   };
-  static_assert(LOADS <= 2 * WM, "a load after each row of products");
-  // The products of half kc; after row i of them load first + i of slab `slab` is asked for (if there is one): the
-  // loads of a slab are spread over its products, so that the waves do not queue up at the memory pipeline
-  // (which takes 16 cycles for each) while the MFMA unit idles.
+  // The products of half kc; after each row of them the next PER_ROW loads of slab `slab`, from load `first` on, are
+  // asked for (if there are any left): the loads of a slab are spread over its products, so that the waves do not
+  // queue up at the memory pipeline (which takes 16 cycles for each) while the MFMA unit idles.
+  constexpr int PER_ROW = (LOADS + 2 * WM - 1) / (2 * WM);
   auto multiply = [&](int kc, int first, int slab, int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
 #pragma unroll
       for (int j = 0; j < WN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kc][j], fa[kc][i], acc[i][j], 0, 0, 0);
-      if (first >= 0 && first + i < LOADS) {
-        __builtin_amdgcn_sched_barrier(0);
-        request_one(first + i, slab, buf);
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < PER_ROW; ++e) {
+        const int n = first + i * PER_ROW + e;
+        if (first >= 0 && n < LOADS) {
+          __builtin_amdgcn_sched_barrier(0);
+          request_one(n, slab, buf);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
   };
@@ -206,7 +209,7 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__
     __builtin_amdgcn_sched_barrier(0);  // (reads moved up among these products would need registers of their own)
     read(stage, 1);
     __builtin_amdgcn_sched_barrier(0);
-    multiply(0, WM, ahead, target);
+    multiply(0, WM * PER_ROW, ahead, target);
     target = cur;
     cur = cur + 1 == NSTAGE ? 0 : cur + 1;
   }
@@ -243,16 +246,16 @@ __global__ __launch_bounds__(512) void gemm_wide_kernel(const bf16* __restrict__
   }
 }
 
-template <int WM, int WN, int WAVES_M, int NSTAGE>
+template <int WM, int WN, int WAVES_M, int NSTAGE, int WAVES = 8>
 static void launch(const bf16* A, int64_t lda, const bf16* W, bf16* C, int64_t ldc, int M, int N, int K, int epi,
                    hipStream_t stream) {
-  constexpr int BM = WAVES_M * WM * 16, BNW = (kWaves / WAVES_M) * WN * 16;
+  constexpr int BM = WAVES_M * WM * 16, BNW = (WAVES / WAVES_M) * WN * 16;
   const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM);
   if (epi == 1)
-    gemm_wide_kernel<WM, WN, WAVES_M, 1, NSTAGE><<<grid, 512, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
+    gemm_wide_kernel<WM, WN, WAVES_M, 1, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
   else
-    gemm_wide_kernel<WM, WN, WAVES_M, 0, NSTAGE><<<grid, 512, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
+    gemm_wide_kernel<WM, WN, WAVES_M, 0, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
 }
 
 }  // namespace wide
@@ -266,21 +269,25 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
 }
 
 // shape: 0: chosen here; else stages * 1000000 + rows * 1000 + weight rows of a workgroup's tile (2256192, 3256128,
-// 3128256, 3192128).
+// 3128256, 3192128; 2128192: workgroups of four waves, two to a CU).
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
               hipStream_t stream) {
   const bf16* a = static_cast<const bf16*>(A);
   const bf16* w = static_cast<const bf16*>(W);
   bf16* c = static_cast<bf16*>(C);
   if (shape == 0) {
-    // one workgroup per CU at a time: the cost of a shape is its rounds over the CUs times the size of its tile;
-    // of equals the first (256 x 192 has the least traffic per product)
+    // The cost of a shape: the workgroups that the busiest CU gets times the size of the tile; of equals the first.
+    // Workgroups of four waves run two to a CU, where one's epilogue and first loads overlap the other's
+    // products (measured: 7-9 % faster than one workgroup of twice the tile once every CU has two of them;
+    // slower when it has one).
     const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-    const int shapes[4][3] = {{2256192, 256, 192}, {3256128, 256, 128}, {3128256, 128, 256}, {3192128, 192, 128}};
+    const int shapes[5][4] = {{2128192, 128, 192, 93}, {2256192, 256, 192, 100}, {3256128, 256, 128, 100},
+                              {3128256, 128, 256, 100}, {3192128, 192, 128, 100}};
     int64_t best = -1;
     for (const auto& sh : shapes) {
       const int64_t tiles = static_cast<int64_t>((M + sh[1] - 1) / sh[1]) * ((NW + sh[2] - 1) / sh[2]);
-      const int64_t cost = ((tiles + wide::kCUs - 1) / wide::kCUs) * sh[1] * sh[2];
+      if (sh[3] < 100 && tiles < 2 * wide::kCUs) continue;
+      const int64_t cost = ((tiles + wide::kCUs - 1) / wide::kCUs) * sh[1] * sh[2] * sh[3];
       if (best < 0 || cost < best) {
         best = cost;
         shape = sh[0];
@@ -292,6 +299,7 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
     case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
     case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
+    case 2128192: wide::launch<4, 6, 2, 2, 4>(a, lda, w, c, ldc, M, N, K, epi, stream); break;  // two workgroups per CU
     default:
       set_error("gemm: unknown wide tile %d", shape);
       return 1;

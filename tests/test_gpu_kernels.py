@@ -406,7 +406,7 @@ def test_gemm_wide(M, N, K):
     tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
     t = dict(rtol=2e-2, atol=2e-2)
     want, want_gated = ref.gemm(a, w).float(), ref.gemm(a, w, w2=w2).float()
-    for shape in (0, 2256192, 3256128, 3128256, 3192128):
+    for shape in (0, 2256192, 3256128, 3128256, 3192128, 2128192):
         kw = dict(algo=ops.ALGO_WIDE, shape=shape)
         torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), want, **t)
         torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), want_gated, **t)
