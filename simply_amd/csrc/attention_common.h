@@ -23,10 +23,36 @@ __device__ inline __bf16 to_bf16_raw(float f) { return static_cast<__bf16>(f); }
 
 // Partial results of key ranges lie in the workspace as [unit * Kh + kh][range][16 rows][hd + kRowExtra] floats:
 // the unnormalised output, then the maximum and the sum of the row (and two unused words: rows stay 16-byte
-// aligned).  Adds them up, range by range in order, into `out`.
-// max_q_len: the most tokens in a unit.
+// aligned).  Adds them up, range by range in order, into `out`.  max_q_len: the most tokens in a unit.
+// chunk_tiles == 0: every unit has all num_ranges ranges.  chunk_tiles > 0: units come in groups of `group`, a
+// group's keys (what some row of it sees, with `window`) are cut into ranges of chunk_tiles tiles of kTile keys,
+// as many as it takes (num_ranges at most); a group with one range has written `out` itself and is skipped.
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
                            int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
-                           hipStream_t stream);
+                           hipStream_t stream, int chunk_tiles = 0, int group = 1, int window = 0);
+
+// The keys [lo, hi) that some row of the units [first, first + group) sees, and their request's slot.  False: no
+// rows.
+__device__ inline bool group_keys(const SeqMeta* units, int first, int group, int window, int* lo, int* hi, int* slot) {
+  int lo_g = 0x7fffffff, hi_g = 0;
+  for (int w = 0; w < group; ++w) {
+    const SeqMeta m = units[first + w];
+    if (m.q_len > 0) {
+      const int lo_w = (window > 0 && m.pos0 - window + 1 > 0) ? m.pos0 - window + 1 : 0;
+      lo_g = lo_w < lo_g ? lo_w : lo_g;
+      hi_g = m.pos0 + m.q_len > hi_g ? m.pos0 + m.q_len : hi_g;
+      *slot = m.slot;
+    }
+  }
+  *lo = lo_g;
+  *hi = hi_g;
+  return hi_g != 0;
+}
+
+// How many ranges of chunk_tiles tiles of kTile keys the keys [lo, hi) are cut into.
+__device__ inline int key_chunks(int lo, int hi, int chunk_tiles) {
+  const int tiles = (hi + kTile - 1) / kTile - lo / kTile;
+  return (tiles + chunk_tiles - 1) / chunk_tiles;
+}
 
 }  // namespace sa

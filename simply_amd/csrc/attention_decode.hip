@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ workspace, int KS, int HD,
                                                                     const SeqMeta* __restrict__ seq_meta, int seq_begin,
                                                                     bf16* __restrict__ out, int64_t out_stride, int Kh,
-                                                                    int G) {
+                                                                    int G, int chunk_tiles, int group, int window) {
   __shared__ float w_s[kMaxSplits];
   __shared__ float scratch[16];
   __shared__ float4 part_s[256];
@@ -286,6 +286,12 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
   const size_t unit = static_cast<size_t>(z) * Kh + kh;
   const float* base = workspace + (unit * KS * 16 + orow) * row_words;
   const size_t stride = 16 * row_words;
+  if (chunk_tiles > 0) {  // the ranges that this unit's group has; one: it has written its output itself
+    int lo, hi, slot;
+    group_keys(seq_meta, seq_begin + z / group * group, group, window, &lo, &hi, &slot);
+    KS = key_chunks(lo, hi, chunk_tiles);
+    if (KS <= 1) return;
+  }
   const float my = tid < KS ? base[tid * stride + HD] : -INFINITY;
   const float ly = tid < KS ? base[tid * stride + HD + 1] : 0.f;
   // maximum over the ranges
@@ -387,7 +393,8 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
 __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const float* __restrict__ workspace, int KS,
                                                                          int HD, const SeqMeta* __restrict__ seq_meta,
                                                                          int seq_begin, bf16* __restrict__ out,
-                                                                         int64_t out_stride, int Kh, int G) {
+                                                                         int64_t out_stride, int Kh, int G,
+                                                                         int chunk_tiles, int group, int window) {
   const int tid = threadIdx.x, kh = blockIdx.x, z = blockIdx.y;
   const SeqMeta sm = seq_meta[seq_begin + z];
   const int orow = tid / 16, part = tid % 16;
@@ -396,6 +403,12 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
   const size_t unit = static_cast<size_t>(z) * Kh + kh;
   const float* base = workspace + (unit * KS * 16 + orow) * row_words;
   const size_t stride = 16 * row_words;
+  if (chunk_tiles > 0) {  // the ranges that this unit's group has; one: it has written its output itself
+    int lo, hi, slot;
+    group_keys(seq_meta, seq_begin + z / group * group, group, window, &lo, &hi, &slot);
+    KS = key_chunks(lo, hi, chunk_tiles);
+    if (KS <= 1) return;
+  }
   float Mg = -INFINITY;
   for (int y = 0; y < KS; ++y) Mg = fmaxf(Mg, base[y * stride + HD]);
   float Lg = 0.f;
@@ -424,16 +437,16 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
 
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
                            int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
-                           hipStream_t stream) {
+                           hipStream_t stream, int chunk_tiles, int group, int window) {
   const int max_rows = G * max_q_len < 16 ? G * max_q_len : 16;
-  if (max_rows > 4 && num_ranges <= 4) {
-    paged_attention_merge_rows_kernel<<<dim3(Kh, unit_count), 256, 0, stream>>>(workspace, num_ranges, hd, units,
-                                                                               unit_begin, out, out_stride, Kh, G);
+  if (max_rows > 4 && num_ranges <= 64) {
+    paged_attention_merge_rows_kernel<<<dim3(Kh, unit_count), 256, 0, stream>>>(
+        workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window);
     return check_launch("paged_attention_merge_rows");
   }
   // one workgroup per row: rows beyond the longest unit's are not launched
-  paged_attention_merge_kernel<<<dim3(Kh, unit_count, max_rows), 256, 0, stream>>>(workspace, num_ranges, hd, units, unit_begin,
-                                                                            out, out_stride, Kh, G);
+  paged_attention_merge_kernel<<<dim3(Kh, unit_count, max_rows), 256, 0, stream>>>(
+      workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window);
   return check_launch("paged_attention_merge");
 }
 

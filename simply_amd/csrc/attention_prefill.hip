@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
-    float* __restrict__ workspace) {
+    float* __restrict__ workspace, int chunk_tiles) {
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;            // output blocks of 16 dimensions
   constexpr int CPW = NDC / 2;            // KiB chunks of keys (and of values) per wave and tile
@@ -74,23 +74,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const int group = gridDim.z - 1 - blockIdx.z;
   const int u0 = unit_begin + group * GROUP;
 
-  // the keys that some row of the workgroup sees: [lo_g, hi_g)
-  int lo_g = 0x7fffffff, hi_g = 0, slot = 0;
-  for (int w = 0; w < GROUP; ++w) {
-    const SeqMeta m = units[u0 + w];
-    if (m.q_len > 0) {
-      const int lo_w = (window > 0 && m.pos0 - window + 1 > 0) ? m.pos0 - window + 1 : 0;
-      lo_g = lo_w < lo_g ? lo_w : lo_g;
-      hi_g = m.pos0 + m.q_len > hi_g ? m.pos0 + m.q_len : hi_g;
-      slot = m.slot;
-    }
-  }
-  if (hi_g == 0) return;  // no rows at all (uniform over the workgroup)
-  const int* table = block_table + static_cast<size_t>(__builtin_amdgcn_readfirstlane(slot)) * table_stride;
+  // the keys that some row of the workgroup sees, in ranges of chunk_tiles tiles: this workgroup takes range `split`
+  int lo_g, hi_g, slot = 0;
+  if (!group_keys(units, u0, GROUP, window, &lo_g, &hi_g, &slot)) return;  // no rows at all
   const int tile0 = lo_g / kTile, tile1 = (hi_g + kTile - 1) / kTile;
-  const int ntiles = tile1 - tile0;
-  const int tb = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * split / num_splits);
-  const int te = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * (split + 1) / num_splits);
+  const int num_chunks = key_chunks(lo_g, hi_g, chunk_tiles);
+  if (split >= num_chunks) return;  // (the same for the whole workgroup)
+  const int* table = block_table + static_cast<size_t>(__builtin_amdgcn_readfirstlane(slot)) * table_stride;
+  const int tb = tile0 + split * chunk_tiles;
+  const int te = tb + chunk_tiles < tile1 ? tb + chunk_tiles : tile1;
 
   // this wave's R units and this lane's row of each: query token qi, query head g of the group
   const int qi = r / G, g = r % G;
@@ -334,7 +326,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
     if (!row_ok[j]) continue;
-    if (num_splits == 1) {
+    if (num_chunks == 1) {
       bf16* op = out + static_cast<size_t>(q_row[j]) * out_stride + static_cast<size_t>(kh * G + g) * HD;
       const float inv = 1.f / l;
 #pragma unroll
@@ -384,18 +376,31 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   int span = window > 0 && window < max_kv_len ? window + 16 * kGroup : max_kv_len;  // keys a workgroup reads at most
   if (span < 1) span = 1;
   const int max_tiles = (span + kTile - 1) / kTile + 1;
-  int KS = num_splits;
-  if (KS <= 0) {
-    const int wgs = groups * Kh;
-    KS = wgs >= 384 ? 1 : (512 + wgs / 2) / wgs;  // about two workgroups per CU at least: they fill each other's waits
-    const int cap_by_work = (max_tiles + 15) / 16;  // at least 16 tiles (512 keys) per workgroup
-    if (KS > cap_by_work) KS = cap_by_work;
+  // Ranges of `chunk` tiles, as many as a group's keys take.  Measured: best is one round of about two workgroups
+  // per CU (every further range costs a set-up, and 16 KiB of partial results per unit and head written and read
+  // again), with ranges of 16 tiles at least.  How many workgroups there will be is estimated from the tokens of
+  // this launch: the groups of a fresh prompt see from a tile to all of it (half on average), a portion late in a
+  // long prompt sees all of its history in every group.
+  int chunk;
+  if (num_splits > 0) {
+    chunk = (max_tiles + num_splits - 1) / num_splits;
+  } else {
+    const int64_t tokens = static_cast<int64_t>(unit_count) * max_q_len;
+    const int64_t avg_keys = span - (tokens < span ? tokens : span) / 2;
+    const int64_t avg_tiles = avg_keys / kTile + 1;
+    const int64_t pairs = static_cast<int64_t>(groups) * Kh;
+    int64_t ranges = 512 * static_cast<int64_t>(max_tiles) / (pairs * avg_tiles);
+    if (ranges > max_tiles / 16) ranges = max_tiles / 16;
+    if (ranges < 1) ranges = 1;
+    chunk = static_cast<int>((max_tiles + ranges - 1) / ranges);
   }
-  if (KS > max_tiles) KS = max_tiles;
-  if (KS > kMaxSplits) KS = kMaxSplits;
-  if (KS < 1) KS = 1;
+  if (chunk > max_tiles) chunk = max_tiles;
+  int KS = (max_tiles + chunk - 1) / chunk;
   const size_t per_split = static_cast<size_t>(unit_count) * Kh * 16 * (hd + kRowExtra) * sizeof(float);
-  while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
+  while (KS > 1 && (KS > kMaxSplits || workspace == nullptr || per_split * KS > workspace_bytes)) {
+    ++chunk;
+    KS = (max_tiles + chunk - 1) / chunk;
+  }
   const dim3 grid(KS, Kh, groups);
   const bf16* qp = static_cast<const bf16*>(q);
   const bf16* kp = static_cast<const bf16*>(k_pages);
@@ -408,11 +413,11 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
     if (soft_cap > 0.f)                                                                                             \
       prefill::paged_attention_prefill_kernel<NDC, R, true><<<grid, 256, 0, stream>>>(                              \
           qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
-          soft_cap, ws);                                                                                            \
+          soft_cap, ws, chunk);                                                                                     \
     else                                                                                                            \
       prefill::paged_attention_prefill_kernel<NDC, R, false><<<grid, 256, 0, stream>>>(                             \
           qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
-          soft_cap, ws);                                                                                            \
+          soft_cap, ws, chunk);                                                                                     \
   } while (0)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
@@ -424,7 +429,8 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
 #undef SA_LAUNCH
   if (check_launch("paged_attention_prefill")) return 1;
   if (KS > 1)
-    return attention_merge_ranges(ws, KS, hd, um, unit_begin, unit_count, max_q_len, op, out_stride, Kh, G, stream);
+    return attention_merge_ranges(ws, KS, hd, um, unit_begin, unit_count, max_q_len, op, out_stride, Kh, G, stream, chunk,
+                                  kGroup, window);
   return 0;
 }
 

@@ -260,7 +260,7 @@ EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
 
 #: scratch memory for partial results (attention over key ranges, products with K cut over workgroups), one per
 #: device, allocated at first use; kernels on one stream use it one after the other
-WORKSPACE_BYTES = 64 << 20
+WORKSPACE_BYTES = 256 << 20
 _scratch: dict = {}
 
 
