@@ -57,6 +57,16 @@ def prefill_flops(cfg, T):
     return gemm + attn + 2 * D * V
 
 
+# BASELINE.json configs[3] and [4]: the larger shapes, for --shape
+SHAPES = {
+    "2b": {},
+    "9b": dict(hidden_size=3584, num_hidden_layers=42, num_attention_heads=16, num_key_value_heads=8, head_dim=256,
+               intermediate_size=14336, query_pre_attn_scalar=256),
+    "27b": dict(hidden_size=4608, num_hidden_layers=46, num_attention_heads=32, num_key_value_heads=16, head_dim=128,
+                intermediate_size=36864, query_pre_attn_scalar=144),
+}
+
+
 def sync():
     import torch
     torch.cuda.synchronize()
@@ -119,6 +129,33 @@ def run_prefill(model, cfg, tokens, reps, page_size, dtype):
     return min(times[1:])
 
 
+def run_requests(model, cfg, requests, prompt_min, prompt_max, new_tokens, page_size, dtype):
+    """A whole workload through the scheduler: `requests` prompts of uniform-random lengths, all submitted at once,
+    each generating `new_tokens` greedily (portions of prompts beside decoded tokens, continuous batching)."""
+    import torch
+    from simply_amd.engine.llm import LMInterface
+    from simply_amd.sampling import SamplingParams
+
+    g = torch.Generator().manual_seed(3)
+    lengths = torch.randint(prompt_min, prompt_max + 1, (requests,), generator=g).tolist()
+    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lengths]
+    lm = LMInterface(config=cfg, random_weights=0, activation_dtype=dtype, batch_size=requests,
+                     max_seq_len=prompt_max + new_tokens + 8, page_size=page_size, max_num_issue_tokens=2048, _model=model)
+    params = SamplingParams(temperature=0.0, max_decode_steps=new_tokens, ignore_eos=True)
+    lm.generate(prompts[:2], sampling_params=SamplingParams(temperature=0.0, max_decode_steps=4, ignore_eos=True))
+    sync()
+    before = dict(lm.stats)
+    t0 = time.perf_counter()
+    outs = lm.generate(prompts, sampling_params=params)
+    sync()
+    dt = time.perf_counter() - t0
+    assert all(len(o.output_token_ids) == new_tokens for o in outs)
+    stats = {k: lm.stats[k] - before.get(k, 0) for k in lm.stats if isinstance(lm.stats[k], (int, float))}
+    del lm
+    torch.cuda.empty_cache()
+    return dt, sum(lengths), requests * new_tokens, stats
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -131,6 +168,12 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
+    ap.add_argument("--requests", type=int, default=0,
+                    help="instead of timed decode steps: a workload of this many requests through the scheduler")
+    ap.add_argument("--prompt-min", type=int, default=128)
+    ap.add_argument("--prompt-max", type=int, default=4096)
+    ap.add_argument("--new-tokens", type=int, default=256)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -142,7 +185,7 @@ def main():
     from simply_amd.kernels import lib
 
     lib.load()
-    d = dict(GEMMA2_2B)
+    d = dict(GEMMA2_2B, **SHAPES[args.shape])
     full_layers = d["num_hidden_layers"]
     if args.layers:
         d["num_hidden_layers"] = args.layers
@@ -150,6 +193,21 @@ def main():
     tdtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     esize = 2 if args.dtype == "bfloat16" else 4
     model = random_model(cfg, 0, tdtype, torch.device("cuda:0"))
+
+    if args.requests:
+        dt, prompt_tokens, new_tokens, stats = run_requests(model, cfg, args.requests, args.prompt_min, args.prompt_max,
+                                                            args.new_tokens, args.page_size, args.dtype)
+        print(json.dumps({
+            "metric": "tokens/s of a workload (prompt and generated tokens, continuous batching)",
+            "value": round((prompt_tokens + new_tokens) / dt, 1), "unit": "tokens/s", "n_gpus": 1,
+            "generated_per_s": round(new_tokens / dt, 1), "seconds": round(dt, 3), "prompt_tokens": prompt_tokens,
+            "generated_tokens": new_tokens, "engine_steps": stats.get("steps"), "higher_is_better": True,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": {"model": f"gemma2-{args.shape}-shape", "layers": cfg.num_hidden_layers,
+                       "layers_of_full_model": full_layers, "requests": args.requests, "prompt_min": args.prompt_min,
+                       "prompt_max": args.prompt_max, "new_tokens": args.new_tokens, "page_size": args.page_size}}),
+              flush=True)
+        return
 
     dt, mean_kv = run_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, args.page_size, args.dtype)
     step_bytes = weight_bytes(cfg, esize) + args.batch * kv_bytes_per_request(cfg, mean_kv, esize)
@@ -169,11 +227,11 @@ def main():
             points[f"decode_b{b}"] = round(b / dtb, 1)
 
     out = {
-        "metric": "decode tokens/s (Gemma 2 2B shape, batch %d, context %d)" % (args.batch, args.context),
+        "metric": "decode tokens/s (Gemma 2 %s shape, batch %d, context %d)" % (args.shape.upper(), args.batch, args.context),
         "value": round(args.batch / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "config": {"model": "gemma2-2b-shape", "layers": cfg.num_hidden_layers, "layers_of_full_model": full_layers,
+        "config": {"model": f"gemma2-{args.shape}-shape", "layers": cfg.num_hidden_layers, "layers_of_full_model": full_layers,
                    "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,

@@ -45,9 +45,10 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
   SA_REQUIRE(algo >= 0 && algo <= 4, "gemm: unknown algorithm %d", algo);
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
-  // up to 16 rows, and up to 32 for products without the gated epilogue (measured: the few-rows kernel, whose waves
-  // read the activations from L2, beats the tiled one with K cut over workgroups there)
-  if (algo == 2 || (algo == 0 && bf16_in && (M <= 16 || (M <= 32 && epilogue != 1)))) {
+  // up to 16 rows, and up to 32 for products without the gated epilogue and with K below 4608 (measured at the
+  // 2B, 9B and 27B sizes: the few-rows kernel, whose waves read the activations from L2, beats the tiled one with
+  // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower)
+  if (algo == 2 || (algo == 0 && bf16_in && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4608)))) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
