@@ -20,7 +20,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 HBM_GBPS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
 
-# BASELINE.json configs[2]: Gemma 2 2B shape
+# the benchmark configuration: Gemma 2 2B layer sizes
 GEMMA2_2B = dict(
     architectures=["Gemma2ForCausalLM"], hidden_size=2304, num_hidden_layers=26, num_attention_heads=8,
     num_key_value_heads=4, head_dim=256, intermediate_size=9216, vocab_size=256000, rms_norm_eps=1e-6,
@@ -57,7 +57,7 @@ def prefill_flops(cfg, T):
     return gemm + attn + 2 * D * V
 
 
-# BASELINE.json configs[3] and [4]: the larger shapes, for --shape
+# the larger Gemma 2 layer sizes, for --shape
 SHAPES = {
     "2b": {},
     "9b": dict(hidden_size=3584, num_hidden_layers=42, num_attention_heads=16, num_key_value_heads=8, head_dim=256,
