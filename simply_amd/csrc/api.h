@@ -126,7 +126,7 @@ int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pa
 // One token per row of 32-bit logits.  temperature 0 or top_k 1: argmax.  top_k <= 0 and top_p >= 1: off.
 int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature, const int* top_k,
               const float* top_p, const uint64_t* seed, const int* counter, int* tokens, float* logprobs,
-              hipStream_t stream);
+              void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // Host function: one block of the Philox4x32-10 generator that sa_sample uses.
 void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* out4);

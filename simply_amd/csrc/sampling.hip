@@ -139,10 +139,45 @@ __device__ uint32_t radix_select(const float* __restrict__ row, int V, float inv
   return prefix;
 }
 
+// The greedy rows' largest entries, for kArgChunks equal parts of each row: one workgroup per (row, part), so that
+// a row of a large vocabulary is read by many compute units instead of one.  sample_kernel picks among the parts.
+constexpr int kArgChunks = 32, kArgThreads = 256;
+__global__ __launch_bounds__(kArgThreads) void argmax_parts_kernel(const float* __restrict__ logits, int64_t row_stride,
+                                                                  int V, const float* __restrict__ temperature,
+                                                                  const int* __restrict__ top_k,
+                                                                  ArgMax* __restrict__ parts) {
+  __shared__ ArgMax am_scratch[kArgThreads / kWave];
+  const int r = blockIdx.x, c = blockIdx.y;
+  if (!(temperature[r] == 0.f || top_k[r] == 1)) return;
+  const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
+  const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
+  ArgMax a{-INFINITY, 0x7fffffff};
+  if ((reinterpret_cast<uintptr_t>(row + lo) & 15u) == 0) {
+    const float4* row4 = reinterpret_cast<const float4*>(row + lo);
+    const int quads = (hi - lo) / 4;
+    for (int b = threadIdx.x; b < quads; b += blockDim.x) {
+      const float4 x = row4[b];
+      const int i = lo + 4 * b;
+      a = better(a, ArgMax{x.x, i});
+      a = better(a, ArgMax{x.y, i + 1});
+      a = better(a, ArgMax{x.z, i + 2});
+      a = better(a, ArgMax{x.w, i + 3});
+    }
+    for (int i = lo + 4 * quads + threadIdx.x; i < hi; i += blockDim.x) a = better(a, ArgMax{row[i], i});
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) a = better(a, ArgMax{row[i], i});
+  }
+  a = block_argmax(a, am_scratch);
+  if (threadIdx.x == 0) parts[static_cast<size_t>(r) * kArgChunks + c] = a;
+}
+
+// parts: what argmax_parts_kernel has left for the greedy rows, or null (they read their rows themselves).
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const uint64_t* __restrict__ seed,
-    const int* __restrict__ counter, int* __restrict__ tokens, float* __restrict__ logprobs) {
+    const int* __restrict__ counter, int* __restrict__ tokens, float* __restrict__ logprobs,
+    const ArgMax* __restrict__ parts) {
   __shared__ ArgMax am_scratch[kSampleThreads / kWave];
   __shared__ float f_scratch[kSampleThreads / kWave];
   __shared__ unsigned long long hist[256];
@@ -164,6 +199,15 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
   if (temp == 0.f || k == 1) {
     ArgMax a{-INFINITY, 0x7fffffff};
+    if (parts != nullptr) {
+      if (threadIdx.x < kArgChunks) a = parts[static_cast<size_t>(r) * kArgChunks + threadIdx.x];
+      a = block_argmax(a, am_scratch);
+      if (threadIdx.x == 0) {
+        tokens[r] = a.i;
+        logprobs[r] = 0.f;
+      }
+      return;
+    }
     for (int i = threadIdx.x; i < head; i += blockDim.x) a = better(a, ArgMax{row[i], i});
     for (int b = threadIdx.x; b < quads; b += blockDim.x) {
       const float4 x = row4[b];
@@ -252,12 +296,20 @@ using namespace sa;
 
 extern "C" int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature,
                          const int* top_k, const float* top_p, const uint64_t* seed, const int* counter, int* tokens,
-                         float* logprobs, hipStream_t stream) {
+                         float* logprobs, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (R == 0) return 0;
   SA_REQUIRE(R > 0 && V > 0 && row_stride >= V, "sample: bad sizes R=%d V=%d stride=%lld", R, V,
              (long long)row_stride);
+  // large vocabularies: the greedy rows are searched by kArgChunks workgroups each first
+  ArgMax* parts = nullptr;
+  if (V >= 16384 && workspace != nullptr &&
+      workspace_bytes >= static_cast<int64_t>(R) * kArgChunks * static_cast<int64_t>(sizeof(ArgMax))) {
+    parts = static_cast<ArgMax*>(workspace);
+    argmax_parts_kernel<<<dim3(R, kArgChunks), kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, parts);
+    if (check_launch("sample (parts)")) return 1;
+  }
   sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed, counter,
-                                                  tokens, logprobs);
+                                                  tokens, logprobs, parts);
   return check_launch("sample");
 }
 

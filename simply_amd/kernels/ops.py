@@ -531,8 +531,9 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if logprobs is None:
         logprobs = torch.empty(R, dtype=torch.float32, device=logits.device)
     _i32(tokens, "sample: tokens", R)
+    ws = _workspace(logits.device)
     _lib.call("sa_sample", _ptr(logits), stride, R, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seed),
-              _ptr(counter), _ptr(tokens), _ptr(logprobs), _stream())
+              _ptr(counter), _ptr(tokens), _ptr(logprobs), _ptr(ws), ws.numel(), _stream())
     return tokens, logprobs
 
 

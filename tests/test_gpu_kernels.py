@@ -467,6 +467,34 @@ def test_sampling_rows_at_odd_addresses():
         assert tok[r].item() == int(logits[r].argmax())
 
 
+@pytest.mark.parametrize("V,offset", [(16384, 0), (50001, 1), (256000, 0), (33333, 3)])
+def test_sampling_greedy_rows_of_a_large_vocabulary(V, offset):
+    """From 16384 entries on the greedy rows are searched in parts by many workgroups: the first of equal maxima
+    wins wherever it lies (a part's edge, the last entry, an unaligned row), and the other rows are sampled as
+    before."""
+    from simply_amd.kernels import ops
+    R = 6
+    wide = rand((R, V + 8), torch.float32, 95, 2.0)
+    logits = wide[:, offset:offset + V]
+    part = ((V + 31) // 32 + 3) // 4 * 4
+    top = 50.0
+    logits[0, V - 1] = top                                   # the last entry
+    logits[1, part - 1] = top; logits[1, part] = top         # equal maxima on both sides of a part's edge
+    logits[2, 7 * part + 5] = top; logits[2, 20 * part] = top; logits[2, 3] = top   # the first of three
+    logits[4, 0] = top
+    temperature = torch.tensor([0.0, 0.0, 0.0, 0.9, 1.0, 0.0]).cuda()
+    top_k = torch.tensor([-1, -1, -1, -1, 1, -1], dtype=torch.int32).cuda()   # row 4: greedy through top_k 1
+    top_p = torch.ones(R).cuda()
+    seed = torch.arange(R, dtype=torch.int64).cuda() + 3
+    counter = torch.zeros(R, dtype=torch.int32).cuda()
+    tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
+    rtok, rlp = ref.sample(logits, temperature, top_k, top_p, seed, counter)
+    assert tok.tolist() == rtok.tolist()
+    assert tok.tolist()[:3] == [V - 1, part - 1, 3] and tok[4].item() == 0
+    assert tok[5].item() == int(logits[5].argmax())
+    torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("M", [1, 8, 13, 16])
 @pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (4608, 64), (96, 40), (72, 64)])
 def test_gemm_normed(M, K, N):
