@@ -42,7 +42,7 @@ struct RotaryArgs {
   int H, Kh, hd, page_size;
 };
 
-// NCH: 256-element pieces of a row (K <= 256 * NCH)
+// NCH: 256-element pieces of a row (K <= 256 * NCH): 10, 14 or 18
 template <int EPI, int NCH>
 __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     const bf16* __restrict__ y, const float* __restrict__ h_in, float* __restrict__ h_out,
@@ -104,8 +104,10 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
   // both sets of fragments are asked for before the norms: a wave's share of a tile is two or three sets, so most
   // of the first tile is on its way while the norms are computed
   const int nseg = (c1 - c0 + kUnroll - 1) / kUnroll;  // sets of fragments per tile for this wave
+  // (rows of more than 3584 elements leave no registers for the second set during the norms)
+  constexpr bool kBothSetsFirst = NCH <= 14;
   load_set(0, c0);
-  if (nseg >= 2) load_set(1, c0 + kUnroll);
+  if (kBothSetsFirst && nseg >= 2) load_set(1, c0 + kUnroll);
 
   // ---- the two norms, one wave per row.  A lane holds 4 consecutive elements of each 256-element piece of the
   // row; all loads of a row are issued before the first use, so a row costs one trip to L2.
@@ -118,8 +120,11 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
       continue;
     }
     const size_t rb = static_cast<size_t>(m) * K;
+    // (rows of more than 2560 elements: the norms' scale factors are read where they are used, from L1 after the
+    // first row, instead of ahead with the row: the registers do not hold both)
+    constexpr bool kAhead = NCH <= 10;
     float4 hv[NCH];
-    bf16x4 yv[NCH], wpv[NCH], wnv[NCH];
+    bf16x4 yv[NCH], wpv[kAhead ? NCH : 1], wnv[kAhead ? NCH : 1];
     const bf16* wp16 = static_cast<const bf16*>(w_post);
     const bf16* wn16 = static_cast<const bf16*>(w_next);
 #pragma unroll
@@ -127,9 +132,19 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
       const int d = c * 256 + lane * 4;
       hv[c] = d < K ? *reinterpret_cast<const float4*>(h_in + rb + d) : float4{0.f, 0.f, 0.f, 0.f};
       yv[c] = (add && d < K) ? *reinterpret_cast<const bf16x4*>(y + rb + d) : bf16x4{};
-      wpv[c] = (post && d < K) ? *reinterpret_cast<const bf16x4*>(wp16 + d) : bf16x4{};
-      wnv[c] = d < K ? *reinterpret_cast<const bf16x4*>(wn16 + d) : bf16x4{};
+      if constexpr (kAhead) {
+        wpv[c] = (post && d < K) ? *reinterpret_cast<const bf16x4*>(wp16 + d) : bf16x4{};
+        wnv[c] = d < K ? *reinterpret_cast<const bf16x4*>(wn16 + d) : bf16x4{};
+      }
     }
+    auto post_scale = [&](int c, int d) __attribute__((always_inline)) {
+      if constexpr (kAhead) return wpv[c];
+      else return *reinterpret_cast<const bf16x4*>(wp16 + d);
+    };
+    auto next_scale = [&](int c, int d) __attribute__((always_inline)) {
+      if constexpr (kAhead) return wnv[c];
+      else return *reinterpret_cast<const bf16x4*>(wn16 + d);
+    };
     if (add) {
       float rr = 1.f;
       if (post) {
@@ -145,10 +160,11 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
         const int d = c * 256 + lane * 4;
         if (d >= K) continue;
         float* h = reinterpret_cast<float*>(&hv[c]);
+        const bf16x4 ws = post ? post_scale(c, d) : bf16x4{};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float v = static_cast<float>(yv[c][e]);
-          h[e] += post ? v * rr * (static_cast<float>(wpv[c][e]) + plus_post) : v;
+          h[e] += post ? v * rr * (static_cast<float>(ws[e]) + plus_post) : v;
         }
         if (blockIdx.x == 0) *reinterpret_cast<float4*>(h_out + rb + d) = hv[c];
       }
@@ -162,12 +178,14 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
       const int d = c * 256 + lane * 4;
       if (d >= K) continue;
       const float* h = reinterpret_cast<const float*>(&hv[c]);
+      const bf16x4 ws = next_scale(c, d);
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        dst[d + e] = float_to_bf16(h[e] * r2 * (static_cast<float>(wnv[c][e]) + plus_next));
+        dst[d + e] = float_to_bf16(h[e] * r2 * (static_cast<float>(ws[e]) + plus_next));
     }
     for (int d = K + lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
   }
+  if (!kBothSetsFirst && nseg >= 2) load_set(1, c0 + kUnroll);
   __syncthreads();
 
   for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -300,7 +318,7 @@ using namespace sa;
 
 extern "C" int sa_gemm_normed_takes(int M, int N, int K) {
   const size_t lds = static_cast<size_t>(M <= 8 ? 8 : 16) * (K + 8) * 2 + 8 * 2 * 16 * 17 * 4;
-  return M >= 1 && M <= 16 && K % 32 == 0 && K <= 256 * 10 && lds <= 160 * 1024;
+  return M >= 1 && M <= 16 && K % 32 == 0 && K <= 256 * 18 && lds <= 160 * 1024;
 }
 
 extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype,
@@ -308,7 +326,7 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
                               int plus_one_next, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
                               int epilogue, float cap, hipStream_t stream) {
   SA_REQUIRE(sa_gemm_normed_takes(M, N, K),
-             "gemm_normed takes 1..16 rows and a width that is a multiple of 32, at most 2560, and fits in LDS; got M=%d K=%d", M, K);
+             "gemm_normed takes 1..16 rows and a width that is a multiple of 32, at most 4608, and fits in LDS; got M=%d K=%d", M, K);
   SA_REQUIRE(N > 0 && ldc >= N && w_next != nullptr && h_in != nullptr && W != nullptr, "gemm_normed: bad arguments");
   SA_REQUIRE(w_next_dtype == kBF16 && (w_post == nullptr || w_post_dtype == kBF16),
              "gemm_normed: the norm weights must be bfloat16");
@@ -321,9 +339,16 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
 #define SA_NORMED(EPI, NCH)                                                                                      \
   return normed::launch<EPI, NCH>(yb, h_in, h_out, w_post, w_post_dtype, eps_post, pp, w_next, w_next_dtype, eps_next, \
                                   pn, w, C, c_dtype, ldc, M, N, K, cap, normed::RotaryArgs{}, stream)
-  if (epilogue == 0) SA_NORMED(0, 10);
-  if (epilogue == 1) SA_NORMED(1, 10);
-  SA_NORMED(2, 10);
+#define SA_NORMED_K(EPI)          \
+  do {                            \
+    if (K <= 2560) SA_NORMED(EPI, 10); \
+    if (K <= 3584) SA_NORMED(EPI, 14); \
+    SA_NORMED(EPI, 18);           \
+  } while (0)
+  if (epilogue == 0) SA_NORMED_K(0);
+  if (epilogue == 1) SA_NORMED_K(1);
+  SA_NORMED_K(2);
+#undef SA_NORMED_K
 #undef SA_NORMED
 }
 
@@ -341,7 +366,7 @@ extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_
              "gemm_normed_rotary: bad head counts, or a head size that is no multiple of 32 (H=%d K=%d hd=%d)", H, Kh, hd);
   const int N = (H + 2 * Kh) * hd;
   SA_REQUIRE(sa_gemm_normed_takes(M, N, K),
-             "gemm_normed takes 1..16 rows and a width that is a multiple of 32, at most 2560, and fits in LDS; got M=%d K=%d", M, K);
+             "gemm_normed takes 1..16 rows and a width that is a multiple of 32, at most 4608, and fits in LDS; got M=%d K=%d", M, K);
   SA_REQUIRE(ldc >= static_cast<int64_t>(H) * hd && w_next != nullptr && h_in != nullptr && W != nullptr && C != nullptr &&
                  positions != nullptr,
              "gemm_normed_rotary: bad arguments");
@@ -354,7 +379,12 @@ extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_
              "gemm_normed_rotary: slots come with key and value pages");
   normed::RotaryArgs rot{positions, timescale, 1.f / scale_factor, q_div, slot_mapping, static_cast<bf16*>(k_pages),
                          static_cast<bf16*>(v_pages), H, Kh, hd, page_size};
-  return normed::launch<3, 10>(static_cast<const bf16*>(y), h_in, h_out, w_post, w_post_dtype, eps_post,
-                               plus_one_post ? 1.f : 0.f, w_next, w_next_dtype, eps_next, plus_one_next ? 1.f : 0.f,
-                               static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, 0.f, rot, stream);
+#define SA_ROTARY(NCH)                                                                                              \
+  return normed::launch<3, NCH>(static_cast<const bf16*>(y), h_in, h_out, w_post, w_post_dtype, eps_post,             \
+                                plus_one_post ? 1.f : 0.f, w_next, w_next_dtype, eps_next, plus_one_next ? 1.f : 0.f, \
+                                static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, 0.f, rot, stream)
+  if (K <= 2560) SA_ROTARY(10);
+  if (K <= 3584) SA_ROTARY(14);
+  SA_ROTARY(18);
+#undef SA_ROTARY
 }

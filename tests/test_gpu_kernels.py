@@ -496,7 +496,8 @@ def test_sampling_greedy_rows_of_a_large_vocabulary(V, offset):
 
 
 @pytest.mark.parametrize("M", [1, 8, 13, 16])
-@pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (4608, 64), (96, 40), (72, 64)])
+@pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (3584, 512), (4608, 64), (4640, 64), (96, 40),
+                                 (72, 64)])
 def test_gemm_normed(M, K, N):
     """Residual sum, two norms and the product in one kernel against the separate references."""
     from simply_amd.kernels import ops
@@ -506,7 +507,7 @@ def test_gemm_normed(M, K, N):
     w, w2 = rand((N, K), torch.bfloat16, 104, 0.05), rand((N, K), torch.bfloat16, 105, 0.05)
     tw, tg = pack_tiles(w), pack_gate_up(w, w2)
     fits = (8 if M <= 8 else 16) * (K + 8) * 2 + 8 * 2 * 16 * 17 * 4 <= 160 * 1024   # activations and tiles in LDS
-    assert ops.gemm_normed_takes(M, tw) == (fits and K % 32 == 0 and K <= 2560)
+    assert ops.gemm_normed_takes(M, tw) == (fits and K % 32 == 0 and K <= 4608)
     if not ops.gemm_normed_takes(M, tw):
         return
     kw = dict(post_weight=wp, post_eps=1e-6, post_plus_one=True, next_weight=wn, next_eps=1e-5, next_plus_one=True)
