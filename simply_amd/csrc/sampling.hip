@@ -139,16 +139,13 @@ __device__ uint32_t radix_select(const float* __restrict__ row, int V, float inv
   return prefix;
 }
 
-// The greedy rows' largest entries, for kArgChunks equal parts of each row: one workgroup per (row, part), so that
-// a row of a large vocabulary is read by many compute units instead of one.  sample_kernel picks among the parts.
+// The rows' largest entries, for kArgChunks equal parts of each row: one workgroup per (row, part), so that a row
+// of a large vocabulary is read by many compute units instead of one.  sample_kernel picks among the parts.
 constexpr int kArgChunks = 32, kArgThreads = 256;
 __global__ __launch_bounds__(kArgThreads) void argmax_parts_kernel(const float* __restrict__ logits, int64_t row_stride,
-                                                                  int V, const float* __restrict__ temperature,
-                                                                  const int* __restrict__ top_k,
-                                                                  ArgMax* __restrict__ parts) {
+                                                                  int V, ArgMax* __restrict__ parts) {
   __shared__ ArgMax am_scratch[kArgThreads / kWave];
   const int r = blockIdx.x, c = blockIdx.y;
-  if (!(temperature[r] == 0.f || top_k[r] == 1)) return;
   const float* row = logits + static_cast<size_t>(r) * row_stride;
   const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
   const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
@@ -172,12 +169,64 @@ __global__ __launch_bounds__(kArgThreads) void argmax_parts_kernel(const float* 
   if (threadIdx.x == 0) parts[static_cast<size_t>(r) * kArgChunks + c] = a;
 }
 
-// parts: what argmax_parts_kernel has left for the greedy rows, or null (they read their rows themselves).
+// For the rows that are sampled from all of their entries (a temperature, no top-k, no top-p), again one workgroup
+// per (row, part): the part's largest entry with its noise added and the part's share of the softmax sum.  The
+// noise of an entry depends on the request's seed, its draw counter and the entry's number alone, so the parts
+// draw what one workgroup would.
+struct DrawPart {
+  ArgMax best;
+  float sum, unused;
+};
+__device__ inline bool draws_from_all(float temp, int k, float p) { return temp != 0.f && k <= 0 && p >= 1.f; }
+
+__global__ __launch_bounds__(kArgThreads) void draw_parts_kernel(const float* __restrict__ logits, int64_t row_stride,
+                                                                int V, const float* __restrict__ temperature,
+                                                                const int* __restrict__ top_k,
+                                                                const float* __restrict__ top_p,
+                                                                const uint64_t* __restrict__ seed,
+                                                                const int* __restrict__ counter,
+                                                                const ArgMax* __restrict__ parts,
+                                                                DrawPart* __restrict__ draws) {
+  __shared__ ArgMax am_scratch[kArgThreads / kWave];
+  __shared__ float f_scratch[kArgThreads / kWave];
+  const int r = blockIdx.x, c = blockIdx.y;
+  const float temp = temperature[r];
+  if (!draws_from_all(temp, top_k[r], top_p[r])) return;
+  const float inv_t = 1.f / temp;
+  float mx = -INFINITY;
+  for (int j = 0; j < kArgChunks; ++j) mx = fmaxf(mx, parts[static_cast<size_t>(r) * kArgChunks + j].v * inv_t);
+  const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
+  const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
+  const uint64_t sd = seed[r];
+  const uint32_t ctr = static_cast<uint32_t>(counter[r]);
+  ArgMax a{-INFINITY, 0x7fffffff};
+  float sum = 0.f;
+  // one generator block gives the noise of four consecutive entries (lo is a multiple of four)
+  for (int b = lo / 4 + threadIdx.x; 4 * b < hi; b += blockDim.x) {
+    float g[4];
+    gumbel_noise4(sd, ctr, static_cast<uint32_t>(b), g);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = 4 * b + j;
+      if (i >= hi) break;
+      const float x = row[i] * inv_t;
+      sum += expf(x - mx);
+      a = better(a, ArgMax{x + g[j], i});
+    }
+  }
+  a = block_argmax(a, am_scratch);
+  sum = block_sum(sum, f_scratch);
+  if (threadIdx.x == 0) draws[static_cast<size_t>(r) * kArgChunks + c] = DrawPart{a, sum, 0.f};
+}
+
+// parts: what argmax_parts_kernel has left for the rows, or null (they read their rows themselves); draws: what
+// draw_parts_kernel has left for the rows that are sampled from all of their entries.
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const uint64_t* __restrict__ seed,
     const int* __restrict__ counter, int* __restrict__ tokens, float* __restrict__ logprobs,
-    const ArgMax* __restrict__ parts) {
+    const ArgMax* __restrict__ parts, const DrawPart* __restrict__ draws) {
   __shared__ ArgMax am_scratch[kSampleThreads / kWave];
   __shared__ float f_scratch[kSampleThreads / kWave];
   __shared__ unsigned long long hist[256];
@@ -227,6 +276,24 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   }
 
   const float inv_t = 1.f / temp;
+  if (draws != nullptr && draws_from_all(temp, k, p)) {
+    float mx = -INFINITY, sum = 0.f;
+    ArgMax a{-INFINITY, 0x7fffffff};
+    if (threadIdx.x < kArgChunks) {
+      const DrawPart d = draws[static_cast<size_t>(r) * kArgChunks + threadIdx.x];
+      a = d.best;
+      sum = d.sum;
+      mx = parts[static_cast<size_t>(r) * kArgChunks + threadIdx.x].v * inv_t;
+    }
+    a = block_argmax(a, am_scratch);
+    mx = block_max(mx, f_scratch);
+    sum = block_sum(sum, f_scratch);
+    if (threadIdx.x == 0) {
+      tokens[r] = a.i;
+      logprobs[r] = row[a.i] * inv_t - mx - logf(sum);
+    }
+    return;
+  }
   float mx = -INFINITY;
   for (int i = threadIdx.x; i < head; i += blockDim.x) mx = fmaxf(mx, row[i] * inv_t);
   for (int b = threadIdx.x; b < quads; b += blockDim.x) {
@@ -302,14 +369,19 @@ extern "C" int sa_sample(const float* logits, int64_t row_stride, int R, int V, 
              (long long)row_stride);
   // large vocabularies: the greedy rows are searched by kArgChunks workgroups each first
   ArgMax* parts = nullptr;
+  DrawPart* draws = nullptr;
   if (V >= 16384 && workspace != nullptr &&
-      workspace_bytes >= static_cast<int64_t>(R) * kArgChunks * static_cast<int64_t>(sizeof(ArgMax))) {
-    parts = static_cast<ArgMax*>(workspace);
-    argmax_parts_kernel<<<dim3(R, kArgChunks), kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, parts);
+      workspace_bytes >= static_cast<int64_t>(R) * kArgChunks * static_cast<int64_t>(sizeof(ArgMax) + sizeof(DrawPart))) {
+    draws = static_cast<DrawPart*>(workspace);
+    parts = reinterpret_cast<ArgMax*>(draws + static_cast<size_t>(R) * kArgChunks);
+    argmax_parts_kernel<<<dim3(R, kArgChunks), kArgThreads, 0, stream>>>(logits, row_stride, V, parts);
     if (check_launch("sample (parts)")) return 1;
+    draw_parts_kernel<<<dim3(R, kArgChunks), kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p,
+                                                                      seed, counter, parts, draws);
+    if (check_launch("sample (draws)")) return 1;
   }
   sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed, counter,
-                                                  tokens, logprobs, parts);
+                                                  tokens, logprobs, parts, draws);
   return check_launch("sample");
 }
 
