@@ -124,8 +124,11 @@ int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pa
                                void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // One token per row of 32-bit logits.  temperature 0 or top_k 1: argmax.  top_k <= 0 and top_p >= 1: off.
+// modes: what some row may ask for, as a sum of 1 (a draw: a temperature other than 0), 2 (top-k) and 4 (top-p); 7
+// when that is not known.  A row that asks for what modes leaves out gets it all the same, from one workgroup.
+// workspace: scratch memory for the kernels that work on large vocabularies in parts (none: one workgroup per row).
 int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature, const int* top_k,
-              const float* top_p, const uint64_t* seed, const int* counter, int* tokens, float* logprobs,
+              const float* top_p, const uint64_t* seed, const int* counter, int* tokens, float* logprobs, int modes,
               void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // Host function: one block of the Philox4x32-10 generator that sa_sample uses.

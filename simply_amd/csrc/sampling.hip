@@ -17,6 +17,8 @@
 namespace sa {
 
 constexpr int kSampleThreads = 1024;
+// what the rows of a call may ask for (sa_sample's modes): a draw at all, top-k, top-p
+constexpr int kSampleDrawn = 1, kSampleTopK = 2, kSampleTopP = 4;
 
 struct Philox4 {
   uint32_t v[4];
@@ -142,10 +144,26 @@ __device__ uint32_t radix_select(const float* __restrict__ row, int V, float inv
 // The rows' largest entries, for kArgChunks equal parts of each row: one workgroup per (row, part), so that a row
 // of a large vocabulary is read by many compute units instead of one.  sample_kernel picks among the parts.
 constexpr int kArgChunks = 32, kArgThreads = 256;
+
+// What the selection of a row's top-k and top-p boundaries in parts keeps per row, in 64-bit words: the histograms
+// of the four passes by count and of the four by mass (added up over the parts with atomics, complete when the
+// kernel that adds them has ended), the mass of the entries that top-k leaves, and the selection's state after
+// 1 .. 4 choices (prefix of the key, count or mass above it) for both.
+constexpr int kSelCount = 0, kSelMass = 4 * 256, kSelTotal = 8 * 256, kSelCountState = kSelTotal + 2,
+              kSelMassState = kSelCountState + 10, kSelWords = kSelMassState + 10;
+__device__ inline bool is_greedy(float temp, int k) { return temp == 0.f || k == 1; }
+__device__ inline bool uses_top_k(float temp, int k) { return !is_greedy(temp, k) && k > 0; }
+__device__ inline bool uses_top_p(float temp, int k, float p) { return !is_greedy(temp, k) && p < 1.f; }
+
+// sel: null, or the rows' selection words, which are cleared here.
 __global__ __launch_bounds__(kArgThreads) void argmax_parts_kernel(const float* __restrict__ logits, int64_t row_stride,
-                                                                  int V, ArgMax* __restrict__ parts) {
+                                                                  int V, ArgMax* __restrict__ parts,
+                                                                  unsigned long long* __restrict__ sel) {
   __shared__ ArgMax am_scratch[kArgThreads / kWave];
   const int r = blockIdx.x, c = blockIdx.y;
+  if (sel != nullptr)
+    for (int i = c * kArgThreads + threadIdx.x; i < kSelWords; i += kArgChunks * kArgThreads)
+      sel[static_cast<size_t>(r) * kSelWords + i] = 0ull;
   const float* row = logits + static_cast<size_t>(r) * row_stride;
   const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
   const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
@@ -169,15 +187,158 @@ __global__ __launch_bounds__(kArgThreads) void argmax_parts_kernel(const float* 
   if (threadIdx.x == 0) parts[static_cast<size_t>(r) * kArgChunks + c] = a;
 }
 
-// For the rows that are sampled from all of their entries (a temperature, no top-k, no top-p), again one workgroup
-// per (row, part): the part's largest entry with its noise added and the part's share of the softmax sum.  The
-// noise of an entry depends on the request's seed, its draw counter and the entry's number alone, so the parts
-// draw what one workgroup would.
+// One choice of the selection (256 threads): from the complete histogram of a pass (bins of the key's next byte)
+// and what lies above the prefix chosen so far, the bin in which the target is reached, going down from the top
+// bin, and what lies above that bin (everything, with bin 0, if the target is beyond the total): what thread 0
+// of radix_select does in a loop, as a suffix sum over the bins.
+struct SelPos {
+  uint32_t prefix;
+  unsigned long long above;
+};
+__device__ inline SelPos choose_bin(const unsigned long long* __restrict__ hist, SelPos at, int pass,
+                                    unsigned long long target, unsigned long long* scan /* [256] LDS */,
+                                    int* chosen_s /* LDS */) {
+  const int b = threadIdx.x;
+  scan[b] = hist[b];
+  if (b == 0) *chosen_s = -1;
+  __syncthreads();
+  for (int o = 1; o < 256; o <<= 1) {
+    const unsigned long long v = b + o < 256 ? scan[b + o] : 0ull;
+    __syncthreads();
+    scan[b] += v;
+    __syncthreads();
+  }
+  if (at.above + scan[b] >= target) atomicMax(chosen_s, b);  // true for every bin from the chosen one down
+  __syncthreads();
+  const int chosen = *chosen_s;
+  SelPos out;
+  out.prefix = at.prefix | (static_cast<uint32_t>(chosen < 0 ? 0 : chosen) << (24 - 8 * pass));
+  out.above = at.above + (chosen < 0 ? scan[0] : chosen + 1 < 256 ? scan[chosen + 1] : 0ull);
+  __syncthreads();
+  return out;
+}
+// The state after `n` choices (1 .. 4): what an earlier kernel has stored after n - 1, and the choice from the
+// histogram of pass n - 1.  Part 0 of the row stores it for the kernels that follow.
+__device__ inline SelPos advance(unsigned long long* __restrict__ S, int hist_base, int state_base, int n,
+                                 unsigned long long target, unsigned long long* scan, int* chosen_s) {
+  SelPos at{0u, 0ull};
+  if (n > 1) {
+    at.prefix = static_cast<uint32_t>(S[state_base + 2 * (n - 1)]);
+    at.above = S[state_base + 2 * (n - 1) + 1];
+  }
+  const SelPos out = choose_bin(S + hist_base + (n - 1) * 256, at, n - 1, target, scan, chosen_s);
+  if (blockIdx.y == 0 && threadIdx.x == 0) {
+    S[state_base + 2 * n] = out.prefix;
+    S[state_base + 2 * n + 1] = out.above;
+  }
+  return out;
+}
+__device__ inline unsigned long long mass_of(float x, float mx) {
+  return static_cast<unsigned long long>(expf(x - mx) * 4294967296.0f);
+}
+
+// Pass `pass` (0 .. 3) of a selection, one workgroup per (row, part): the histogram of the next byte of the keys of
+// the part's entries whose key continues the prefix chosen so far, added to the row's.  by_mass 0: top-k (entries
+// count 1); 1: top-p (entries count their mass, among those that top-k leaves).
+__global__ __launch_bounds__(kArgThreads) void select_pass_kernel(const float* __restrict__ logits, int64_t row_stride,
+                                                                 int V, const float* __restrict__ temperature,
+                                                                 const int* __restrict__ top_k,
+                                                                 const float* __restrict__ top_p,
+                                                                 const ArgMax* __restrict__ parts,
+                                                                 unsigned long long* __restrict__ sel, int pass,
+                                                                 int by_mass) {
+  __shared__ unsigned long long hist[256], scan[256];
+  __shared__ int chosen_s;
+  const int r = blockIdx.x, c = blockIdx.y;
+  const float temp = temperature[r];
+  const int k = top_k[r];
+  const float p = top_p[r];
+  if (by_mass ? !uses_top_p(temp, k, p) : !uses_top_k(temp, k)) return;
+  unsigned long long* S = sel + static_cast<size_t>(r) * kSelWords;
+  const float inv_t = 1.f / temp;
+  float mx = -INFINITY;
+  for (int j = 0; j < kArgChunks; ++j) mx = fmaxf(mx, parts[static_cast<size_t>(r) * kArgChunks + j].v * inv_t);
+  uint32_t floor_key = 0u;
+  unsigned long long target;
+  if (by_mass) {
+    if (uses_top_k(temp, k)) floor_key = static_cast<uint32_t>(S[kSelCountState + 2 * 4]);  // (the mass kernel's)
+    target = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(S[kSelTotal]));
+    if (target < 1ull) target = 1ull;
+  } else {
+    target = static_cast<unsigned long long>(k < V ? k : V);
+  }
+  SelPos at{0u, 0ull};
+  if (pass > 0) at = advance(S, by_mass ? kSelMass : kSelCount, by_mass ? kSelMassState : kSelCountState, pass, target, scan, &chosen_s);
+  const uint32_t mask = pass == 0 ? 0u : 0xffffffffu << (32 - 8 * pass);
+  const int shift = 24 - 8 * pass;
+  hist[threadIdx.x] = 0ull;
+  __syncthreads();
+  const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
+  const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const float x = row[i] * inv_t;
+    const uint32_t key = ordered_key(x);
+    if (key < floor_key || (key & mask) != at.prefix) continue;
+    atomicAdd(&hist[(key >> shift) & 0xffu], by_mass ? mass_of(x, mx) : 1ull);
+  }
+  __syncthreads();
+  const unsigned long long mine = hist[threadIdx.x];
+  if (mine != 0ull) atomicAdd(&S[(by_mass ? kSelMass : kSelCount) + pass * 256 + threadIdx.x], mine);
+}
+
+// Between the two selections, for the rows with top-p: the mass of the entries that top-k leaves (all, without
+// top-k), added up over the parts.
+__global__ __launch_bounds__(kArgThreads) void select_mass_kernel(const float* __restrict__ logits, int64_t row_stride,
+                                                                 int V, const float* __restrict__ temperature,
+                                                                 const int* __restrict__ top_k,
+                                                                 const float* __restrict__ top_p,
+                                                                 const ArgMax* __restrict__ parts,
+                                                                 unsigned long long* __restrict__ sel) {
+  __shared__ unsigned long long scan[256];
+  __shared__ int chosen_s;
+  const int r = blockIdx.x, c = blockIdx.y;
+  const float temp = temperature[r];
+  const int k = top_k[r];
+  if (!uses_top_p(temp, k, top_p[r])) return;
+  unsigned long long* S = sel + static_cast<size_t>(r) * kSelWords;
+  const float inv_t = 1.f / temp;
+  float mx = -INFINITY;
+  for (int j = 0; j < kArgChunks; ++j) mx = fmaxf(mx, parts[static_cast<size_t>(r) * kArgChunks + j].v * inv_t);
+  uint32_t floor_key = 0u;
+  if (uses_top_k(temp, k))
+    floor_key = advance(S, kSelCount, kSelCountState, 4, static_cast<unsigned long long>(k < V ? k : V), scan, &chosen_s).prefix;
+  const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
+  const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
+  unsigned long long local = 0ull;
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const float x = row[i] * inv_t;
+    if (ordered_key(x) >= floor_key) local += mass_of(x, mx);
+  }
+  scan[threadIdx.x] = local;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (static_cast<int>(threadIdx.x) < o) scan[threadIdx.x] += scan[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0 && scan[0] != 0ull) atomicAdd(&S[kSelTotal], scan[0]);
+}
+
+// For the rows that are sampled (a temperature), again one workgroup per (row, part): among the part's entries that
+// top-k and top-p leave (sel null: only rows without them are served), the largest with its noise added and the
+// part's share of the softmax sum.  The noise of an entry depends on the request's seed, its draw counter and the
+// entry's number alone, so the parts draw what one workgroup would.
 struct DrawPart {
   ArgMax best;
   float sum, unused;
 };
-__device__ inline bool draws_from_all(float temp, int k, float p) { return temp != 0.f && k <= 0 && p >= 1.f; }
+// Whether a row is drawn in parts: its top-k and top-p, if it has them, must have been selected in parts (`selected`: the
+// modes whose selection kernels have run).
+__device__ inline bool drawn_in_parts(float temp, int k, float p, int selected) {
+  return !is_greedy(temp, k) && (!uses_top_k(temp, k) || (selected & kSampleTopK)) &&
+         (!uses_top_p(temp, k, p) || (selected & kSampleTopP));
+}
 
 __global__ __launch_bounds__(kArgThreads) void draw_parts_kernel(const float* __restrict__ logits, int64_t row_stride,
                                                                 int V, const float* __restrict__ temperature,
@@ -186,15 +347,36 @@ __global__ __launch_bounds__(kArgThreads) void draw_parts_kernel(const float* __
                                                                 const uint64_t* __restrict__ seed,
                                                                 const int* __restrict__ counter,
                                                                 const ArgMax* __restrict__ parts,
-                                                                DrawPart* __restrict__ draws) {
+                                                                DrawPart* __restrict__ draws,
+                                                                unsigned long long* __restrict__ sel, int selected) {
   __shared__ ArgMax am_scratch[kArgThreads / kWave];
   __shared__ float f_scratch[kArgThreads / kWave];
+  __shared__ unsigned long long scan[256];
+  __shared__ int chosen_s;
   const int r = blockIdx.x, c = blockIdx.y;
   const float temp = temperature[r];
-  if (!draws_from_all(temp, top_k[r], top_p[r])) return;
+  const int k = top_k[r];
+  const float p = top_p[r];
+  if (!drawn_in_parts(temp, k, p, selected)) return;
   const float inv_t = 1.f / temp;
   float mx = -INFINITY;
   for (int j = 0; j < kArgChunks; ++j) mx = fmaxf(mx, parts[static_cast<size_t>(r) * kArgChunks + j].v * inv_t);
+  // entries whose key is >= floor_key stay
+  uint32_t floor_key = 0u;
+  if (selected != 0) {
+    unsigned long long* S = sel + static_cast<size_t>(r) * kSelWords;
+    if (uses_top_k(temp, k))
+      floor_key = uses_top_p(temp, k, p)
+                      ? static_cast<uint32_t>(S[kSelCountState + 2 * 4])  // (the mass kernel has stored it)
+                      : advance(S, kSelCount, kSelCountState, 4, static_cast<unsigned long long>(k < V ? k : V), scan,
+                                &chosen_s).prefix;
+    if (uses_top_p(temp, k, p)) {
+      unsigned long long target = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(S[kSelTotal]));
+      if (target < 1ull) target = 1ull;
+      const uint32_t p_key = advance(S, kSelMass, kSelMassState, 4, target, scan, &chosen_s).prefix;
+      floor_key = p_key > floor_key ? p_key : floor_key;
+    }
+  }
   const float* row = logits + static_cast<size_t>(r) * row_stride;
   const int len = ((V + kArgChunks - 1) / kArgChunks + 3) / 4 * 4;
   const int lo = c * len < V ? c * len : V, hi = lo + len < V ? lo + len : V;
@@ -211,6 +393,7 @@ __global__ __launch_bounds__(kArgThreads) void draw_parts_kernel(const float* __
       const int i = 4 * b + j;
       if (i >= hi) break;
       const float x = row[i] * inv_t;
+      if (ordered_key(x) < floor_key) continue;
       sum += expf(x - mx);
       a = better(a, ArgMax{x + g[j], i});
     }
@@ -221,12 +404,12 @@ __global__ __launch_bounds__(kArgThreads) void draw_parts_kernel(const float* __
 }
 
 // parts: what argmax_parts_kernel has left for the rows, or null (they read their rows themselves); draws: what
-// draw_parts_kernel has left for the rows that are sampled from all of their entries.
+// draw_parts_kernel has left for the sampled rows (selected: the modes, top-k and top-p, that were selected in parts).
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const uint64_t* __restrict__ seed,
     const int* __restrict__ counter, int* __restrict__ tokens, float* __restrict__ logprobs,
-    const ArgMax* __restrict__ parts, const DrawPart* __restrict__ draws) {
+    const ArgMax* __restrict__ parts, const DrawPart* __restrict__ draws, int selected) {
   __shared__ ArgMax am_scratch[kSampleThreads / kWave];
   __shared__ float f_scratch[kSampleThreads / kWave];
   __shared__ unsigned long long hist[256];
@@ -276,7 +459,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   }
 
   const float inv_t = 1.f / temp;
-  if (draws != nullptr && draws_from_all(temp, k, p)) {
+  if (draws != nullptr && drawn_in_parts(temp, k, p, selected)) {
     float mx = -INFINITY, sum = 0.f;
     ArgMax a{-INFINITY, 0x7fffffff};
     if (threadIdx.x < kArgChunks) {
@@ -363,25 +546,49 @@ using namespace sa;
 
 extern "C" int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature,
                          const int* top_k, const float* top_p, const uint64_t* seed, const int* counter, int* tokens,
-                         float* logprobs, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+                         float* logprobs, int modes, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (R == 0) return 0;
   SA_REQUIRE(R > 0 && V > 0 && row_stride >= V, "sample: bad sizes R=%d V=%d stride=%lld", R, V,
              (long long)row_stride);
-  // large vocabularies: the greedy rows are searched by kArgChunks workgroups each first
+  // Large vocabularies: the rows are worked on in kArgChunks parts by as many workgroups, in several kernels (a
+  // row of 256,000 logits in one workgroup took 40 us for the argmax, 150 us for a draw, 350-600 us with top-k
+  // and top-p).  modes says what the rows may ask for, so that kernels nobody needs are not launched.
   ArgMax* parts = nullptr;
   DrawPart* draws = nullptr;
-  if (V >= 16384 && workspace != nullptr &&
-      workspace_bytes >= static_cast<int64_t>(R) * kArgChunks * static_cast<int64_t>(sizeof(ArgMax) + sizeof(DrawPart))) {
+  unsigned long long* sel = nullptr;
+  const bool any_drawn = (modes & (kSampleDrawn | kSampleTopK | kSampleTopP)) != 0;
+  const bool any_selection = (modes & (kSampleTopK | kSampleTopP)) != 0;
+  int selected = 0;  // the selections that run in parts
+  const int64_t need = static_cast<int64_t>(R) * (kArgChunks * static_cast<int64_t>(sizeof(ArgMax) + sizeof(DrawPart)) +
+                                                  kSelWords * static_cast<int64_t>(sizeof(unsigned long long)));
+  if (V >= 16384 && workspace != nullptr && workspace_bytes >= need) {
     draws = static_cast<DrawPart*>(workspace);
     parts = reinterpret_cast<ArgMax*>(draws + static_cast<size_t>(R) * kArgChunks);
-    argmax_parts_kernel<<<dim3(R, kArgChunks), kArgThreads, 0, stream>>>(logits, row_stride, V, parts);
+    if (any_selection) {
+      sel = reinterpret_cast<unsigned long long*>(parts + static_cast<size_t>(R) * kArgChunks);
+      selected = modes & (kSampleTopK | kSampleTopP);
+    }
+    const dim3 grid(R, kArgChunks);
+    argmax_parts_kernel<<<grid, kArgThreads, 0, stream>>>(logits, row_stride, V, parts, sel);
+    if (modes & kSampleTopK)
+      for (int pass = 0; pass < 4; ++pass)
+        select_pass_kernel<<<grid, kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, parts,
+                                                             sel, pass, 0);
+    if (modes & kSampleTopP) {
+      select_mass_kernel<<<grid, kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, parts, sel);
+      for (int pass = 0; pass < 4; ++pass)
+        select_pass_kernel<<<grid, kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, parts,
+                                                             sel, pass, 1);
+    }
+    if (any_drawn)
+      draw_parts_kernel<<<grid, kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed,
+                                                          counter, parts, draws, sel, selected);
+    else
+      draws = nullptr;
     if (check_launch("sample (parts)")) return 1;
-    draw_parts_kernel<<<dim3(R, kArgChunks), kArgThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p,
-                                                                      seed, counter, parts, draws);
-    if (check_launch("sample (draws)")) return 1;
   }
   sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed, counter,
-                                                  tokens, logprobs, parts, draws);
+                                                  tokens, logprobs, parts, draws, selected);
   return check_launch("sample");
 }
 

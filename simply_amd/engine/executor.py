@@ -174,7 +174,7 @@ class Executor:
                                  self.cache.page_size, ctx.groups[g.group_id].slot_mapping)
 
         ops.fill_(counter, 0)
-        key = ("many", B, self._context_bucket(ctx), max_steps, id(sampler))
+        key = ("many", B, self._context_bucket(ctx), max_steps, id(sampler), sampler.modes)
         entry = self._graphs.get(key)
         done = 0
         if entry is None:

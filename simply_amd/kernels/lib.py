@@ -42,7 +42,7 @@ _SIGNATURES = {
     "sa_gemm_normed_takes": [_I, _I, _I],
     "sa_gemm_normed_rotary": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _P, _P, _F, _F, _P, _P,
                               _P, _I, _I, _I, _I, _P],
-    "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P],
+    "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }
 
 

@@ -513,10 +513,14 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
 # --------------------------------------------------------------------------- sampling
 
 
+SAMPLE_DRAWN, SAMPLE_TOP_K, SAMPLE_TOP_P = 1, 2, 4
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            seed: torch.Tensor, counter: torch.Tensor, tokens: torch.Tensor | None = None,
-           logprobs: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
-    """One token per row.  All per-row parameter tensors are on the device, [R]."""
+           logprobs: torch.Tensor | None = None, modes: int = 7) -> tuple[torch.Tensor, torch.Tensor]:
+    """One token per row.  All per-row parameter tensors are on the device, [R].  modes: what some row may ask
+    for (SAMPLE_DRAWN + SAMPLE_TOP_K + SAMPLE_TOP_P); the kernels for what no row asks for are left out."""
     _dev(logits, temperature, top_k, top_p, seed, counter, tokens, logprobs)
     if logits.dtype != torch.float32:
         raise KernelError("sample: logits must be float32")
@@ -533,7 +537,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     _i32(tokens, "sample: tokens", R)
     ws = _workspace(logits.device)
     _lib.call("sa_sample", _ptr(logits), stride, R, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seed),
-              _ptr(counter), _ptr(tokens), _ptr(logprobs), _ptr(ws), ws.numel(), _stream())
+              _ptr(counter), _ptr(tokens), _ptr(logprobs), int(modes), _ptr(ws), ws.numel(), _stream())
     return tokens, logprobs
 
 

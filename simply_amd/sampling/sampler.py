@@ -36,6 +36,9 @@ class Sampler:
         self._s_dev = torch.empty(max_rows, dtype=torch.int64, device=self.device)
         self._tokens = torch.empty(max_rows, dtype=torch.int32, device=self.device)
         self._logprobs = torch.empty(max_rows, dtype=torch.float32, device=self.device)
+        #: what the staged rows ask for (ops.SAMPLE_*): `launch` leaves out the kernels that none of them needs, so
+        #: a recorded launch serves only rows that ask for no more than these
+        self.modes = 0
 
     def stage(self, params: Sequence[SamplingParams], seeds: Sequence[int], counters: Sequence[int]) -> None:
         """Puts the rows' parameters, seeds and draw counters where `launch` reads them (fixed device buffers)."""
@@ -45,6 +48,7 @@ class Sampler:
         if R > self.max_rows:
             raise ValueError(f"sample: {R} rows, room for {self.max_rows}")
         n = self.max_rows
+        self.modes = self.modes_of(params)
         for r, (p, s, c) in enumerate(zip(params, seeds, counters)):
             self._f_host[r] = p.temperature
             self._f_host[n + r] = p.top_p
@@ -54,6 +58,19 @@ class Sampler:
         self._f_dev.copy_(self._f_host, non_blocking=True)
         self._i_dev.copy_(self._i_host, non_blocking=True)
         self._s_dev.copy_(self._s_host, non_blocking=True)
+
+    @staticmethod
+    def modes_of(params: Sequence[SamplingParams]) -> int:
+        """What these rows ask of the sampling kernels: a draw at all, top-k, top-p."""
+        modes = 0
+        for p in params:
+            if p.temperature != 0.0 and p.top_k != 1:
+                modes |= ops.SAMPLE_DRAWN
+                if p.top_k > 0:
+                    modes |= ops.SAMPLE_TOP_K
+                if p.top_p < 1.0:
+                    modes |= ops.SAMPLE_TOP_P
+        return modes
 
     @property
     def draw_counters(self) -> torch.Tensor:
@@ -65,7 +82,7 @@ class Sampler:
         float32, [max_rows], the same every time) without waiting for it."""
         n = self.max_rows
         return ops.sample(logits, self._f_dev[:n], self._i_dev[:n], self._f_dev[n:], self._s_dev, self._i_dev[n:],
-                          self._tokens, self._logprobs)
+                          self._tokens, self._logprobs, modes=self.modes)
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
                counters: Sequence[int]) -> tuple[list[int], list[float]]:

@@ -495,6 +495,41 @@ def test_sampling_greedy_rows_of_a_large_vocabulary(V, offset):
     torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("V", [20000, 256000])
+def test_sampling_top_k_and_top_p_of_a_large_vocabulary(V):
+    """From 16384 entries on the boundaries of top-k and top-p are selected by 32 workgroups per row over several
+    kernels (histograms added up with atomics): the same tokens and log-probabilities as the reference, for every
+    mix of rows, with equal entries at a boundary, and whatever the caller says of what the rows may ask for (rows
+    that ask for more than it says are served by the one-workgroup path)."""
+    from simply_amd.kernels import ops
+    R = 9
+    logits = rand((R, V), torch.float32, 96, 2.5)
+    logits[6, 100:105] = 20.0         # five equal largest entries against top_k 3: all of them stay
+    logits[7, 7] = 30.0               # one entry holds nearly all the mass
+    temperature = torch.tensor([0.8, 1.3, 0.7, 1.0, 0.0, 0.9, 0.5, 2.0, 1.1]).cuda()
+    top_k = torch.tensor([40, -1, 50, V + 5, -1, -1, 3, -1, 2], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 0.9, 0.8, 1.0, 1.0, 1.0, 1.0, 0.05, 0.999]).cuda()
+    seed = torch.arange(R, dtype=torch.int64).cuda() * 7 + 11
+    rtok = rlp = None
+    for counter0 in (0, 5):
+        counter = torch.full((R,), counter0, dtype=torch.int32).cuda()
+        rtok, rlp = ref.sample(logits, temperature, top_k, top_p, seed, counter)
+        for modes in (7, 1, 3, 5, 0):
+            tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter, modes=modes)
+            assert tok.tolist() == rtok.tolist(), (modes, tok.tolist(), rtok.tolist())
+            torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+    assert rtok[6].item() in range(100, 105) and rtok[7].item() == 7
+    # rows that ask for one thing only, with the kernels for exactly that
+    for modes, rows in ((ops.SAMPLE_DRAWN | ops.SAMPLE_TOP_K, [0, 3, 6]), (ops.SAMPLE_DRAWN | ops.SAMPLE_TOP_P, [1, 7]),
+                        (ops.SAMPLE_DRAWN, [5]), (0, [4])):
+        idx = torch.tensor(rows).cuda()
+        counter = torch.full((len(rows),), 5, dtype=torch.int32).cuda()
+        tok, lp = ops.sample(logits[idx].contiguous(), temperature[idx], top_k[idx], top_p[idx], seed[idx], counter,
+                             modes=modes)
+        assert tok.tolist() == rtok[idx].tolist()
+        torch.testing.assert_close(lp, rlp[idx], rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("M", [1, 8, 13, 16])
 @pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (3584, 512), (4608, 64), (4640, 64), (96, 40),
                                  (72, 64)])
