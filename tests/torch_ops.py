@@ -198,7 +198,7 @@ def gumbel_noise(seed: int, counter: int, vocab: int) -> torch.Tensor:
     return torch.from_numpy(-np.log(-np.log(u)))
 
 
-def sample(logits, temperature, top_k, top_p, seed, counter, tokens=None, logprobs=None):
+def sample(logits, temperature, top_k, top_p, seed, counter, tokens=None, logprobs=None, modes=7):
     import sys, os
     sys.path.insert(0, os.path.dirname(__file__))
     import plain_gemma2 as plain
