@@ -262,6 +262,12 @@ static void launch(const bf16* A, int64_t lda, const bf16* W, void* C, int c_dty
 
 }  // namespace tiled
 
+// Whether a product of M rows against NW weight rows is bound by streaming the weights rather than by the MFMA
+// units: then workgroups take 64 rows x 256 weight rows with K cut over them.  Measured at the 2B sizes against
+// the wide-tile kernel: up to 64 rows always, beyond that while M * NW stays below about a million (192 rows of
+// the q/k/v projection, 384 of the output and down projections, never the paired gate/up weight).
+bool gemm_streams_weights(int M, int NW) { return M <= 64 || static_cast<int64_t>(M) * NW <= 1000000; }
+
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed) {
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   return packed && W2 == nullptr && M >= 1 && K % 8 == 0 && lda % 8 == 0 && aligned(A) && aligned(W) &&
@@ -276,7 +282,7 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
   float* ws = static_cast<float*>(workspace);
   const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const int stages = (K + tiled::BK - 1) / tiled::BK;
-  const bool few = M <= 64;
+  const bool few = gemm_streams_weights(M, NW);
   int ks = 1;
   if (ksplit > 0) {
     ks = ksplit;

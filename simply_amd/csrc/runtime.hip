@@ -56,8 +56,9 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
     if (takes)
       return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, shape, stream);
   }
-  // from 256 rows on, the wide tiles (both operands through LDS)
-  if (algo == 4 || (algo == 0 && bf16_in && packed && M >= 256)) {
+  // once the product is no longer bound by streaming the weights: the wide tiles (both operands through LDS)
+  const int NW = epilogue == 1 ? 2 * ((N + 15) / 16) * 16 : N;
+  if (algo == 4 || (algo == 0 && bf16_in && packed && !gemm_streams_weights(M, NW))) {
     const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the wide MFMA kernel takes bfloat16 in and out with tiled weights, no soft-cap, K a multiple of "

@@ -414,7 +414,7 @@ def test_gemm_wide(M, N, K):
     one = ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=2256192)
     assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=3128256))
     assert torch.equal(one[: M // 2 + 1], ops.gemm(a[: M // 2 + 1], tw, algo=ops.ALGO_WIDE))
-    assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_TILED))
+    assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_TILED, shape=1))   # (K in one piece: the same order)
     # rows inside wider rows, in and out
     kw = dict(algo=ops.ALGO_WIDE)
     big = rand((M, K + 16), torch.bfloat16, 93)
@@ -430,7 +430,8 @@ def test_gemm_wide(M, N, K):
         ops.gemm(a[:, :K - 32], pack_tiles(w[:, :K - 32].contiguous()), **kw)   # K that is no multiple of 64
     with pytest.raises(KernelError, match="wide"):
         ops.gemm(a, pack_tiles(w[:N - 2].contiguous()), **kw)  # N that is no multiple of 4
-    # from 256 rows on it is what the library chooses by itself; below, and for what it refuses, the tiled kernel
+    # it is what the library chooses by itself for products that are not bound by streaming the weights; for what it
+    # refuses, the tiled kernel
     torch.testing.assert_close(ops.gemm(a, pack_tiles(w[:N - 2].contiguous())).float(), want[:, :N - 2], **t)
 
 
