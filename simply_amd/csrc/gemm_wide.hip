@@ -3,8 +3,8 @@
 // slab of 64 columns through a CU's 64 bytes a clock, which caps it at about a third of the MFMA rate.
 //
 // A workgroup of eight waves (one per CU) owns 256 x 192, 256 x 128, 128 x 256 or 192 x 128 outputs (or one of four
-// waves, two per CU, 128 x 192) and takes both operands through LDS, in slabs of 64 columns of K that go round two or three buffers, with loads that go from
-// global memory straight into LDS (no registers in between).
+// waves, two per CU, 128 x 192) and takes both operands through LDS, in slabs of 64 columns of K that go round two
+// or three buffers, with loads that go from global memory straight into LDS (no registers in between).
 //   * Layout in LDS: W as KiB blocks in MFMA operand order (16 rows x 32 columns, lane l holds row l % 16,
 //     columns 8 (l / 16) ..), which is how it lies in global memory, so a block is a copy.  A as rows of 128 bytes
 //     (eight lanes load a row: whole lines) whose eight 16-byte pieces are permuted by the row's number, so that
@@ -57,7 +57,7 @@ __device__ __forceinline__ void load_to_lds(const bf16* base, uint32_t offset, u
                : "memory");
 }
 
-// WM x WN: 16 x 16 tiles of a wave (rows of A x rows of W); WAVES_M x (8 / WAVES_M) waves.
+// WM x WN: 16 x 16 tiles of a wave (rows of A x rows of W); WAVES_M x (WAVES / WAVES_M) waves.
 template <int WM, int WN, int WAVES_M, int EPI, int NSTAGE, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __restrict__ A, int64_t lda,
                                                         const bf16* __restrict__ W, bf16* __restrict__ C, int64_t ldc,
