@@ -5,7 +5,8 @@
 // the keys once for all of its rows.
 //
 // Keys and values go from the pages straight into LDS (global_load_lds: no staging registers), into two buffers
-// of one 32-key tile each, so that the loads of the next tile are in flight while one tile is computed; two
+// of one 32-key tile each, so that the loads of the next tile are in flight while one tile is computed (they are
+// asked for one by one among the tile's first products; a third buffer, loads two tiles ahead, was slower); two
 // workgroups fit on a compute unit and fill each other's waits.  Both lie in LDS as they lie in their pages: keys in 16-key x 32-dimension blocks of MFMA operand
 // order, values per 16-key sub-tile as blocks of 16 dimensions, [keys 0..7 | keys 8..15][dimension][8 keys].  Every wave reads every block of a tile and computes,
 // for its own rows,
@@ -19,8 +20,7 @@
 //
 // The two buffers are kept in step by one workgroup barrier per tile.  The barrier is the bare instruction, with the
 // count of outstanding loads given by hand: the usual barrier with its fence would wait for all loads in flight,
-// which is the pipeline.  Each buffer is an array of its own so that the compiler can tell a read of one buffer
-// from the loads in flight into the others.
+// which is the pipeline.  The loads are written as instructions that the compiler does not know of (load_to_lds below).
 //
 // When few workgroups would result (a short portion over a long context), the keys are also cut into ranges over
 // workgroups, and the ranges are merged by the second kernel of the few-rows path.
@@ -44,10 +44,13 @@ __device__ inline void bare_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// 16 bytes per lane from global memory into LDS at dst + 16 * lane (dst is the same for the whole wave).  In a
-// function of its own: written into the kernel's body, the host pass of the compiler drops the kernel's stub.
-__device__ __forceinline__ void load_to_lds(const bf16* src, __bf16* dst) {
-  __builtin_amdgcn_global_load_lds(src, dst, 16, 0, 0);
+// 16 bytes per lane from global memory (an address per lane) into LDS at byte address lds + 16 * lane (lds is the
+// same for the whole wave).  Written as an instruction: the compiler counts a load into LDS that it knows of as a
+// pending LDS access for as long as the load is under way, and then makes every wait for an operand read a wait for
+// all of them.  It does not know of these loads: the kernel waits for them itself (vmcnt) before the barrier that
+// precedes the first read of what they bring.
+__device__ __forceinline__ void load_to_lds(const bf16* src, uint32_t lds) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds) : "memory");
 }
 
 template <int NDC, int R, bool CAP>
@@ -65,6 +68,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   // [keys: sub-tile, dc, lane, 8][values: sub-tile, d, 16]
   __shared__ __attribute__((aligned(16))) __bf16 stage0[2 * HALF];
   __shared__ __attribute__((aligned(16))) __bf16 stage1[2 * HALF];
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) __bf16*)stage0));
+  const uint32_t lds1 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) __bf16*)stage1));
 
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -143,8 +148,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     v_off[i] = (c * 16 + lane % 16) * page_size + ((lane / 16) % 2) * 8;
     lds_off[i] = __builtin_amdgcn_readfirstlane(c * 512);
   }
-  // Where the tile's two sub-tiles lie for the tile asked for next: block blk[n] of the table, key off[n] of its
-  // page; kept by stepping, without divisions.  All of it is the same for the whole wave: scalar registers.
+  // Where the two sub-tiles lie of the tile whose pages are looked up next: block blk[n] of the table, key off[n] of
+  // its page; kept by stepping, without divisions.  All of it is the same for the whole wave: scalar registers.
   int blk[2], off[2];
 #pragma unroll
   for (int n = 0; n < 2; ++n) {
@@ -157,18 +162,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
   const bf16* const v_head = v_pages + static_cast<int64_t>(kh) * page_size * HD;
   // sub-tiles (of 16 keys) with a page that this workgroup may read: [sub_lo, sub_hi)
   const int sub_lo = lo_g / 16, sub_hi = min((hi_g + 15) / 16, te * 2);
-  // Asks for this wave's blocks of `tile` (called for consecutive tiles) into a buffer.  A sub-tile without a page
-  // (beyond the keys, or given back by a windowed layer) reads page 0; its values are dropped when they are used.
-  auto request = [&](int tile, __bf16* stage) __attribute__((always_inline)) {
-    const bf16* kb[2];
-    const bf16* vb[2];
+  // The loads of a tile are prepared in steps, so that no step waits for the one before it: the pages of its two
+  // sub-tiles are looked up two tiles ahead (`look_up`, called for consecutive tiles: a sub-tile without a page,
+  // beyond the keys or given back by a windowed layer, reads page 0, and its values are dropped when they are
+  // used), this lane's addresses follow one tile ahead (`locate`), and the loads themselves are asked for one by
+  // one among the products of the tile before (`ask`).
+  struct Pages {
+    uint32_t page[2], at[2];
+  };
+  auto look_up = [&](int tile) __attribute__((always_inline)) {
+    Pages p;
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
       const int sub = tile * 2 + n;
-      const uint32_t page = (sub >= sub_lo && sub < sub_hi) ? static_cast<uint32_t>(table[blk[n]]) : 0u;
-      const uint64_t at = static_cast<uint64_t>(page) * page_stride;
-      kb[n] = k_head + at + static_cast<uint32_t>(off[n] >> 4) * (NDC * 512);
-      vb[n] = v_head + at + static_cast<uint32_t>(off[n]);
+      p.page[n] = (sub >= sub_lo && sub < sub_hi) ? static_cast<uint32_t>(table[blk[n]]) : 0u;
+      p.at[n] = static_cast<uint32_t>(off[n]);
       off[n] += kTile;
 #pragma unroll
       for (int twice = 0; twice < 2; ++twice)
@@ -177,47 +185,80 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
           ++blk[n];
         }
     }
-    const bf16* const k_from = k_sub ? kb[1] : kb[0];
-    const bf16* const v_from = v_sub ? vb[1] : vb[0];
-#pragma unroll
-    for (int i = 0; i < CPW; ++i) {
-      __bf16* const k_to = stage + lds_off[i];
-      __bf16* const v_to = k_to + HALF;
-      load_to_lds(k_from + k_off[i], k_to);
-      load_to_lds(v_from + v_off[i], v_to);
-    }
+    return p;
+  };
+  const bf16* k_from;
+  const bf16* v_from;
+  auto locate = [&](const Pages& p) __attribute__((always_inline)) {
+    const uint32_t page = k_sub ? p.page[1] : p.page[0], at_k = k_sub ? p.at[1] : p.at[0];
+    k_from = k_head + static_cast<uint64_t>(page) * page_stride + (at_k >> 4) * (NDC * 512);
+    const uint32_t page_v = v_sub ? p.page[1] : p.page[0], at_v = v_sub ? p.at[1] : p.at[0];
+    v_from = v_head + static_cast<uint64_t>(page_v) * page_stride + at_v;
+  };
+  // load i (of CPW) of the keys and of the values of the located tile, into the buffer at byte address `to`
+  auto ask = [&](int i, uint32_t to) __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    load_to_lds(k_from + k_off[i], to + lds_off[i] * 2);
+    load_to_lds(v_from + v_off[i], to + (lds_off[i] + HALF) * 2);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // one tile from LDS, for this wave's rows
-  auto compute = [&](int tile, const __bf16* stage) __attribute__((always_inline)) {
+  // one tile from the buffer `stage`, for this wave's rows; meanwhile the located tile is asked for into the buffer
+  // at byte address `to`
+  auto compute = [&](int tile, const __bf16* stage, uint32_t to) __attribute__((always_inline)) {
     const int key0 = tile * kTile;
     bool any = false;
 #pragma unroll
     for (int j = 0; j < R; ++j) any = any || (rows[j] > 0 && key0 <= pos_last[j] && key0 + kTile > lo_first[j]);
-    if (tile >= te || !any) return;  // no row of the wave sees a key of it
+    if (tile >= te || !any) {  // no row of the wave sees a key of it
+#pragma unroll
+      for (int i = 0; i < CPW; ++i) ask(i, to);
+      return;
+    }
     const __bf16* k_s = stage;
     const __bf16* v_s = stage + HALF;
-    // Operands come from LDS in batches that are issued together, so that their latency is paid once per batch.
+    // Operands come from LDS in batches; the reads of a batch are issued before the products of the batch before it,
+    // which cover their latency.  After every second chunk of dimensions the next of the CPW loads is asked for:
+    // asked for together, the waves queue up at the memory pipeline while the MFMA unit idles.
     constexpr int KB = NDC < 4 ? NDC : 4;  // dimension chunks per batch of key operands
+    constexpr int KBATCHES = NDC / KB;
     floatx4 s[R][2];
 #pragma unroll
     for (int j = 0; j < R; ++j) s[j][0] = s[j][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int dc0 = 0; dc0 < NDC; dc0 += KB) {
-      bf16x8 kf[2][KB];
+    bf16x8 kf[2][2][KB];
+    auto read_keys = [&](int batch) __attribute__((always_inline)) {
 #pragma unroll
       for (int b = 0; b < KB; ++b)
 #pragma unroll
         for (int t = 0; t < 2; ++t)
-          kf[t][b] = *reinterpret_cast<const bf16x8*>(k_s + ((t * NDC + dc0 + b) * 64 + lane) * 8);
+          kf[batch % 2][t][b] = *reinterpret_cast<const bf16x8*>(k_s + ((t * NDC + batch * KB + b) * 64 + lane) * 8);
+    };
+    read_keys(0);
 #pragma unroll
-      for (int b = 0; b < KB; ++b)
+    for (int batch = 0; batch < KBATCHES; ++batch) {
+      if (batch + 1 < KBATCHES) read_keys(batch + 1);
+#pragma unroll
+      for (int b = 0; b < KB; ++b) {
+        const int dc = batch * KB + b;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int j = 0; j < R; ++j)
-            s[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][b], qf[j][dc0 + b], s[j][t], 0, 0, 0);
+            s[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[batch % 2][t][b], qf[j][dc], s[j][t], 0, 0, 0);
+        if (dc % 2 == 1) ask(dc / 2, to);
+      }
     }
+    // the first value operands are on their way during the softmax arithmetic
+    constexpr int VB = 4;  // output blocks per batch of value operands
+    bf16x8 vf[2][VB];
+    auto read_values = [&](int batch) __attribute__((always_inline)) {
+#pragma unroll
+      for (int b = 0; b < VB; ++b)
+        vf[batch % 2][b] = *reinterpret_cast<const bf16x8*>(v_s + ((batch * VB + b) * 64 + lane) * 8);
+    };
+    read_values(0);
+    __builtin_amdgcn_sched_barrier(0);
     bf16x8 pf[R];
     float alpha[R];
     bool rescale = false;
@@ -278,44 +319,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
     // Lane (d = r, grp) of the value operand holds V^T[db * 16 + r][keys 8 * grp .. + 7 of the tile].  Values of
     // keys that no row may use (unwritten, given back, another request's) count as 0; their scores are masked
     // anyway.  That concerns the last tile of the keys and tiles at a window's lower edge.
-    constexpr int VB = 4;  // output blocks per batch of value operands
     const bool fix = key0 + kTile > hi_g || key0 < lo_g;  // uniform
 #pragma unroll
-    for (int db0 = 0; db0 < NDB; db0 += VB) {
-      bf16x8 vf[VB];
-#pragma unroll
-      for (int b = 0; b < VB; ++b) vf[b] = *reinterpret_cast<const bf16x8*>(v_s + ((db0 + b) * 64 + lane) * 8);
+    for (int batch = 0; batch < NDB / VB; ++batch) {
+      if (batch + 1 < NDB / VB) read_values(batch + 1);
       if (fix) {
 #pragma unroll
         for (int b = 0; b < VB; ++b)
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int key = key0 + grp * 8 + e;
-            if (key >= hi_g || key < lo_g) vf[b][e] = to_bf16_raw(0.f);
+            if (key >= hi_g || key < lo_g) vf[batch % 2][b][e] = to_bf16_raw(0.f);
           }
       }
 #pragma unroll
       for (int b = 0; b < VB; ++b)
 #pragma unroll
         for (int j = 0; j < R; ++j)
-          acc[j][db0 + b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf[j], acc[j][db0 + b], 0, 0, 0);
+          acc[j][batch * VB + b] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[batch % 2][b], pf[j], acc[j][batch * VB + b], 0, 0, 0);
     }
   };
 
   if (tb < te) {
-    request(tb, stage0);
+    locate(look_up(tb));
+#pragma unroll
+    for (int i = 0; i < CPW; ++i) ask(i, lds0);
+    Pages next = look_up(tb + 1);
     // tile `tile` has been asked for into `cur`; `other` held tile - 1 and takes tile + 1
-    auto step = [&](int tile, const __bf16* cur, __bf16* other) __attribute__((always_inline)) {
+    auto step = [&](int tile, const __bf16* cur, uint32_t other) __attribute__((always_inline)) {
+      __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's chunks of `tile` have arrived
       bare_barrier();  // and everyone's; and every wave has finished tile - 1
-      request(tile + 1, other);
-      compute(tile, cur);
+      locate(next);
+      next = look_up(tile + 2);
+      compute(tile, cur, other);
     };
     const int te2 = tb + (te - tb + 1) / 2 * 2;
     for (int tile = tb; tile < te2; tile += 2) {
-      step(tile, stage0, stage1);
-      step(tile + 1, stage1, stage0);
+      step(tile, stage0, lds1);
+      step(tile + 1, stage1, lds0);
     }
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // the load asked for beyond the range
   }
 
