@@ -119,3 +119,64 @@ def test_graph_replays_match_eager(tmp_path, dtype):
         want = plain_logits(d, t, dtype)[0][19:]
         err = (outs[True][r].double() - want).abs().max().item() / want.abs().max().item()
         assert err <= TOL[dtype], (r, err)
+
+
+@pytest.mark.parametrize("seed", range(100, 112))
+def test_random_configurations_mixed(tmp_path, seed):
+    """Configurations drawn at random (tiny.random_config), each with up to four live requests cut at random into
+    portions and single tokens, in a pool that is smaller than what all requests hold: in 32-bit against the plain
+    implementation; in bfloat16 against the plain implementation and against the same requests run whole and
+    alone, where only the rounding of other kernels may differ."""
+    d = tiny.write_random_config_model(seed, str(tmp_path / "m"))
+    w0, pcfg = plain.load(d)
+    rng = np.random.default_rng(seed)
+    page = int(rng.choice([4, 8, 16, 16, 32]))
+    lens = [int(rng.integers(2, 130)) for _ in range(int(rng.integers(3, 6)))]
+    reqs = {f"r{i}": tiny.random_tokens(n, pcfg["vocab_size"], seed * 100 + i) for i, n in enumerate(lens)}
+    pages_of = lambda n: -(-n // page) + 1
+    num_pages = max(pages_of(max(lens)) + 2, int(sum(pages_of(n) for n in lens) * 0.6))
+    for dtype in ("float32", "bfloat16"):
+        w = w0 if dtype == "float32" else {k: v.to(torch.bfloat16) for k, v in w0.items()}
+        want = {r: plain.forward(w, pcfg, t, torch.float64) for r, t in reqs.items()}
+        ex = make_executor(d, dtype, page_size=page, num_pages=num_pages)
+        pending, live, got = list(reqs), {}, {r: {} for r in reqs}
+        while pending or live:
+            while pending and len(live) < 4:
+                if sum(pages_of(len(reqs[r])) for r in live) + pages_of(len(reqs[pending[0]])) > num_pages:
+                    break
+                live[pending[0]] = 0
+                ex.add_request(pending.pop(0))
+            entries = []
+            for r in list(live):
+                left = len(reqs[r]) - live[r]
+                if rng.random() < 0.25 and len(live) > 1:
+                    continue
+                n = 1 if (left < 2 or rng.random() < 0.4) else int(rng.integers(2, min(left, 40) + 1))
+                entries.append(StepEntry(r, reqs[r][live[r]:live[r] + n], list(range(n)) if rng.random() < 0.8 else []))
+            if not entries:
+                continue
+            logits = ex.step(entries)
+            i = 0
+            for e in entries:
+                r = e.request_id
+                for at in e.want:
+                    got[r][live[r] + at] = logits[i].cpu()
+                    i += 1
+                live[r] += len(e.tokens)
+                if live[r] == len(reqs[r]):
+                    ex.finish_request(r)
+                    del live[r]
+            ex.cache.check()
+        for r, t in reqs.items():
+            at = sorted(got[r])
+            if not at:
+                continue
+            g = torch.stack([got[r][p] for p in at]).double()
+            scale = want[r].abs().max().item()
+            assert torch.isfinite(g).all()
+            assert (g - want[r][at]).abs().max().item() / scale <= TOL[dtype], (dtype, r)
+            if dtype == "bfloat16":
+                ex.add_request(r)
+                whole = ex.step([StepEntry(r, t, list(range(len(t))))]).cpu().double()
+                ex.finish_request(r)
+                assert (g - whole[at]).abs().max().item() / scale <= 1e-2, (dtype, r)

@@ -54,3 +54,37 @@ def write_model(name: str, out_dir: str, dtype=torch.float32, std: float | None 
 def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def random_config(seed: int) -> dict:
+    """A tiny configuration drawn at random: head counts and groups, head sizes in steps of 16 up to 256, widths
+    that are no multiple of 8, layer kinds in any order, caps present or not."""
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    kv, group = int(rng.choice([1, 2, 3, 4])), int(rng.choice([1, 2, 3, 4, 8]))
+    hd = int(rng.choice([16, 32, 48, 64, 80, 96, 128, 256]))
+    if hd >= 128:
+        kv, group = min(kv, 2), min(group, 2)
+    layers = int(rng.integers(1, 5))
+    return dict(
+        architectures=["Gemma2ForCausalLM"], hidden_size=int(rng.choice([64, 96, 120, 128, 136, 200, 100, 264])),
+        num_hidden_layers=layers, num_attention_heads=kv * group, num_key_value_heads=kv, head_dim=hd,
+        intermediate_size=int(rng.choice([128, 200, 320, 264, 72, 500])),
+        vocab_size=int(rng.choice([256, 333, 512, 1000, 1001, 4099])), rms_norm_eps=float(rng.choice([1e-6, 1e-5])),
+        rope_theta=float(rng.choice([10000.0, 1e6, 500.0])), sliding_window=int(rng.integers(3, 60)),
+        query_pre_attn_scalar=int(rng.choice([hd, 24, 144])),
+        attn_logit_softcapping=None if rng.random() < 0.3 else float(rng.choice([50.0, 20.0, 5.0])),
+        final_logit_softcapping=None if rng.random() < 0.3 else float(rng.choice([30.0, 15.0])),
+        tie_word_embeddings=True, max_position_embeddings=1024,
+        layer_types=[str(rng.choice(["full_attention", "sliding_attention"])) for _ in range(layers)],
+        hidden_activation="gelu_pytorch_tanh", initializer_range=0.05)
+
+
+def write_random_config_model(seed: int, out_dir: str) -> str:
+    from simply_amd.config import config_from_dict
+    from simply_amd.weights import write_random_model
+
+    d = random_config(seed)
+    std = 0.15 * (64.0 / d["hidden_size"]) ** 0.5
+    return write_random_model(config_from_dict(d), out_dir, seed, torch.float32, std=std, norm_std=0.2)
