@@ -114,9 +114,10 @@ int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pag
                               void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // The same for portions of prompts: the units (rows of seq_meta, each with (query heads per key head) * tokens <= 16)
-// unit_begin .. unit_begin + unit_count - 1 are taken four at a time by one workgroup, which reads the keys once for
-// all of them.  unit_count is a multiple of 4 and the four units of a workgroup belong to one request; units with
-// no tokens fill up a request's last four.
+// unit_begin .. unit_begin + unit_count - 1 are taken a group at a time by one workgroup, which reads the keys once
+// for all of them.  unit_count is a multiple of the group (sa_paged_attention_prefill_group units) and the units of a
+// group belong to one request; units with no tokens fill up a request's last group.
+int sa_paged_attention_prefill_group();
 int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
                                int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
@@ -147,6 +148,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
                            hipStream_t stream);
+int paged_attention_prefill_group();  // units that one workgroup takes
 bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q,
                                    int64_t out_stride, const void* out);
 int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,

@@ -54,7 +54,7 @@ __device__ __forceinline__ void load_to_lds(const bf16* src, uint32_t lds) {
 }
 
 template <int NDC, int R, bool CAP>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void paged_attention_prefill_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 : 1, R == 1 ? 2 : 1))) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
 
 }  // namespace prefill
 
-constexpr int kPrefillRowTiles = 1;  // R: units per wave
+constexpr int kPrefillRowTiles = 1;  // R: units per wave (2 was tried: three times slower, the registers of 32 rows spill)
 
 int paged_attention_prefill_group() { return prefill::kWaves * kPrefillRowTiles; }
 

@@ -113,6 +113,8 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
                                 workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
 }
 
+extern "C" int sa_paged_attention_prefill_group() { return paged_attention_prefill_group(); }
+
 extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                           const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
                                           int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd,
@@ -120,8 +122,9 @@ extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const
                                           int num_splits, void* workspace, int64_t workspace_bytes,
                                           hipStream_t stream) {
   if (unit_count == 0) return 0;
-  SA_REQUIRE(unit_count > 0 && unit_count % 4 == 0 && unit_begin >= 0 && H > 0 && Kh > 0 && H % Kh == 0,
-             "paged_attention_prefill: bad counts (units come in fours)");
+  SA_REQUIRE(unit_count > 0 && unit_count % paged_attention_prefill_group() == 0 && unit_begin >= 0 && H > 0 && Kh > 0 &&
+                 H % Kh == 0,
+             "paged_attention_prefill: bad counts (units come in groups of %d)", paged_attention_prefill_group());
   SA_REQUIRE(window >= 0 && table_stride > 0 && max_kv_len > 0, "paged_attention_prefill: bad window, table or length");
   SA_REQUIRE(paged_attention_prefill_takes(H, Kh, hd, page_size, max_q_len, q_stride, q, out_stride, out),
              "paged_attention_prefill takes head size 64, 128 or 256, a page size that is a multiple of 16 and "

@@ -501,7 +501,9 @@ def paged_attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torc
                             seq_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
 
 
-PREFILL_UNITS_PER_GROUP = 4
+def prefill_units_per_group() -> int:
+    """How many units one workgroup of the portion kernel takes (they must belong to one request)."""
+    return int(_lib.load().sa_paged_attention_prefill_group())
 
 
 def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
@@ -509,11 +511,11 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                             window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
                             out: torch.Tensor, num_splits: int = 0) -> torch.Tensor:
     """Attention of portions of prompts cut into units of few tokens ((heads per key head) * tokens <= 16), rows
-    unit_begin .. unit_begin + unit_count - 1 of `units` in the layout of seq_meta.  One workgroup takes four
-    consecutive units, which must belong to one request (units without tokens fill up the last four), and
+    unit_begin .. unit_begin + unit_count - 1 of `units` in the layout of seq_meta.  One workgroup takes a group of
+    consecutive units, which must belong to one request (units without tokens fill up the last group), and
     reads the keys once for all of them."""
-    if unit_count % PREFILL_UNITS_PER_GROUP:
-        raise KernelError("paged_attention_prefill: units come in fours")
+    if unit_count % prefill_units_per_group():
+        raise KernelError(f"paged_attention_prefill: units come in groups of {prefill_units_per_group()}")
     return _attention_units("sa_paged_attention_prefill", q, k_pages, v_pages, block_table, units, unit_begin,
                             unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
 

@@ -84,7 +84,7 @@ class PagedAttention(Mixer):
             # the MFMA kernels take up to 16 query rows (tokens x heads per key head) as a unit: a decoding request
             # is one unit and its keys are cut over workgroups; portions of prompts are cut into units of 16 / G
             # tokens, of which one workgroup takes four
-            units, few, many, max_q = ctx.attention_units(16 // (H // K), ops.PREFILL_UNITS_PER_GROUP)
+            units, few, many, max_q = ctx.attention_units(16 // (H // K), ops.prefill_units_per_group())
             kw = dict(window=self.window, soft_cap=self.soft_cap, max_kv_len=ctx.max_kv_len, max_q_len=max_q, out=o)
             if few:
                 ops.paged_attention_decode(qkv, cache.k_pages, cache.v_pages, group.block_table, units, 0, few, H, **kw)

@@ -571,12 +571,13 @@ def test_gemm_normed(M, K, N):
 
 def prefill_units(lens, q_lens, per_unit):
     """Units of at most per_unit tokens of requests whose last q tokens are this step's, each request's units
-    filled up to a multiple of four: what the host hands to the prompt-portion kernel."""
+    filled up to a multiple of the kernel's group: what the host hands to the prompt-portion kernel."""
+    from simply_amd.kernels import ops
     units, t0 = [], 0
     for s, (l, q) in enumerate(zip(lens, q_lens)):
         for o in range(0, q, per_unit):
             units.append((s, t0 + o, min(per_unit, q - o), l - q + o))
-        while len(units) % 4:
+        while len(units) % ops.prefill_units_per_group():
             units.append((s, t0 + q, 0, l))
         t0 += q
     return torch.tensor(units, dtype=torch.int32).cuda()
@@ -620,7 +621,7 @@ def test_paged_attention_prefill(H, Kh, hd, P, window, cap, splits):
     a, b = sum(q_lens[:2]), sum(q_lens[:3])
     torch.testing.assert_close(out3[a:b].float(), out[a:b].float(), rtol=2e-2, atol=2e-2)
     assert (out3[:a] == 7).all() and (out3[b:] == 7).all()
-    with pytest.raises(Exception, match="fours"):
+    with pytest.raises(Exception, match="groups of"):
         ops.paged_attention_prefill(q, kp, vp, table, units, 0, 3, H, window=window, soft_cap=cap,
                                     max_kv_len=max(lens), max_q_len=per_unit, out=out3)
 
