@@ -3,7 +3,7 @@ __version__ = "0.1.0"
 
 
 def __getattr__(name):
-    if name in ("LLM", "LMInterface", "SamplingParams", "SamplingOutput"):
+    if name in ("LLM", "LMInterface", "SamplingParams", "ScoringParams", "SamplingOutput"):
         from .engine import llm as _llm
 
         return getattr(_llm, name)

@@ -132,6 +132,12 @@ int sa_sample(const float* logits, int64_t row_stride, int R, int V, const float
               const float* top_p, const uint64_t* seed, const int* counter, int* tokens, float* logprobs, int modes,
               void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
+// The log-probability of a given token per row under the row's temperature, top-k and top-p (what sa_sample reports
+// for the token it draws): 0 or -0.5 * FLT_MAX for greedy rows (the token is the argmax or not), -0.5 * FLT_MAX for
+// a token that the masks leave out.  One workgroup per row.
+int sa_score(const float* logits, int64_t row_stride, int R, int V, const float* temperature, const int* top_k,
+             const float* top_p, const int* tokens, float* scores, hipStream_t stream);
+
 // Host function: one block of the Philox4x32-10 generator that sa_sample uses.
 void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* out4);
 }

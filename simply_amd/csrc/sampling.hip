@@ -405,6 +405,11 @@ __global__ __launch_bounds__(kArgThreads) void draw_parts_kernel(const float* __
 
 // parts: what argmax_parts_kernel has left for the rows, or null (they read their rows themselves); draws: what
 // draw_parts_kernel has left for the sampled rows (selected: the modes, top-k and top-p, that were selected in parts).
+// SCORE: nothing is drawn; tokens holds a given token per row, and logprobs receives its log-probability under the
+// row's temperature, top-k and top-p: 0 or kMasked for greedy rows (simply/utils/sampling_lib.py:550-558), kMasked
+// for a token that the masks leave out (simply/utils/distributions.py:104-121).
+constexpr float kMasked = -0.5f * 3.402823466e38f;  // simply/utils/common.py:543-551 for float32
+template <bool SCORE>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const uint64_t* __restrict__ seed,
@@ -435,8 +440,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
       if (threadIdx.x < kArgChunks) a = parts[static_cast<size_t>(r) * kArgChunks + threadIdx.x];
       a = block_argmax(a, am_scratch);
       if (threadIdx.x == 0) {
-        tokens[r] = a.i;
-        logprobs[r] = 0.f;
+        if (SCORE) {
+          logprobs[r] = tokens[r] == a.i ? 0.f : kMasked;
+        } else {
+          tokens[r] = a.i;
+          logprobs[r] = 0.f;
+        }
       }
       return;
     }
@@ -452,14 +461,18 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     for (int i = tail0 + threadIdx.x; i < V; i += blockDim.x) a = better(a, ArgMax{row[i], i});
     a = block_argmax(a, am_scratch);
     if (threadIdx.x == 0) {
-      tokens[r] = a.i;
-      logprobs[r] = 0.f;
+      if (SCORE) {
+        logprobs[r] = tokens[r] == a.i ? 0.f : kMasked;
+      } else {
+        tokens[r] = a.i;
+        logprobs[r] = 0.f;
+      }
     }
     return;
   }
 
   const float inv_t = 1.f / temp;
-  if (draws != nullptr && drawn_in_parts(temp, k, p, selected)) {
+  if (!SCORE && draws != nullptr && drawn_in_parts(temp, k, p, selected)) {
     float mx = -INFINITY, sum = 0.f;
     ArgMax a{-INFINITY, 0x7fffffff};
     if (threadIdx.x < kArgChunks) {
@@ -514,6 +527,34 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     floor_key = p_key > floor_key ? p_key : floor_key;
   }
 
+  if (SCORE) {
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      const float x = row[i] * inv_t;
+      if (ordered_key(x) >= floor_key) sum += expf(x - mx);
+    }
+    sum = block_sum(sum, f_scratch);
+    if (threadIdx.x == 0) {
+      const int given = tokens[r];
+      const float x = (given >= 0 && given < V) ? row[given] * inv_t : -INFINITY;
+      logprobs[r] = (given >= 0 && given < V && ordered_key(x) >= floor_key) ? x - mx - logf(sum) : kMasked;
+    }
+    return;
+  }
+  if (SCORE) {
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      const float x = row[i] * inv_t;
+      if (ordered_key(x) >= floor_key) sum += expf(x - mx);
+    }
+    sum = block_sum(sum, f_scratch);
+    if (threadIdx.x == 0) {
+      const int given = tokens[r];
+      const float x = (given >= 0 && given < V) ? row[given] * inv_t : -INFINITY;
+      logprobs[r] = (given >= 0 && given < V && ordered_key(x) >= floor_key) ? x - mx - logf(sum) : kMasked;
+    }
+    return;
+  }
   const uint64_t sd = seed[r];
   const uint32_t ctr = static_cast<uint32_t>(counter[r]);
   ArgMax a{-INFINITY, 0x7fffffff};
@@ -587,9 +628,18 @@ extern "C" int sa_sample(const float* logits, int64_t row_stride, int R, int V, 
       draws = nullptr;
     if (check_launch("sample (parts)")) return 1;
   }
-  sample_kernel<<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed, counter,
-                                                  tokens, logprobs, parts, draws, selected);
+  sample_kernel<false><<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, seed, counter,
+                                                         tokens, logprobs, parts, draws, selected);
   return check_launch("sample");
+}
+
+extern "C" int sa_score(const float* logits, int64_t row_stride, int R, int V, const float* temperature,
+                        const int* top_k, const float* top_p, const int* tokens, float* scores, hipStream_t stream) {
+  if (R == 0) return 0;
+  SA_REQUIRE(R > 0 && V > 0 && row_stride >= V, "score: bad sizes R=%d V=%d stride=%lld", R, V, (long long)row_stride);
+  sample_kernel<true><<<R, kSampleThreads, 0, stream>>>(logits, row_stride, V, temperature, top_k, top_p, nullptr, nullptr,
+                                                        const_cast<int*>(tokens), scores, nullptr, nullptr, 0);
+  return check_launch("score");
 }
 
 // Host-side copy of the generator, for tests of the kernel's random stream.

@@ -13,7 +13,7 @@ from typing import Sequence
 import torch
 
 from ..config import EngineConfig, load_config
-from ..sampling import Sampler, SamplingParams, request_seed
+from ..sampling import Sampler, SamplingParams, ScoringParams, request_seed
 from .executor import Executor, StepEntry
 from .loading import load_model, random_model
 from .scheduler import Request, Scheduled, Scheduler, Status
@@ -185,6 +185,46 @@ class LMInterface:
         self.stats["seconds"] += time.perf_counter() - t0
         return [SamplingOutput(list(r.prompt_token_ids), list(r.output_token_ids), list(r.output_token_logprobs),
                                r.is_truncated, r.finish_reason or "", r.num_preemptions) for r in requests]
+
+
+    # ------------------------------------------------------------------ score
+    def score_tokens(self, tokens: Sequence[int], scoring_params: ScoringParams | None = None) -> list[float]:
+        """The log-likelihood of tokens[1:], each given the tokens before it (simply/model_lib.py:4995-5036:
+        the model runs on tokens[:-1], the scores are `compute_log_likelihood` of simply/utils/sampling_lib.py:540-601
+        under the scoring parameters' temperature, top-k and top-p).  The tokens go through the step function in
+        portions, as a request of their own beside whatever else is live; logits of a portion are scored on the
+        device and only the scores come back."""
+        from ..kernels import ops
+
+        sp = scoring_params or ScoringParams()
+        sp.validate()
+        vocab = self.model.spec.vocab_size
+        ids = [int(t) for t in tokens]
+        if any(t < 0 or t >= vocab for t in ids):
+            raise ValueError(f"score_tokens: token id outside [0, {vocab})")
+        n = len(ids) - 1
+        if n < 1:
+            return []
+        if n > self.engine_config.max_seq_len:
+            raise ValueError(f"score_tokens: {n} tokens to run, max_seq_len is {self.engine_config.max_seq_len}")
+        ex, dev = self.executor, self.executor.device
+        # logits of a portion: float32 [rows, vocab], 256 MiB at most
+        rows = max(1, min(self.engine_config.issue_budget, (64 << 20) // vocab))
+        self._num_scored = getattr(self, "_num_scored", 0) + 1
+        rid = ("score", self._num_scored)
+        out = []
+        ex.add_request(rid)
+        try:
+            for i in range(0, n, rows):
+                part = ids[i:min(i + rows, n)]
+                logits = ex.step([StepEntry(rid, part, list(range(len(part))))])
+                given = torch.tensor(ids[i + 1:i + 1 + len(part)], dtype=torch.int32, device=dev)
+                full = lambda v, dt: torch.full((len(part),), v, dtype=dt, device=dev)
+                out.append(ops.score(logits, full(sp.temperature, torch.float32), full(sp.top_k, torch.int32),
+                                     full(sp.top_p, torch.float32), given))
+        finally:
+            ex.finish_request(rid)
+        return torch.cat(out).tolist()
 
 
 LLM = LMInterface

@@ -43,6 +43,7 @@ _SIGNATURES = {
     "sa_paged_attention_prefill_group": [],
     "sa_gemm_normed_rotary": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _P, _P, _F, _F, _P, _P,
                               _P, _I, _I, _I, _I, _P],
+    "sa_score": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }
 

@@ -551,6 +551,34 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     return tokens, logprobs
 
 
+#: what `score` gives for a token that is left out (the reference's neg_inf for float32)
+SCORE_MASKED = -0.5 * 3.4028234663852886e38
+
+
+def score(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+          tokens: torch.Tensor, scores: torch.Tensor | None = None) -> torch.Tensor:
+    """The log-probability of tokens[r] under row r's temperature, top-k and top-p, as `sample` reports it for the
+    token it draws: greedy rows give 0 for the argmax and SCORE_MASKED otherwise, a token that the masks leave out
+    gives SCORE_MASKED."""
+    _dev(logits, temperature, top_k, top_p, tokens, scores)
+    if logits.dtype != torch.float32:
+        raise KernelError("score: logits must be float32")
+    stride = _rows(logits, "score: logits")
+    R, V = logits.shape
+    for t, dt, name in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                        (top_p, torch.float32, "top_p")):
+        if t.dtype != dt or t.numel() < R or not t.is_contiguous():
+            raise KernelError(f"score: {name} must be a contiguous {dt} tensor with one entry per row")
+    _i32(tokens, "score: tokens", R)
+    if scores is None:
+        scores = torch.empty(R, dtype=torch.float32, device=logits.device)
+    if scores.dtype != torch.float32 or scores.numel() < R or not scores.is_contiguous():
+        raise KernelError("score: scores must be a contiguous float32 tensor with one entry per row")
+    _lib.call("sa_score", _ptr(logits), stride, R, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(tokens),
+              _ptr(scores), _stream())
+    return scores
+
+
 def philox4x32_10(counter: tuple[int, int, int, int], key: tuple[int, int]) -> tuple[int, int, int, int]:
     """Host function: one block of the generator that `sample` uses."""
     c = (ctypes.c_uint32 * 4)(*counter)

@@ -1,4 +1,4 @@
-from .params import SamplingParams
+from .params import SamplingParams, ScoringParams
 from .sampler import Sampler, request_seed
 
-__all__ = ["SamplingParams", "Sampler", "request_seed"]
+__all__ = ["SamplingParams", "ScoringParams", "Sampler", "request_seed"]

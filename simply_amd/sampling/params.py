@@ -38,3 +38,19 @@ class SamplingParams:
     @property
     def is_greedy(self) -> bool:
         return self.temperature == 0 or self.top_k == 1
+
+
+@dataclasses.dataclass(frozen=True)
+class ScoringParams:
+    """What a token's score is computed under (simply/model_lib.py:4521-4533)."""
+
+    temperature: float = 1.0
+    top_k: int = -1
+    top_p: float = 1.0
+
+    @classmethod
+    def from_sampling_params(cls, sampling_params: SamplingParams) -> "ScoringParams":
+        return cls(temperature=sampling_params.temperature, top_k=sampling_params.top_k, top_p=sampling_params.top_p)
+
+    def validate(self) -> None:
+        SamplingParams(temperature=self.temperature, top_k=self.top_k, top_p=self.top_p).validate()

@@ -31,7 +31,7 @@ def cpu_ops(monkeypatch):
     from simply_amd.kernels import ops
 
     for name in ("embed", "rmsnorm", "add_rmsnorm", "rope_cache_write", "rope", "gather_rows", "fill_", "gemm",
-                 "paged_attention", "sample", "decode_attention_takes"):
+                 "paged_attention", "sample", "score", "decode_attention_takes"):
         monkeypatch.setattr(ops, name, getattr(torch_ops, name))
     return torch_ops
 

@@ -5,7 +5,7 @@ import torch
 import plain_gemma2 as plain
 import tiny
 from simply_amd.engine.llm import LMInterface
-from simply_amd.sampling import SamplingParams
+from simply_amd.sampling import SamplingParams, ScoringParams
 
 
 def lm(d, **kw):
@@ -80,3 +80,26 @@ def test_steps_in_a_row_change_nothing(tmp_path, cpu_ops):
         assert [o.finish_reason for o in outs] == [o.finish_reason for o in one]
         many.executor.cache.check()
         assert many.stats["steps"] >= max(len(o.output_token_ids) for o in one)
+
+
+def test_score_tokens(tmp_path, cpu_ops):
+    """Scores are the log-softmax of the plain implementation's logits at the next token, in portions beside a
+    pool that is used again; greedy scoring says 0 where the token is the argmax."""
+    d = tiny.write_model("A", str(tmp_path / "A"), std=0.5)
+    w, cfg = plain.load(d)
+    toks = tiny.random_tokens(41, cfg["vocab_size"], 90)
+    logits = plain.forward(w, cfg, toks[:-1], torch.float64)
+    m = lm(d, max_num_issue_tokens=7)
+    for _ in range(2):
+        got = m.score_tokens(toks)
+        want = [plain.log_prob(logits[i], toks[i + 1], 1.0) for i in range(40)]
+        assert len(got) == 40 and max(abs(a - b) for a, b in zip(got, want)) < 1e-4
+    got = m.score_tokens(toks, ScoringParams(temperature=0.7))
+    want = [plain.log_prob(logits[i], toks[i + 1], 0.7) for i in range(40)]
+    assert max(abs(a - b) for a, b in zip(got, want)) < 1e-4
+    best = [int(torch.argmax(logits[i])) for i in range(40)]
+    got = m.score_tokens(toks, ScoringParams(temperature=0.0))
+    assert all((g == 0.0) == (toks[i + 1] == best[i]) for i, g in enumerate(got)) and min(got) < -1e37
+    assert m.score_tokens([5]) == [] and m.score_tokens([]) == []
+    m.executor.cache.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in m.executor.cache.groups)

@@ -11,7 +11,7 @@ import torch
 import plain_gemma2 as plain
 import tiny
 from simply_amd.engine.llm import LMInterface
-from simply_amd.sampling import SamplingParams
+from simply_amd.sampling import SamplingParams, ScoringParams
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -101,3 +101,27 @@ def test_steps_in_a_row_on_the_device(tmp_path, gpu_lib, dtype):
     out = lm_eos.generate([prompts[0]], sampling_params=[SamplingParams(temperature=0.0, max_decode_steps=37)])[0]
     assert out.output_token_ids == one[0].output_token_ids[:one[0].output_token_ids.index(eos) + 1]
     assert out.finish_reason == "eos"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_score_tokens(tmp_path, gpu_lib, dtype):
+    """`score_tokens` against the log-softmax of the plain implementation's logits, in portions, beside live
+    requests' pages; what `generate` reports for the tokens it drew is what scoring them gives."""
+    d = tiny.write_model("D", str(tmp_path / "D"), dtype=torch.bfloat16, std=0.15)
+    w, cfg = plain.load(d)
+    toks = tiny.random_tokens(150, cfg["vocab_size"], 91)
+    logits = plain.forward(w, cfg, toks[:-1], torch.float64)
+    tol = 1e-4 if dtype == "float32" else 0.15
+    m = lm(d, activation_dtype=dtype, max_seq_len=256, page_size=16, max_num_issue_tokens=48)
+    for temp in (1.0, 0.6):
+        got = m.score_tokens(toks, ScoringParams(temperature=temp))
+        want = [plain.log_prob(logits[i], toks[i + 1], temp) for i in range(len(toks) - 1)]
+        assert len(got) == len(want) and max(abs(a - b) for a, b in zip(got, want)) < tol
+    sp = SamplingParams(temperature=0.8, top_k=20, max_decode_steps=12, seed=5, ignore_eos=True)
+    out = m.generate([toks[:30]], sampling_params=sp)[0]
+    seq = out.input_token_ids + out.output_token_ids
+    scores = m.score_tokens(seq, ScoringParams.from_sampling_params(sp))
+    tail = scores[len(out.input_token_ids) - 1:]
+    assert max(abs(a - b) for a, b in zip(tail, out.output_token_logprobs)) < (1e-4 if dtype == "float32" else 0.1)
+    m.executor.cache.check()
+    assert all(g.pool.num_free == g.pool.num_pages for g in m.executor.cache.groups)

@@ -531,6 +531,36 @@ def test_sampling_top_k_and_top_p_of_a_large_vocabulary(V):
         torch.testing.assert_close(lp, rlp[idx], rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("V", [333, 1001, 20000])
+def test_score(V):
+    """The log-probability of a given token under temperature, top-k and top-p against the reference: the token
+    that the sampler draws scores what the sampler reports for it; tokens inside and outside the masks; greedy rows;
+    equal entries at a top-k boundary; rows at odd addresses."""
+    from simply_amd.kernels import ops
+    R = 9
+    wide = rand((R, V + 3), torch.float32, 97, 2.5)
+    logits = wide[:, 1:1 + V]
+    logits[6, 100:105] = 20.0
+    temperature = torch.tensor([0.8, 1.3, 0.7, 1.0, 0.0, 0.9, 0.5, 2.0, 1.0]).cuda()
+    top_k = torch.tensor([40, -1, 50, V + 5, -1, -1, 3, -1, 1], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 0.9, 0.8, 1.0, 1.0, 1.0, 1.0, 0.3, 1.0]).cuda()
+    seed = torch.arange(R, dtype=torch.int64).cuda() * 5 + 3
+    counter = torch.full((R,), 2, dtype=torch.int32).cuda()
+    tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
+    torch.testing.assert_close(ops.score(logits, temperature, top_k, top_p, tok), lp, rtol=1e-5, atol=1e-5)
+    best, worst = logits.argmax(-1).int(), logits.argmin(-1).int()
+    fifth = logits.topk(5).indices[:, 4].int().contiguous()
+    for given in (tok, best, worst, fifth, torch.full((R,), 104, dtype=torch.int32).cuda()):
+        got = ops.score(logits, temperature, top_k, top_p, given)
+        want = ref.score(logits, temperature, top_k, top_p, given)
+        masked = want < -1e37
+        assert torch.equal(got < -1e37, masked), (given.tolist(), got.tolist(), want.tolist())
+        torch.testing.assert_close(got[~masked], want[~masked], rtol=1e-4, atol=1e-4)
+        assert (got[masked] == ops.SCORE_MASKED).all()
+    got = ops.score(logits, temperature, top_k, top_p, worst)
+    assert got[4] == ops.SCORE_MASKED and got[8] == ops.SCORE_MASKED and got[5] > -1e3   # greedy rows; a plain draw
+
+
 @pytest.mark.parametrize("M", [1, 8, 13, 16])
 @pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (3584, 512), (4608, 64), (4640, 64), (96, 40),
                                  (72, 64)])

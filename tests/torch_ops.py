@@ -232,3 +232,36 @@ def sample(logits, temperature, top_k, top_p, seed, counter, tokens=None, logpro
         logprobs[:R] = lps
         lps = logprobs
     return toks, lps
+
+
+SCORE_MASKED = -0.5 * 3.4028234663852886e38
+
+
+def score(logits, temperature, top_k, top_p, tokens, scores=None):
+    """simply/utils/sampling_lib.py:540-601: the log-probability of a given token under temperature, top-k, top-p."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(__file__))
+    import plain_gemma2 as plain
+
+    R, V = logits.shape
+    out = torch.empty(R, dtype=torch.float32)
+    for r in range(R):
+        row = logits[r].double().cpu()
+        t, k, p, tok = float(temperature[r]), int(top_k[r]), float(top_p[r]), int(tokens[r])
+        if t == 0.0 or k == 1:
+            out[r] = 0.0 if int(torch.argmax(row)) == tok else SCORE_MASKED
+            continue
+        x = row / t
+        keep = torch.ones(V, dtype=torch.bool)
+        if k > 0:
+            keep &= x >= torch.topk(x, min(k, V)).values[-1]
+        if p < 1.0:
+            xm = torch.where(keep, x, torch.full_like(x, -float("inf")))
+            keep &= plain.top_p_mask(xm, p)
+        xm = torch.where(keep, x, torch.full_like(x, -float("inf")))
+        out[r] = float(torch.log_softmax(xm, -1)[tok]) if bool(keep[tok]) else SCORE_MASKED
+    out = out.to(logits.device)
+    if scores is not None:
+        scores[:R] = out
+        out = scores
+    return out
