@@ -302,13 +302,14 @@ class CacheManager:
                 return False
         return True
 
-    def reserve(self, rid: Hashable, num_computed: int, q_len: int) -> None:
+    def reserve(self, rid: Hashable, num_computed: int, q_len: int, *, fits: bool = False) -> None:
         """Makes room for tokens [num_computed, num_computed + q_len) in every group: first gives back
         the pages that the window has passed, then takes new ones.  Raises OutOfPages, with nothing
-        changed, if any group is short."""
+        changed, if any group is short (fits: the caller has asked `can_reserve` for this and the rest of what it
+        reserves, so that is not asked again)."""
         if num_computed + q_len > self.max_seq_len:
             raise CacheError(f"request {rid!r}: {num_computed + q_len} tokens exceed max_seq_len {self.max_seq_len}")
-        for g in self.groups:
+        for g in self.groups if not fits else ():
             short = g.pages_needed(rid, num_computed, q_len) - g.pool.num_free
             if short > 0:
                 raise OutOfPages(f"group {g.group_id} (window {g.need.window}): {short} pages short for request "
@@ -347,6 +348,11 @@ class CacheManager:
     def slot_mapping(self, group_id: int, rid: Hashable, start: int, q_len: int) -> np.ndarray:
         """Storage slot (page * page_size + offset) of positions [start, start + q_len)."""
         g = self.groups[group_id]
+        if q_len == 1:  # a decoded token: plain integers
+            page = int(g.table[g.seqs[rid].slot, start // g.page_size])
+            if page < 0:
+                raise CacheError(f"request {rid!r}: position {start} has no page in group {group_id}")
+            return np.array([page * g.page_size + start % g.page_size], dtype=np.int64)
         pos = np.arange(start, start + q_len, dtype=np.int64)
         pages = g.table[g.seqs[rid].slot, pos // g.page_size].astype(np.int64)
         if (pages < 0).any():

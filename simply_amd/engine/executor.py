@@ -231,7 +231,7 @@ class Executor:
             raise OutOfPages("the cache cannot hold this step's tokens: " + ", ".join(
                 f"{rid!r}+{q}" for rid, _, q in wants))
         for rid, start, q in wants:
-            cache.reserve(rid, start, q)
+            cache.reserve(rid, start, q, fits=True)
 
         if self._copied is not None:
             self._copied.synchronize()  # the last step's copy out of the staging buffer has finished
@@ -245,12 +245,18 @@ class Executor:
         for j, i in enumerate(order):
             e, (rid, start, reserved) = entries[i], wants[i]
             q = len(e.tokens)
-            ids = np.asarray(e.tokens, dtype=np.int64)
-            if ids.min() < 0 or ids.max() >= self.vocab_size:
-                raise ValueError(f"request {rid!r}: token id outside [0, {self.vocab_size})")
             slot = cache.slot_of(rid)
+            if q == 1:  # a decoded token: no arrays
+                ids = int(e.tokens[0])
+                bad = not 0 <= ids < self.vocab_size
+                pos[t0] = start
+            else:
+                ids = np.asarray(e.tokens, dtype=np.int64)
+                bad = ids.min() < 0 or ids.max() >= self.vocab_size
+                pos[t0:t0 + q] = np.arange(start, start + q)
+            if bad:
+                raise ValueError(f"request {rid!r}: token id outside [0, {self.vocab_size})")
             tok[t0:t0 + q] = ids
-            pos[t0:t0 + q] = np.arange(start, start + q)
             seq[t0:t0 + q] = slot
             meta[j] = (slot, t0, q, start)
             for g in cache.groups:
