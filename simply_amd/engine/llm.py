@@ -87,6 +87,7 @@ class LMInterface:
         self.intermediate_steps = max(1, int(intermediate_steps))
         self.seed = int(seed)
         self._num_requests = 0
+        self._num_scored = 0
         self.stats = {"steps": 0, "tokens": 0, "preemptions": 0, "seconds": 0.0}
 
     # ------------------------------------------------------------------ requests
@@ -210,7 +211,7 @@ class LMInterface:
         ex, dev = self.executor, self.executor.device
         # logits of a portion: float32 [rows, vocab], 256 MiB at most
         rows = max(1, min(self.engine_config.issue_budget, (64 << 20) // vocab))
-        self._num_scored = getattr(self, "_num_scored", 0) + 1
+        self._num_scored += 1
         rid = ("score", self._num_scored)
         out = []
         ex.add_request(rid)
