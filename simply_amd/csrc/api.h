@@ -118,6 +118,8 @@ int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pag
 // for all of them.  unit_count is a multiple of the group (sa_paged_attention_prefill_group units) and the units of a
 // group belong to one request; units with no tokens fill up a request's last group.
 int sa_paged_attention_prefill_group();
+// Whether the bfloat16 MFMA attention kernels (sa_paged_attention_decode and _prefill) take these sizes.
+int sa_paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q);
 int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
                                int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,

@@ -113,6 +113,11 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
                                 workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
 }
 
+extern "C" int sa_paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride,
+                                               const void* q) {
+  return H > 0 && Kh > 0 && H % Kh == 0 && paged_attention_decode_takes(H, Kh, hd, page_size, max_q_len, q_stride, q);
+}
+
 extern "C" int sa_paged_attention_prefill_group() { return paged_attention_prefill_group(); }
 
 extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,

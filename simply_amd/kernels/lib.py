@@ -41,6 +41,7 @@ _SIGNATURES = {
     "sa_gemm_normed": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _I, _I, _F, _P],
     "sa_gemm_normed_takes": [_I, _I, _I],
     "sa_paged_attention_prefill_group": [],
+    "sa_paged_attention_decode_takes": [_I, _I, _I, _I, _I, _L, _P],
     "sa_gemm_normed_rotary": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _P, _P, _F, _F, _P, _P,
                               _P, _I, _I, _I, _I, _P],
     "sa_score": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P],

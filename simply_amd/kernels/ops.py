@@ -461,9 +461,8 @@ def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tenso
 def decode_attention_takes(q: torch.Tensor, k_pages: torch.Tensor, num_heads: int, max_q_len: int) -> bool:
     """Whether `paged_attention_decode` takes requests of up to max_q_len tokens at these sizes."""
     _, Kh, page_size, hd = k_pages.shape
-    G = num_heads // Kh
-    return (q.dtype == torch.bfloat16 and hd in (64, 128, 256) and page_size % 16 == 0 and G * max_q_len <= 16
-            and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
+    return q.dtype == torch.bfloat16 and q.is_cuda and bool(_lib.load().sa_paged_attention_decode_takes(
+        int(num_heads), int(Kh), int(hd), int(page_size), int(max_q_len), q.stride(0), _ptr(q)))
 
 
 def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, begin, count, num_heads, window, soft_cap,
