@@ -684,6 +684,52 @@ def test_paged_attention_prefill_far_key_and_window_edge():
         assert torch.equal(found, sees), (window, (found != sees).nonzero().flatten().tolist()[:10])
 
 
+@pytest.mark.parametrize("window", [None, 30000])
+def test_paged_attention_far_keys_of_a_long_context(window):
+    """70,000 keys (more than 16 bits count): every query must find the one key, planted 3 to 69,000 positions back,
+    whose score stands out for it; in the prompt-portion kernel, the few-rows kernel (keys cut over workgroups) and
+    the generic kernel, with and without a window."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
+    H, Kh, hd, P, L, Q = 2, 1, 128, 16, 70000, 64
+    kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 75)
+    kp = keys_to_rows(kp) * 0.01
+    far = [3, 40001, 65535, 65536, 69000, L - 70]
+    for f, at in enumerate(far):
+        page, off = int(table[0, at // P]), at % P
+        kp[page, 0, off] = 0.0
+        kp[page, 0, off, 5 + f] = 60.0
+        vp[page, 0, :, off] = float(f + 1)
+    kp = rows_to_keys(kp)
+    q = torch.zeros((Q, 4 * hd), dtype=torch.bfloat16).cuda()
+    which = torch.arange(Q) % len(far)
+    for i in range(Q):
+        q[i, 5 + int(which[i])] = 1.0
+        q[i, hd + 5 + int(which[i])] = 1.0
+    positions = torch.arange(L - Q, L)
+    at = torch.tensor(far)[which]
+    sees = (at <= positions) & ((positions - at < window) if window else torch.ones(Q, dtype=torch.bool))
+    want = torch.where(sees, (which + 1).float(), torch.zeros(Q))
+
+    def found(out):
+        m = out.float().mean(dim=1).cpu()
+        return torch.where((m - m.round()).abs() < 0.05, m.round(), torch.full_like(m, -1.0)) * (m.abs() > 0.5)
+
+    units = prefill_units([L], [Q], 8)
+    out = torch.zeros((Q, H * hd), dtype=torch.bfloat16).cuda()
+    ops.paged_attention_prefill(q, kp, vp, table, units, 0, units.shape[0], H, window=window, soft_cap=None,
+                                max_kv_len=L, max_q_len=8, out=out)
+    assert torch.equal(found(out), want), found(out).tolist()
+    out = torch.zeros_like(out)
+    ops.paged_attention_decode(q, kp, vp, table, units, 0, units.shape[0], H, window=window, soft_cap=None,
+                               max_kv_len=L, max_q_len=8, out=out)
+    assert torch.equal(found(out), want), found(out).tolist()
+    out = torch.zeros_like(out)
+    ts, ps = torch.zeros(Q, dtype=torch.int32).cuda(), positions.int().cuda()
+    ops.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=None, out=out)
+    assert torch.equal(found(out), want), found(out).tolist()
+
+
 def test_bfloat16_rounding_of_the_kernels():
     """The device's conversion to bfloat16 rounds to nearest even, as torch does: all exponents, ties, subnormals."""
     from simply_amd.kernels import ops
