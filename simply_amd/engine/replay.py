@@ -28,6 +28,10 @@ MAX_LIVE_REQUESTS = 4
 ROUND_TOKENS_TO = 64
 
 
+class ReplayError(RuntimeError):
+    """A step that could not be run: the line, and what the engine said."""
+
+
 def build_executor(model_dir: str, dtype: str, max_tokens: int, *, device: str = "cuda:0",
                    page_size: int = 16, poison: bool = False) -> Executor:
     if ROUND_TOKENS_TO % page_size:
@@ -71,8 +75,14 @@ def replay(executor: Executor, lines: IO[str], out_dir: str, done: IO[str] = sys
         line = line.strip()
         if not line:
             continue
-        record = json.loads(line)
-        run_step(executor, record, out_dir)
+        try:
+            record = json.loads(line)
+            if not isinstance(record, dict) or "step" not in record:
+                raise ValueError('a step is a JSON object with "step", "entries" and "end"')
+            run_step(executor, record, out_dir)
+        except Exception as e:  # which step, then the error as it is
+            raise ReplayError(f"line {n + 1} ({line[:60]}{'...' if len(line) > 60 else ''}): "
+                              f"{type(e).__name__}: {e}") from e
         print(f"done {record['step']}", file=done, flush=True)
         n += 1
     return n
@@ -90,11 +100,20 @@ def main(argv=None) -> int:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--poison", action="store_true", help="fill freed pages with NaN")
     args = ap.parse_args(argv)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("trace_run: no GPU is visible; this engine has no CPU path", file=sys.stderr, flush=True)
+        return 3
     print("[trace_run] loading kernels and model ...", file=sys.stderr, flush=True)
     from ..kernels import lib
 
     lib.load()
     executor = build_executor(args.model, args.dtype, args.max_tokens, page_size=args.page_size, poison=args.poison)
     print("[trace_run] ready", file=sys.stderr, flush=True)
-    replay(executor, sys.stdin, args.out)
+    try:
+        replay(executor, sys.stdin, args.out)
+    except ReplayError as e:
+        print(f"trace_run: {e}", file=sys.stderr, flush=True)
+        return 1
     return 0

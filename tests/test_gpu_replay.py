@@ -142,3 +142,24 @@ def test_replay_long_decoding(tmp_path, dtype):
         assert rel_err(got, want) <= TOL[dtype]
     finally:
         tr.close()
+
+
+def test_replay_says_which_line_is_wrong(tmp_path):
+    """A step that cannot be run ends the program with status 1 and one line that names it: broken JSON, a wanted
+    place outside the tokens, a token outside the vocabulary, more tokens than the pool holds."""
+    d = tiny.write_model("A", str(tmp_path / "m"), dtype=torch.bfloat16, std=0.3)
+    good = '{"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [2]}], "end": []}'
+    bad = {
+        "JSONDecodeError": '{"step": 1, "entries": [',
+        "wanted place": '{"step": 1, "entries": [{"id": "a", "tokens": [5, 6], "want": [2]}], "end": []}',
+        "token id": '{"step": 1, "entries": [{"id": "a", "tokens": [5, 100000], "want": []}], "end": []}',
+        "OutOfPages": json.dumps({"step": 1, "entries": [{"id": "b", "tokens": [1] * 64, "want": []}], "end": []}),
+    }
+    for what, line in bad.items():
+        p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", "float32",
+                            "--out", str(tmp_path / "out"), "--max-tokens", "64"], input=good + "\n" + line + "\n",
+                           capture_output=True, text=True, timeout=120)
+        assert p.returncode == 1, (what, p.returncode, p.stderr[-300:])
+        assert p.stdout.strip() == "done 0"
+        last = p.stderr.strip().splitlines()[-1]
+        assert last.startswith("trace_run: line 2") and what in last, (what, last)
