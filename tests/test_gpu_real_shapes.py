@@ -1,4 +1,4 @@
-"""The layer sizes of Gemma 2 2B and 27B (width, heads, head size, feed-forward width as in the reference's
+"""The layer sizes of Gemma 2 2B, 9B and 27B (width, heads, head size, feed-forward width as in the reference's
 configs, simply/config_lib.py:852-949) with two layers, a cut-down vocabulary and random weights: the
 bfloat16 kernels at the sizes they are built for, and the float32 path, against the plain implementation."""
 import pytest
@@ -16,13 +16,15 @@ pytestmark = pytest.mark.gpu
 SHAPES = {
     "2b": dict(hidden_size=2304, num_attention_heads=8, num_key_value_heads=4, head_dim=256, intermediate_size=9216,
                query_pre_attn_scalar=256),
+    "9b": dict(hidden_size=3584, num_attention_heads=16, num_key_value_heads=8, head_dim=256, intermediate_size=14336,
+               query_pre_attn_scalar=256),
     "27b": dict(hidden_size=4608, num_attention_heads=32, num_key_value_heads=16, head_dim=128, intermediate_size=36864,
                 query_pre_attn_scalar=144),
 }
 
 
 @pytest.mark.parametrize("dtype,tol", [("float32", 5e-5), ("bfloat16", 3e-2)])
-@pytest.mark.parametrize("shape", ["2b", "27b"])
+@pytest.mark.parametrize("shape", ["2b", "9b", "27b"])
 def test_real_layer_shapes(tmp_path, gpu_lib, shape, dtype, tol):
     d = dict(architectures=["Gemma2ForCausalLM"], num_hidden_layers=2, vocab_size=2000, rms_norm_eps=1e-6,
              rope_theta=10000.0, sliding_window=48, attn_logit_softcapping=50.0, final_logit_softcapping=30.0,
