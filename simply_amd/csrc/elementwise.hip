@@ -51,7 +51,7 @@ __global__ void rmsnorm_kernel(const void* __restrict__ x, int x_dtype, int64_t 
 // Rows of up to kRowRegs * blockDim elements are held in registers: every input is read once and all loads are
 // issued before the first reduction, so that the kernel pays the memory latency once (it runs a hundred times
 // per decode step on a handful of rows).
-constexpr int kRowRegs = 4;
+constexpr int kRowRegs = 5;  // (1024 threads hold 5120: the width of the 27B shape is 4608)
 __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, const void* __restrict__ w_post,
                                    int w_post_dtype, float eps_post, float plus_one_post, float* __restrict__ residual,
                                    const void* __restrict__ w_next, int w_next_dtype, float eps_next,

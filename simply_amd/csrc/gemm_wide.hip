@@ -279,14 +279,15 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     // The cost of a shape: the workgroups that the busiest CU gets times the size of the tile; of equals the first.
     // Workgroups of four waves run two to a CU, where one's epilogue and first loads overlap the other's
     // products (measured: 7-9 % faster than one workgroup of twice the tile once every CU has two of them;
-    // slower when it has one).
+    // slower when it has one; from one and a half per CU on it is also the best for few rows of very many weight
+    // rows, which are bound by streaming them).
     const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
     const int shapes[5][4] = {{2128192, 128, 192, 93}, {2256192, 256, 192, 100}, {3256128, 256, 128, 100},
                               {3128256, 128, 256, 100}, {3192128, 192, 128, 100}};
     int64_t best = -1;
     for (const auto& sh : shapes) {
       const int64_t tiles = static_cast<int64_t>((M + sh[1] - 1) / sh[1]) * ((NW + sh[2] - 1) / sh[2]);
-      if (sh[3] < 100 && tiles < 2 * wide::kCUs) continue;
+      if (sh[3] < 100 && tiles < wide::kCUs * 3 / 2) continue;
       const int64_t cost = ((tiles + wide::kCUs - 1) / wide::kCUs) * sh[1] * sh[2] * sh[3];
       if (best < 0 || cost < best) {
         best = cost;
