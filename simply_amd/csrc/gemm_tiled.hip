@@ -289,10 +289,11 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
   } else if (few) {
     // few rows: the product is bound by streaming W, so it needs a workgroup or two per CU even when N is small:
     // waves side by side (64 rows x 256 weight rows per workgroup), K cut over workgroups
-    // (measured at 64 rows: about 200 workgroups of at least four slabs each; more cuts cost more in the sum of
-    // the partial tiles than they gain)
+    // (measured at 32 and 64 rows at the 2B, 9B and 27B sizes: about a workgroup per CU of at least four slabs
+    // each, nearly two per CU where K is long; more cuts cost more in the sum of the partial tiles than they gain)
     const int tiles = (NW + 255) / 256;
-    ks = (200 + tiles / 2) / tiles;
+    const int target = K >= 8192 ? 440 : 256;
+    ks = (target + tiles / 2) / tiles;
     if (ks > stages / 4) ks = stages / 4;
   }
   if (ks > stages) ks = stages;
