@@ -47,8 +47,12 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
   // up to 16 rows, and up to 32 for products without the gated epilogue and with K below 4608 (measured at the
   // 2B, 9B and 27B sizes: the few-rows kernel, whose waves read the activations from L2, beats the tiled one with
-  // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower)
-  if (algo == 2 || (algo == 0 && bf16_in && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4608)))) {
+  // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower).  Not from 8 rows on
+  // against so many weight rows that the tiled kernel fills the GPU without a cut of K (the head over a large
+  // vocabulary: 7 % faster at 8 rows, 30 % at 16, 80 % at 32; up to 6 rows the few-rows kernel wins).
+  const bool many_weight_rows = packed && epilogue != 1 && M >= 8 && N >= 65536;
+  if (algo == 2 ||
+      (algo == 0 && bf16_in && !many_weight_rows && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4608)))) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
@@ -70,7 +74,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                (long long)ldc, packed);
     if (takes) return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, algo == 4 ? shape : 0, stream);
   }
-  if (algo == 3 || (algo == 0 && bf16_in && packed && M > 16)) {
+  if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || many_weight_rows))) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
