@@ -50,9 +50,13 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower).  Not from 8 rows on
   // against so many weight rows that the tiled kernel fills the GPU without a cut of K (the head over a large
   // vocabulary: 7 % faster at 8 rows, 30 % at 16, 80 % at 32; up to 6 rows the few-rows kernel wins).
+  // Nor against a very long K (the 27B down projection, 36864: the tiled kernel with its cut of K is 15 % faster at
+  // one row and 40 % at 16; at the 9B size, 14336, the few-rows kernel still wins up to 12 rows).
   const bool many_weight_rows = packed && epilogue != 1 && M >= 8 && N >= 65536;
+  const bool long_k = packed && epilogue != 1 && K >= 24576;
+  const bool tiled_first = many_weight_rows || long_k;
   if (algo == 2 ||
-      (algo == 0 && bf16_in && !many_weight_rows && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4608)))) {
+      (algo == 0 && bf16_in && !tiled_first && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4608)))) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
@@ -74,7 +78,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                (long long)ldc, packed);
     if (takes) return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, algo == 4 ? shape : 0, stream);
   }
-  if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || many_weight_rows))) {
+  if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || tiled_first))) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
