@@ -117,7 +117,7 @@ class PendingNorm:
 
 def pending_fits_product(x, w) -> bool:
     """Whether the product kernel with the norms in front takes the pending norm `x` against the weight `w`
-    (bfloat16, up to 16 rows, a tiled weight, RMSNorms with bfloat16 scales)."""
+    (bfloat16, up to 16 rows, a tiled weight of rows up to 2560 wide, RMSNorms with bfloat16 scales)."""
     from ..kernels import ops
     from ..kernels.packing import TiledWeight
 
@@ -128,6 +128,10 @@ def pending_fits_product(x, w) -> bool:
             and nn.scale.dtype == torch.bfloat16
             and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
             and isinstance(w, TiledWeight) and w.rows <= 16 * 2048   # every workgroup redoes the norms
+            # wider rows than 2560 leave the kernel too few registers to have its first weights on their way during
+            # the norms: measured at widths 3584 and 4608, the separate kernels are as fast at 8 rows and 10-20 %
+            # faster at 16
+            and w.cols <= 2560
             and ops.gemm_normed_takes(x.residual.shape[0], w)
             and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
 
