@@ -168,7 +168,7 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
                      const void* C, int c_dtype, int epi, int packed);
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
               hipStream_t stream);
-bool gemm_streams_weights(int M, int NW);
+bool gemm_streams_weights(int M, int NW, int K);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
                int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream);

@@ -13,6 +13,7 @@
 //
 // Epilogues: none; gated (C = gelu_tanh(A.Wg^T) * (A.Wu^T), both rounded to bfloat16 first, from one weight
 // whose tiles alternate between Wg and Wu); soft-cap (C = cap * tanh(. / cap), float32 out).
+#include <cmath>
 #include "api.h"
 #include "common.h"
 
@@ -262,11 +263,15 @@ static void launch(const bf16* A, int64_t lda, const bf16* W, void* C, int c_dty
 
 }  // namespace tiled
 
-// Whether a product of M rows against NW weight rows is bound by streaming the weights rather than by the MFMA
-// units: then workgroups take 64 rows x 256 weight rows with K cut over them.  Measured at the 2B sizes against
-// the wide-tile kernel: up to 64 rows always, beyond that while M * NW stays below about a million (192 rows of
-// the q/k/v projection, 384 of the output and down projections, never the paired gate/up weight).
-bool gemm_streams_weights(int M, int NW) { return M <= 64 || static_cast<int64_t>(M) * NW <= 1000000; }
+// Whether a product of M rows against NW weight rows of length K is better off with 64 rows x 256 weight rows per
+// workgroup and K cut over workgroups than with the wide-tile kernel.  Measured at the 2B, 9B and 27B sizes: up to
+// 64 rows always; beyond that while M * NW stays below about a million (192 rows of a q/k/v projection, 256 to 384
+// of an output projection), and further the longer K is (the down projections: to 384 rows at K = 9216 and 14336,
+// to 512 at 36864), where the wide kernel's few tiles would each walk all of K on a fraction of the CUs.
+bool gemm_streams_weights(int M, int NW, int K) {
+  const double limit = K <= 9216 ? 1.0e6 : 1.0e6 * pow(static_cast<double>(K) / 9216.0, 0.85);
+  return M <= 64 || static_cast<double>(M) * NW <= limit;
+}
 
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed) {
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
@@ -282,7 +287,7 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
   float* ws = static_cast<float*>(workspace);
   const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const int stages = (K + tiled::BK - 1) / tiled::BK;
-  const bool few = gemm_streams_weights(M, NW);
+  const bool few = gemm_streams_weights(M, NW, K);
   int ks = 1;
   if (ksplit > 0) {
     ks = ksplit;

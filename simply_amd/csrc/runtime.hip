@@ -69,7 +69,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   // without a cut of K (measured at 32 and 64 rows: 10-20 % faster than the tiled kernel with its sum kernel at the
   // 2B, 9B and 27B sizes)
   const int NW = epilogue == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-  const bool wide_first = !gemm_streams_weights(M, NW) || (epilogue == 1 && M > 16);
+  const bool wide_first = !gemm_streams_weights(M, NW, K) || (epilogue == 1 && M > 16);
   if (algo == 4 || (algo == 0 && bf16_in && packed && wide_first)) {
     const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
     SA_REQUIRE(takes || algo == 0,
