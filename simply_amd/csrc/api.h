@@ -113,6 +113,24 @@ int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pag
                               int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                               void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
+// sa_paged_attention_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
+// serving loops, harnesses that forbid hipMalloc): the same kernels, the same result, but the partial results of
+// the key ranges go into an array of sa_paged_attention_decode_static_bytes() bytes (16 MiB) that is part of the
+// library's code object, so no workspace is passed and nothing is allocated, by this call or by anything it calls.
+// It has no counterpart in the reference (whose attention kernel keeps its scratch inside a compiled program).
+// Sizes whose partial results (requests x key heads x key ranges x 16 x (head size + 4) floats, for the number of
+// ranges that sa_paged_attention_decode would choose or that num_splits asks for) exceed the array are refused with
+// an error, never run with fewer ranges.  Each GPU has one such array, every call on that GPU uses it and leaves
+// its partial results there: calls on one GPU that overlap in time (two streams, two threads) race and must be
+// ordered by the caller.  Nothing in the array has to be zero beforehand: every word that the merge reads has been
+// written by the same call.
+int sa_paged_attention_decode_static_bytes();
+int sa_paged_attention_decode_static(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                     const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
+                                     int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
+                                     int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
+                                     hipStream_t stream);
+
 // The same for portions of prompts: the units (rows of seq_meta, each with (query heads per key head) * tokens <= 16)
 // unit_begin .. unit_begin + unit_count - 1 are taken a group at a time by one workgroup, which reads the keys once
 // for all of them.  unit_count is a multiple of the group (sa_paged_attention_prefill_group units) and the units of a

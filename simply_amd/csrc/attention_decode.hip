@@ -16,8 +16,15 @@
 // turn and merge their (maximum, sum, output) through LDS; key ranges are merged by a second, small
 // kernel from a workspace, in a fixed order (a merge by the workgroup that finishes last would need a
 // device-wide fence, which on this GPU writes back the whole L2).
+#include <mutex>
+
 #include "api.h"
 #include "attention_common.h"
+
+// Scratch memory of sa_paged_attention_decode_static (below): the partial results of the key ranges.  Every GPU that
+// the library runs on holds its own copy, at its own address, until the process ends.
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace sa {
 
@@ -342,13 +349,8 @@ bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_
          (reinterpret_cast<uintptr_t>(q) & 15u) == 0;
 }
 
-int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
-                           const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
-                           void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
-                           float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream) {
-  if (seq_count == 0) return 0;
-  const int G = H / Kh;
+// Into how many ranges the keys of each request are cut (num_splits > 0 asks for that many).
+int paged_attention_decode_ranges(int seq_count, int Kh, int window, int max_kv_len, int num_splits) {
   const int units = seq_count * Kh;
   int span = window > 0 && window < max_kv_len ? window + 16 : max_kv_len;  // keys a request reads at most
   if (span < 1) span = 1;
@@ -362,6 +364,18 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   if (KS > max_tiles) KS = max_tiles;
   if (KS > kMaxSplits) KS = kMaxSplits;
   if (KS < 1) KS = 1;
+  return KS;
+}
+
+int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                           const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
+                           void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
+                           float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
+                           hipStream_t stream) {
+  if (seq_count == 0) return 0;
+  const int G = H / Kh;
+  const int units = seq_count * Kh;
+  int KS = paged_attention_decode_ranges(seq_count, Kh, window, max_kv_len, num_splits);
   const size_t per_split = static_cast<size_t>(units) * 16 * (hd + kRowExtra) * sizeof(float);
   while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
   const dim3 grid(KS, Kh, seq_count);
@@ -386,6 +400,60 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   if (check_launch("paged_attention_decode")) return 1;
   if (KS > 1) return attention_merge_ranges(ws, KS, hd, sm, seq_begin, seq_count, max_q_len, op, out_stride, Kh, G, stream);
   return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same attention with the partial results of the key ranges in memory that the library owns: for callers that
+// cannot allocate.  `scratch` is a host-side stand-in for a device array; its device address on each GPU is asked
+// for once per device (hipGetSymbolAddress) and only that address is ever handed to kernels.
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// The address of `scratch` on the current device (asked for at the first call on that device), or null after
+// set_error().
+static void* static_scratch() {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error("paged_attention_decode_static: no current device (%s, device %d, at most %d devices)",
+              hipGetErrorString(e), device, kMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(::scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("paged_attention_decode_static: the address of the scratch array on device %d is not known: %s",
+                device, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[device] = ptr;
+  }
+  return g_scratch_ptr[device];
+}
+
+int paged_attention_decode_static(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                  const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
+                                  int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
+                                  int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
+                                  hipStream_t stream) {
+  if (seq_count == 0) return 0;
+  // the ranges that the entry point with a workspace chooses when it has room for all of them; here they must fit
+  const int KS = paged_attention_decode_ranges(seq_count, Kh, window, max_kv_len, num_splits);
+  const size_t need = KS > 1 ? static_cast<size_t>(seq_count) * Kh * KS * 16 * (hd + kRowExtra) * sizeof(float) : 0;
+  if (need > kStaticScratchBytes) {
+    set_error("paged_attention_decode_static: %d requests x %d key heads x %d key ranges of head size %d need %zu bytes "
+              "of partial results, the library's own scratch memory holds %zu: fewer requests at a time, or fewer "
+              "ranges (num_splits)", seq_count, Kh, KS, hd, need, kStaticScratchBytes);
+    return 1;
+  }
+  void* ptr = static_scratch();
+  if (ptr == nullptr) return 1;
+  return paged_attention_decode(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, seq_begin, seq_count,
+                                out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len, max_q_len, KS, ptr,
+                                kStaticScratchBytes, stream);
 }
 
 // The same for units with many rows (portions of prompts): one workgroup per (unit, head) takes all 16 rows, 16
@@ -451,3 +519,27 @@ int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const
 }
 
 }  // namespace sa
+
+extern "C" int sa_paged_attention_decode_static_bytes() { return static_cast<int>(kStaticScratchBytes); }
+
+extern "C" int sa_paged_attention_decode_static(const void* q, int64_t q_stride, const void* k_pages,
+                                                const void* v_pages, const int* block_table, int table_stride,
+                                                const int* seq_meta, int seq_begin, int seq_count, void* out,
+                                                int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
+                                                float soft_cap, int max_kv_len, int max_q_len, int num_splits,
+                                                hipStream_t stream) {
+  using namespace sa;
+  if (seq_count == 0) return 0;
+  SA_REQUIRE(seq_count > 0 && seq_begin >= 0 && H > 0 && Kh > 0 && H % Kh == 0,
+             "paged_attention_decode_static: bad counts");
+  SA_REQUIRE(window >= 0 && table_stride > 0 && max_kv_len > 0,
+             "paged_attention_decode_static: bad window, table or length");
+  SA_REQUIRE(num_splits <= kMaxSplits, "paged_attention_decode_static: at most %d key ranges", kMaxSplits);
+  SA_REQUIRE(paged_attention_decode_takes(H, Kh, hd, page_size, max_q_len, q_stride, q),
+             "paged_attention_decode_static takes head size 64, 128 or 256, a page size that is a multiple of 16 and "
+             "(heads per key head) * tokens <= 16; got hd=%d P=%d G=%d tokens=%d", hd, page_size, H / Kh, max_q_len);
+  SA_REQUIRE(out_stride >= static_cast<int64_t>(H) * hd, "paged_attention_decode_static: output rows are too short");
+  return paged_attention_decode_static(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, seq_begin,
+                                       seq_count, out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len,
+                                       max_q_len, num_splits, stream);
+}
