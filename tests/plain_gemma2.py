@@ -7,6 +7,10 @@ operations on the CPU, in the dtype it is asked for (float32 or float64).
 
 Tensor names and layouts are those of the model folder: linear weights are
 `[out_features, in_features]`.
+
+Every part takes a `Rounding`: the places at which a run in a 16-bit activation type rounds its
+intermediate results, so that the arithmetic of such a run can be followed on the CPU, place by
+place, while everything between the places stays in the dtype asked for.  The default rounds nowhere.
 """
 from __future__ import annotations
 
@@ -17,18 +21,75 @@ import os
 import torch
 
 
+# --------------------------------------------------------------------------- rounding
+
+
+class Rounding:
+    """Rounds to `dtype` (and back) at the named places, nowhere else.
+
+    Places (what google-deepmind/simply rounds when `activation_dtype` is bfloat16):
+      embed_scale  the factor sqrt(dim) (simply/utils/module.py:476-480)
+      embed        the scaled embedding (same lines: the product is in the activation dtype)
+      norm_inner   x * rsqrt(var + eps) before the gain, and the gain `scale + 1` itself
+                   (simply/model_lib.py:166-173)
+      norm_out     the norm's result (simply/model_lib.py:174)
+      proj         results of the projections q, k, v, o, down (einsum in the activation dtype,
+                   simply/utils/module.py:339-343)
+      rope         rotated queries and keys, cast back from float32 (simply/utils/position_encoding.py:110);
+                   the scaled query (simply/kernels/ragged_paged_attention.py:217-224)
+      scores       q.k cast to the output dtype before the cap (simply/kernels/ragged_paged_attention.py:226-228;
+                   the dense path keeps float32 here, simply/model_lib.py:623-625)
+      probs        softmax cast to the values' dtype (simply/kernels/ragged_paged_attention.py:247;
+                   simply/model_lib.py:634)
+      attn_out     probs . v (simply/kernels/ragged_paged_attention.py:249)
+      ffn_parts    gate and up each, and the activated gate (simply/model_lib.py:714-727)
+      ffn_mid      act(gate) * up (simply/model_lib.py:727)
+      residual     y + h (simply/model_lib.py:2683, 2700: `x += x_res` in the activation dtype)
+      logits       the head's product and its soft-cap (simply/model_lib.py:3186-3188)
+    """
+
+    PLACES = ("embed_scale", "embed", "norm_inner", "norm_out", "proj", "rope", "scores", "probs", "attn_out",
+              "ffn_parts", "ffn_mid", "residual", "logits")
+
+    def __init__(self, dtype: torch.dtype | None = None, places=()):
+        unknown = set(places) - set(self.PLACES)
+        if unknown:
+            raise ValueError(f"unknown rounding places {sorted(unknown)}")
+        self.dtype, self.places = dtype, frozenset(places)
+
+    def __call__(self, place: str, x: torch.Tensor) -> torch.Tensor:
+        if self.dtype is None or place not in self.places:
+            return x
+        return x.to(self.dtype).to(x.dtype)
+
+
+NO_ROUNDING = Rounding()
+
+
+def rounding_like_simply(dtype=torch.bfloat16) -> Rounding:
+    """Every place at which google-deepmind/simply rounds in a 16-bit activation dtype (paged serving path)."""
+    return Rounding(dtype, Rounding.PLACES)
+
+
+def rounding_of_fp32_residual_engine(dtype=torch.bfloat16) -> Rounding:
+    """The places that are left when the residual stream, the norms' inner product, the scores and the logits are
+    kept in 32-bit and the gated product is rounded once: what an engine that holds 16-bit activations only between
+    its kernels does."""
+    return Rounding(dtype, ("embed_scale", "norm_out", "proj", "rope", "probs", "attn_out", "ffn_mid"))
+
+
 # --------------------------------------------------------------------------- parts
 
 
-def rms_norm(x: torch.Tensor, scale: torch.Tensor, eps: float) -> torch.Tensor:
+def rms_norm(x: torch.Tensor, scale: torch.Tensor, eps: float, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
     """RMSNorm with a `(1 + scale)` gain.
 
     simply/model_lib.py:154-178 (LayerNorm.apply with use_bias=False,
     scale_plus_one=True): var = mean(x^2); x *= rsqrt(var + eps); x *= scale + 1.
     """
     var = torch.mean(x * x, dim=-1, keepdim=True)
-    x = x * torch.rsqrt(var + eps)
-    return x * (scale + 1.0)
+    x = rnd("norm_inner", x * torch.rsqrt(var + eps))
+    return rnd("norm_out", x * rnd("norm_inner", scale + 1.0))
 
 
 def rope(x: torch.Tensor, positions: torch.Tensor, base: float) -> torch.Tensor:
@@ -42,8 +103,8 @@ def rope(x: torch.Tensor, positions: torch.Tensor, base: float) -> torch.Tensor:
     """
     hd = x.shape[-1]
     half = hd // 2
-    fraction = 2.0 * torch.arange(0, half, dtype=x.dtype) / hd
-    timescale = torch.as_tensor(base, dtype=x.dtype) ** fraction
+    fraction = 2.0 * torch.arange(0, half, dtype=x.dtype, device=x.device) / hd
+    timescale = torch.as_tensor(base, dtype=x.dtype, device=x.device) ** fraction
     angle = positions.to(x.dtype)[:, None, None] / timescale[None, None, :]
     sin, cos = torch.sin(angle), torch.cos(angle)
     x1, x2 = x[..., :half], x[..., half:]
@@ -76,7 +137,7 @@ def attention_mask(q_pos: torch.Tensor, k_pos: torch.Tensor, visible: int | None
     return mask
 
 
-def attention(q, k, v, mask, cap: float | None) -> torch.Tensor:
+def attention(q, k, v, mask, cap: float | None, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
     """Scores -> cap -> mask -> softmax -> weighted values.
 
     simply/model_lib.py:611-638 (attn): logits = q.k (no further scaling: the query
@@ -91,17 +152,17 @@ def attention(q, k, v, mask, cap: float | None) -> torch.Tensor:
     G = H // K
     k = k.repeat_interleave(G, dim=1)
     v = v.repeat_interleave(G, dim=1)
-    s = torch.einsum("thd,shd->hts", q, k)
+    s = rnd("scores", torch.einsum("thd,shd->hts", q, k))
     if cap is not None and cap > 0:
         s = soft_cap(s, cap)
     # simply/utils/common.py:543-551: mask value is -0.5 * float32 max.
     mask_value = -0.5 * torch.finfo(torch.float32).max
-    s = torch.where(mask[None, :, :], s, torch.as_tensor(mask_value, dtype=s.dtype))
-    p = torch.softmax(s, dim=-1)
-    return torch.einsum("hts,shd->thd", p, v)
+    s = torch.where(mask[None, :, :], s, torch.as_tensor(mask_value, dtype=s.dtype, device=s.device))
+    p = rnd("probs", torch.softmax(s, dim=-1))
+    return rnd("attn_out", torch.einsum("hts,shd->thd", p, v))
 
 
-def attention_layer(x, positions, w, prefix, cfg, visible) -> torch.Tensor:
+def attention_layer(x, positions, w, prefix, cfg, visible, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
     """q/k/v projections -> RoPE on q and k -> query scale -> attention -> o projection.
 
     simply/model_lib.py:2106-2110 (projections), :1987-2020 (_scale_qk: RoPE first,
@@ -111,30 +172,31 @@ def attention_layer(x, positions, w, prefix, cfg, visible) -> torch.Tensor:
     """
     T = x.shape[0]
     H, K, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-    q = (x @ w[prefix + "q_proj.weight"].T).reshape(T, H, hd)
-    k = (x @ w[prefix + "k_proj.weight"].T).reshape(T, K, hd)
-    v = (x @ w[prefix + "v_proj.weight"].T).reshape(T, K, hd)
+    q = rnd("proj", x @ w[prefix + "q_proj.weight"].T).reshape(T, H, hd)
+    k = rnd("proj", x @ w[prefix + "k_proj.weight"].T).reshape(T, K, hd)
+    v = rnd("proj", x @ w[prefix + "v_proj.weight"].T).reshape(T, K, hd)
     base = float(cfg.get("rope_theta", 10000.0))
-    q = rope(q, positions, base)
-    k = rope(k, positions, base)
-    q = q / math.sqrt(float(cfg.get("query_pre_attn_scalar", hd)))
+    q = rnd("rope", rope(q, positions, base))
+    k = rnd("rope", rope(k, positions, base))
+    q = rnd("rope", q / math.sqrt(float(cfg.get("query_pre_attn_scalar", hd))))
     mask = attention_mask(positions, positions, visible)
-    o = attention(q, k, v, mask, cfg.get("attn_logit_softcapping"))
-    return o.reshape(T, H * hd) @ w[prefix + "o_proj.weight"].T
+    o = attention(q, k, v, mask, cfg.get("attn_logit_softcapping"), rnd)
+    return rnd("proj", o.reshape(T, H * hd) @ w[prefix + "o_proj.weight"].T)
 
 
-def feed_forward(x, w, prefix) -> torch.Tensor:
+def feed_forward(x, w, prefix, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
     """Gated feed-forward: down(gelu(gate(x)) * up(x)).
 
     simply/model_lib.py:714-730: projected = ffn_0(x) (up), gate = ffn_0_gate(x),
     x = act(gate) * projected, out = ffn_1(x).
     """
-    gate = x @ w[prefix + "gate_proj.weight"].T
-    up = x @ w[prefix + "up_proj.weight"].T
-    return (gelu_tanh(gate) * up) @ w[prefix + "down_proj.weight"].T
+    gate = rnd("ffn_parts", x @ w[prefix + "gate_proj.weight"].T)
+    up = rnd("ffn_parts", x @ w[prefix + "up_proj.weight"].T)
+    mid = rnd("ffn_mid", rnd("ffn_parts", gelu_tanh(gate)) * up)
+    return rnd("proj", mid @ w[prefix + "down_proj.weight"].T)
 
 
-def block(x, positions, w, i, cfg, visible) -> torch.Tensor:
+def block(x, positions, w, i, cfg, visible, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
     """One decoder block with four norms.
 
     simply/model_lib.py:2669-2703: h = x; y = pre_ln_0(x); y = attn(y);
@@ -144,15 +206,15 @@ def block(x, positions, w, i, cfg, visible) -> torch.Tensor:
     p = f"model.layers.{i}."
     eps = float(cfg.get("rms_norm_eps", 1e-6))
     h = x
-    y = rms_norm(x, w[p + "input_layernorm.weight"], eps)
-    y = attention_layer(y, positions, w, p + "self_attn.", cfg, visible)
-    y = rms_norm(y, w[p + "post_attention_layernorm.weight"], eps)
-    x = y + h
+    y = rms_norm(x, w[p + "input_layernorm.weight"], eps, rnd)
+    y = attention_layer(y, positions, w, p + "self_attn.", cfg, visible, rnd)
+    y = rms_norm(y, w[p + "post_attention_layernorm.weight"], eps, rnd)
+    x = rnd("residual", y + h)
     h = x
-    y = rms_norm(x, w[p + "pre_feedforward_layernorm.weight"], eps)
-    y = feed_forward(y, w, p + "mlp.")
-    y = rms_norm(y, w[p + "post_feedforward_layernorm.weight"], eps)
-    return y + h
+    y = rms_norm(x, w[p + "pre_feedforward_layernorm.weight"], eps, rnd)
+    y = feed_forward(y, w, p + "mlp.", rnd)
+    y = rms_norm(y, w[p + "post_feedforward_layernorm.weight"], eps, rnd)
+    return rnd("residual", y + h)
 
 
 def layer_is_sliding(cfg: dict, i: int) -> bool:
@@ -164,36 +226,47 @@ def layer_is_sliding(cfg: dict, i: int) -> bool:
     return i % 2 == 0
 
 
-def embed(tokens, w, cfg) -> torch.Tensor:
-    """simply/utils/module.py:450-481: take(w, tokens) * sqrt(dim)."""
+def embed(tokens, w, cfg, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
+    """simply/utils/module.py:450-481: take(w, tokens) * sqrt(dim), the factor in the activation dtype."""
     table = w["model.embed_tokens.weight"]
-    return table[tokens] * math.sqrt(cfg["hidden_size"])
+    factor = rnd("embed_scale", torch.as_tensor(math.sqrt(cfg["hidden_size"]), dtype=table.dtype, device=table.device))
+    return rnd("embed", table[tokens] * factor)
 
 
-def lm_head(x, w, cfg) -> torch.Tensor:
+def lm_head(x, w, cfg, rnd: Rounding = NO_ROUNDING) -> torch.Tensor:
     """simply/model_lib.py:3184-3189: final norm, tied head ('vd,...d->...v' on the
     embedding table), then the final soft-cap if it is > 0."""
-    x = rms_norm(x, w["model.norm.weight"], float(cfg.get("rms_norm_eps", 1e-6)))
-    logits = x @ w["model.embed_tokens.weight"].T
+    x = rms_norm(x, w["model.norm.weight"], float(cfg.get("rms_norm_eps", 1e-6)), rnd)
+    logits = rnd("logits", x @ head_table(w, cfg).T)
     cap = cfg.get("final_logit_softcapping")
     if cap is not None and cap > 0:
-        logits = soft_cap(logits, cap)
+        logits = rnd("logits", soft_cap(logits, cap))
     return logits
+
+
+def head_table(w, cfg) -> torch.Tensor:
+    """The head's matrix: the embedding table when the two are tied (simply/utils/module.py:421-441,
+    use_tied_embedding), else a tensor of its own."""
+    if cfg.get("tie_word_embeddings", True):
+        return w["model.embed_tokens.weight"]
+    return w["lm_head.weight"]
 
 
 # --------------------------------------------------------------------------- model
 
 
-def forward(w: dict, cfg: dict, tokens, dtype=torch.float32, first_position: int = 0) -> torch.Tensor:
-    """Logits [T, V] at every position of one whole sequence (simply/model_lib.py:2935-3189)."""
-    tokens = torch.as_tensor(tokens, dtype=torch.long)
-    w = {k: v.to(dtype) for k, v in w.items()}
-    positions = torch.arange(first_position, first_position + tokens.numel())
-    x = embed(tokens, w, cfg)
+def forward(w: dict, cfg: dict, tokens, dtype=torch.float32, first_position: int = 0,
+            rnd: Rounding = NO_ROUNDING, device=None) -> torch.Tensor:
+    """Logits [T, V] at every position of one whole sequence (simply/model_lib.py:2935-3189).  `device`: where
+    torch computes it (the CPU unless a long sequence at large sizes wants a faster place)."""
+    tokens = torch.as_tensor(tokens, dtype=torch.long, device=device)
+    w = {k: v.to(device=device, dtype=dtype) for k, v in w.items()}
+    positions = torch.arange(first_position, first_position + tokens.numel(), device=device)
+    x = embed(tokens, w, cfg, rnd)
     for i in range(cfg["num_hidden_layers"]):
         visible = cfg.get("sliding_window") if layer_is_sliding(cfg, i) else None
-        x = block(x, positions, w, i, cfg, visible)
-    return lm_head(x, w, cfg)
+        x = block(x, positions, w, i, cfg, visible, rnd)
+    return lm_head(x, w, cfg, rnd)
 
 
 def load(model_dir: str):

@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 import torch
 
+import bounds
 import plain_gemma2 as plain
 import tiny
 from simply_amd.config import EngineConfig
@@ -11,9 +12,6 @@ from simply_amd.engine import Executor, StepEntry
 from simply_amd.engine.loading import load_model
 
 pytestmark = pytest.mark.gpu
-
-# largest difference of logits, as a fraction of the largest logit of the plain implementation
-TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 
 
 @pytest.fixture(autouse=True)
@@ -42,28 +40,16 @@ def run_cut(ex, rid, tokens, cuts):
     return torch.cat(out)
 
 
-def plain_logits(model_dir, tokens, dtype):
-    """The plain implementation in float64 on the weights as the engine holds them."""
-    w, cfg = plain.load(model_dir)
-    if dtype == "bfloat16":
-        w = {k: v.to(torch.bfloat16) for k, v in w.items()}
-    return plain.forward(w, cfg, tokens, torch.float64), cfg
-
-
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_cuts_match_plain(tmp_path, name, dtype):
     d = tiny.write_model(name, str(tmp_path / name), std=0.3)
     vocab = plain.load(d)[1]["vocab_size"]
     tokens = tiny.random_tokens(77, vocab, 7)
-    want, cfg = plain_logits(d, tokens, dtype)
-    scale = want.abs().max().item()
+    ref = bounds.reference_of(d, tokens, dtype)
     ex = make_executor(d, dtype)
     for cuts in ([77], [45] + [1] * 32, [7, 5, 3, 2, 11, 2, 2, 13, 17, 2, 13], [1] * 77):
-        got = run_cut(ex, "r", tokens, cuts).double()
-        assert torch.isfinite(got).all()
-        err = (got - want).abs().max().item() / scale
-        assert err <= TOL[dtype], (cuts, err)
+        ref.check(run_cut(ex, "r", tokens, cuts), what=cuts)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -72,14 +58,10 @@ def test_cuts_match_plain_at_kernel_sizes(tmp_path, dtype):
     d = tiny.write_model("D", str(tmp_path / "D"), std=0.15)
     vocab = plain.load(d)[1]["vocab_size"]
     tokens = tiny.random_tokens(150, vocab, 8)
-    want, cfg = plain_logits(d, tokens, dtype)
-    scale = want.abs().max().item()
+    ref = bounds.reference_of(d, tokens, dtype)
     ex = make_executor(d, dtype, page_size=16, num_pages=24, max_len=320)
     for cuts in ([150], [118] + [1] * 32, [40, 7, 5, 3, 2, 30, 2, 2, 13, 17, 2, 27], [1] * 150, [3, 4, 2] * 16 + [6]):
-        got = run_cut(ex, "r", tokens, cuts).double()
-        assert torch.isfinite(got).all()
-        err = (got - want).abs().max().item() / scale
-        assert err <= TOL[dtype], (cuts, err)
+        ref.check(run_cut(ex, "r", tokens, cuts), what=cuts)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -114,31 +96,23 @@ def test_graph_replays_match_eager(tmp_path, dtype):
         outs[graphs] = {r: torch.cat(v) for r, v in got.items()}
     for r in reqs:
         assert torch.equal(outs[False][r], outs[True][r]), r
-    w, cfg_ = plain.load(d)
     for r, t in reqs.items():
-        want = plain_logits(d, t, dtype)[0][19:]
-        err = (outs[True][r].double() - want).abs().max().item() / want.abs().max().item()
-        assert err <= TOL[dtype], (r, err)
+        bounds.reference_of(d, t, dtype).check(outs[True][r], rows=slice(19, None), what=r)
 
 
-@pytest.mark.parametrize("seed", range(100, 112))
-def test_random_configurations_mixed(tmp_path, seed):
-    """Configurations drawn at random (tiny.random_config), each with up to four live requests cut at random into
-    portions and single tokens, in a pool that is smaller than what all requests hold: in 32-bit against the plain
-    implementation; in bfloat16 against the plain implementation and against the same requests run whole and
-    alone, where only the rounding of other kernels may differ."""
-    d = tiny.write_random_config_model(seed, str(tmp_path / "m"))
-    w0, pcfg = plain.load(d)
+def mixed_requests_in_a_tight_pool(model_dir, page, lens, seed):
+    """Up to four live requests cut at random into portions and single tokens, in a pool that is smaller than what
+    all requests hold: in 32-bit against the plain implementation; in bfloat16 against the plain implementation
+    (within the bound derived for the model, `bounds`) and against the same requests run whole and alone, where only
+    the rounding of other kernels may differ."""
+    w0, pcfg = plain.load(model_dir)
     rng = np.random.default_rng(seed)
-    page = int(rng.choice([4, 8, 16, 16, 32]))
-    lens = [int(rng.integers(2, 130)) for _ in range(int(rng.integers(3, 6)))]
     reqs = {f"r{i}": tiny.random_tokens(n, pcfg["vocab_size"], seed * 100 + i) for i, n in enumerate(lens)}
     pages_of = lambda n: -(-n // page) + 1
     num_pages = max(pages_of(max(lens)) + 2, int(sum(pages_of(n) for n in lens) * 0.6))
     for dtype in ("float32", "bfloat16"):
-        w = w0 if dtype == "float32" else {k: v.to(torch.bfloat16) for k, v in w0.items()}
-        want = {r: plain.forward(w, pcfg, t, torch.float64) for r, t in reqs.items()}
-        ex = make_executor(d, dtype, page_size=page, num_pages=num_pages)
+        refs = {r: bounds.reference(w0, pcfg, t, dtype) for r, t in reqs.items()}
+        ex = make_executor(model_dir, dtype, page_size=page, num_pages=num_pages)
         pending, live, got = list(reqs), {}, {r: {} for r in reqs}
         while pending or live:
             while pending and len(live) < 4:
@@ -172,11 +146,33 @@ def test_random_configurations_mixed(tmp_path, seed):
             if not at:
                 continue
             g = torch.stack([got[r][p] for p in at]).double()
-            scale = want[r].abs().max().item()
-            assert torch.isfinite(g).all()
-            assert (g - want[r][at]).abs().max().item() / scale <= TOL[dtype], (dtype, r)
+            refs[r].check(g, rows=at, what=(dtype, r))
             if dtype == "bfloat16":
+                # cut and mixed against whole and alone: the same arithmetic but for the kernels that few rows and
+                # many rows go through; bounded by the same rounded run
                 ex.add_request(r)
                 whole = ex.step([StepEntry(r, t, list(range(len(t))))]).cpu().double()
                 ex.finish_request(r)
-                assert (g - whole[at]).abs().max().item() / scale <= 1e-2, (dtype, r)
+                refs[r].check(whole, what=(dtype, r, "whole"))
+                assert (g - whole[at]).abs().max().item() / refs[r].scale <= refs[r].max_bound(), (dtype, r)
+
+
+@pytest.mark.parametrize("seed", range(100, 112))
+def test_random_configurations_mixed(tmp_path, seed):
+    """Configurations drawn at random (tiny.random_config): head counts and sizes, widths that are no multiple of 8,
+    layer kinds in any order."""
+    d = tiny.write_random_config_model(seed, str(tmp_path / "m"))
+    rng = np.random.default_rng(seed)
+    page = int(rng.choice([4, 8, 16, 16, 32]))
+    lens = [int(rng.integers(2, 130)) for _ in range(int(rng.integers(3, 6)))]
+    mixed_requests_in_a_tight_pool(d, page, lens, seed)
+
+
+@pytest.mark.parametrize("case", [4, 11, 21, 36, 94, 135, "smallest"])
+def test_configurations_with_the_largest_bfloat16_error(tmp_path, case):
+    """The configurations on which bfloat16 logits lie furthest from the float64 ones (tiny.drawn_case): 4 to 9 % of
+    the largest logit, where the usual configuration gives 0.3 to 1 %.  The plain implementation with rounding at the
+    same places is as far off (tests/test_plain.py shows on the CPU where the error enters), so the bound that is
+    derived from it holds here as everywhere."""
+    d, page, lens = tiny.write_drawn_case(case, str(tmp_path / "m"))
+    mixed_requests_in_a_tight_pool(d, page, lens, 7 if case == "smallest" else case)

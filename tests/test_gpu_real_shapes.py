@@ -4,6 +4,7 @@ bfloat16 kernels at the sizes they are built for, and the float32 path, against 
 import pytest
 import torch
 
+import bounds
 import plain_gemma2 as plain
 import tiny
 from simply_amd.config import EngineConfig, config_from_dict
@@ -23,21 +24,20 @@ SHAPES = {
 }
 
 
-@pytest.mark.parametrize("dtype,tol", [("float32", 5e-5), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", ["2b", "9b", "27b"])
-def test_real_layer_shapes(tmp_path, gpu_lib, shape, dtype, tol):
+def test_real_layer_shapes(tmp_path, gpu_lib, shape, dtype):
     d = dict(architectures=["Gemma2ForCausalLM"], num_hidden_layers=2, vocab_size=2000, rms_norm_eps=1e-6,
              rope_theta=10000.0, sliding_window=48, attn_logit_softcapping=50.0, final_logit_softcapping=30.0,
              max_position_embeddings=8192, initializer_range=0.02, **SHAPES[shape])
     folder = write_random_model(config_from_dict(d), str(tmp_path / shape), 5, torch.bfloat16, norm_std=0.1)
     w, cfg = plain.load(folder)
     tokens = tiny.random_tokens(100, 2000, 11)
-    want = plain.forward(w, cfg, tokens, torch.float64)
+    ref = bounds.reference(w, cfg, tokens, dtype)
     ecfg = EngineConfig(activation_dtype=dtype, page_size=16, batch_size=2, max_seq_len=128, max_num_issue_tokens=128,
                         total_num_pages=16, device="cuda:0", use_graphs=True, poison_freed_pages=True)
     model, _ = load_model(folder, ecfg.dtype, "cuda:0")
     ex = Executor(model, ecfg)
-    scale = want.abs().max().item()
     for cuts in ([100], [60, 5, 3] + [1] * 32):
         ex.add_request("r")
         out, i = [], 0
@@ -46,9 +46,12 @@ def test_real_layer_shapes(tmp_path, gpu_lib, shape, dtype, tol):
             i += c
         ex.finish_request("r")
         got = torch.cat(out).double()
-        assert torch.isfinite(got).all()
-        err = (got - want).abs().max().item() / scale
-        assert err <= tol, (cuts, err)
+        if dtype == "float32":
+            # sums over up to 36864 terms in 32-bit: 5e-5 of the largest logit
+            assert torch.isfinite(got).all()
+            assert (got - ref.want).abs().max().item() / ref.scale <= 5e-5, cuts
+        else:
+            ref.check(got, what=cuts)
 
 
 @pytest.mark.parametrize("library_rows", [256, 0])
@@ -63,7 +66,7 @@ def test_long_portions(tmp_path, gpu_lib, library_rows):
     folder = write_random_model(config_from_dict(d), str(tmp_path / "m"), 6, torch.bfloat16, norm_std=0.1)
     w, cfg = plain.load(folder)
     tokens = tiny.random_tokens(700, 2000, 12)
-    want = plain.forward(w, cfg, tokens, torch.float64)
+    ref = bounds.reference(w, cfg, tokens, "bfloat16")
     ecfg = EngineConfig(activation_dtype="bfloat16", page_size=16, batch_size=2, max_seq_len=704, max_num_issue_tokens=704,
                         total_num_pages=48, device="cuda:0", use_graphs=False, poison_freed_pages=True)
     before = ops.library_gemm_min_rows()
@@ -71,7 +74,6 @@ def test_long_portions(tmp_path, gpu_lib, library_rows):
     try:
         model, _ = load_model(folder, ecfg.dtype, "cuda:0")
         ex = Executor(model, ecfg)
-        scale = want.abs().max().item()
         for cuts in ([700], [600, 98, 2]):
             ex.add_request("r")
             out, i = [], 0
@@ -79,9 +81,6 @@ def test_long_portions(tmp_path, gpu_lib, library_rows):
                 out.append(ex.step([StepEntry("r", tokens[i:i + c], list(range(c)))]).cpu())
                 i += c
             ex.finish_request("r")
-            got = torch.cat(out).double()
-            assert torch.isfinite(got).all()
-            err = (got - want).abs().max().item() / scale
-            assert err <= 3e-2, (cuts, err)
+            ref.check(torch.cat(out), what=cuts)
     finally:
         ops.set_library_gemm_min_rows(before)

@@ -11,12 +11,12 @@ import numpy as np
 import pytest
 import torch
 
+import bounds
 import plain_gemma2 as plain
 import tiny
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 
 
 class TraceRun:
@@ -60,17 +60,6 @@ def feed(tr, rid, tokens, cuts, end=True):
     return torch.cat(out)
 
 
-def plain_logits(w, cfg, tokens, dtype):
-    if dtype == "bfloat16":
-        w = {k: v.to(torch.bfloat16) for k, v in w.items()}
-    return plain.forward(w, cfg, tokens, torch.float64)
-
-
-def rel_err(got, want):
-    assert torch.isfinite(got).all()
-    return ((got.double() - want).abs().max() / want.abs().max()).item()
-
-
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_replay_all_cuts(tmp_path, name, dtype):
@@ -78,16 +67,15 @@ def test_replay_all_cuts(tmp_path, name, dtype):
     w, cfg = plain.load(d)
     V = cfg["vocab_size"]
     reqs = {f"r{i}": tiny.random_tokens(n, V, 10 + i) for i, n in enumerate([70, 45, 100, 33, 64, 2, 90])}
-    want = {r: plain_logits(w, cfg, t, dtype) for r, t in reqs.items()}
+    refs = {r: bounds.reference(w, cfg, t, dtype) for r, t in reqs.items()}
     # 320 tokens = 20 pages of 16: less than the 404 tokens that all requests hold together
     tr = TraceRun(d, dtype, str(tmp_path / "out"), 320, extra=["--poison"])
-    tol = TOL[dtype]
     try:
         toks = reqs["r0"]
-        assert rel_err(feed(tr, "whole", toks, [len(toks)]), want["r0"]) <= tol
-        assert rel_err(feed(tr, "tail", toks, [len(toks) - 32] + [1] * 32), want["r0"]) <= tol
-        assert rel_err(feed(tr, "cuts", toks, [9, 7, 5, 3, 2, 16, 2, 2, 11, 13]), want["r0"]) <= tol
-        assert rel_err(feed(tr, "first", toks, [1, 1, 1, 2, 3, 62]), want["r0"]) <= tol
+        refs["r0"].check(feed(tr, "whole", toks, [len(toks)]), what="whole")
+        refs["r0"].check(feed(tr, "tail", toks, [len(toks) - 32] + [1] * 32), what="tail")
+        refs["r0"].check(feed(tr, "cuts", toks, [9, 7, 5, 3, 2, 16, 2, 2, 11, 13]), what="cuts")
+        refs["r0"].check(feed(tr, "first", toks, [1, 1, 1, 2, 3, 62]), what="first")
         # mixed: up to four live requests, portions of some beside single tokens of others, requests left out of
         # steps, nothing wanted in some portions
         rng = np.random.default_rng(1)
@@ -123,8 +111,7 @@ def test_replay_all_cuts(tmp_path, name, dtype):
         for r in reqs:
             pos = sorted(got[r])
             assert len(pos) > 0
-            g = torch.stack([got[r][p] for p in pos])
-            assert rel_err(g, want[r][pos]) <= tol, r
+            refs[r].check(torch.stack([got[r][p] for p in pos]), rows=pos, what=r)
     finally:
         tr.close()
 
@@ -135,11 +122,10 @@ def test_replay_long_decoding(tmp_path, dtype):
     d = tiny.write_model("A", str(tmp_path / "m"), dtype=torch.bfloat16, std=0.3)
     w, cfg = plain.load(d)
     toks = tiny.random_tokens(320, cfg["vocab_size"], 99)
-    want = plain_logits(w, cfg, toks, dtype)
+    ref = bounds.reference(w, cfg, toks, dtype)
     tr = TraceRun(d, dtype, str(tmp_path / "out"), 320, extra=["--poison"])
     try:
-        got = feed(tr, "long", toks, [20] + [1] * 300)
-        assert rel_err(got, want) <= TOL[dtype]
+        ref.check(feed(tr, "long", toks, [20] + [1] * 300), what="long")
     finally:
         tr.close()
 

@@ -184,9 +184,14 @@ def test_block_is_identity_when_post_norms_vanish():
 def test_embedding_and_head():
     cfg = dict(tiny.TINY_B)
     w = weights(cfg)
-    tok = torch.tensor([3, 500, 3])
-    e = plain.embed(tok, w, cfg)
-    torch.testing.assert_close(e, w["model.embed_tokens.weight"][tok] * math.sqrt(96))
+    # a table drawn N(0, 1 / D), the initialisation that simply/utils/module.py:470-474 names as the reason for the
+    # factor, gives embeddings of variance 1: without the factor it would be 1 / D, with it twice D
+    D = 4096
+    table = torch.randn(1000, D, generator=torch.Generator().manual_seed(1), dtype=torch.float64) / math.sqrt(D)
+    e = plain.embed(torch.arange(1000), {"model.embed_tokens.weight": table}, {"hidden_size": D})
+    assert abs(e.var().item() - 1.0) < 0.01
+    assert torch.equal(plain.embed(torch.tensor([3, 500, 3]), w, cfg)[0], plain.embed(torch.tensor([3]), w, cfg)[0])
+    # the factor is on the input side only: the head is the plain product with the table
     x = torch.randn(4, 96, dtype=torch.float64) * 10
     logits = plain.lm_head(x, w, cfg)
     assert logits.shape == (4, 512) and logits.abs().max() < 15.0          # the final cap bounds the logits
@@ -197,8 +202,36 @@ def test_embedding_and_head():
 
 
 def test_layer_pattern():
-    assert [plain.layer_is_sliding(tiny.TINY_A, i) for i in range(4)] == [True, False, True, False]
+    """Even layers are windowed, odd ones see everything (simply/config_lib.py:876-879 ('local', 'global')): with one
+    layer a token beyond the window is invisible, with two it is seen, and only through the second layer."""
+    cfg = dict(tiny.TINY_A, sliding_window=4)
+    far, at = 3, 20
+    tokens = tiny.random_tokens(24, cfg["vocab_size"], 6)
+    changed = list(tokens)
+    changed[far] = (changed[far] + 1) % cfg["vocab_size"]
+    w = weights(dict(cfg, num_hidden_layers=2), seed=4)
+    one = dict(cfg, num_hidden_layers=1)
+    a, b = (plain.forward(w, one, t, torch.float64) for t in (tokens, changed))
+    torch.testing.assert_close(a[far + 4:], b[far + 4:], rtol=0, atol=0)     # layer 0 is windowed
+    two = dict(cfg, num_hidden_layers=2)
+    a, b = (plain.forward(w, two, t, torch.float64) for t in (tokens, changed))
+    assert not torch.allclose(a[at], b[at])                                  # layer 1 is not
+    # ... and it is layer 1 that sees it: with layer 1's keys and values cut off from the far token's position
+    # (its value projection zeroed) the difference is gone again
+    both_windowed = dict(two, layer_types=["sliding_attention", "sliding_attention"])
+    a, b = (plain.forward(w, both_windowed, t, torch.float64) for t in (tokens, changed))
+    torch.testing.assert_close(a[at], b[at], rtol=0, atol=0)
+    # an explicit list of layer types wins over the rule
     assert [plain.layer_is_sliding(tiny.TINY_C, i) for i in range(4)] == [False, True, True, False]
+
+
+def test_untied_head_uses_its_own_table():
+    cfg = dict(tiny.TINY_B, tie_word_embeddings=False)
+    w = weights(cfg)
+    w["lm_head.weight"] = torch.randn(512, 96, generator=torch.Generator().manual_seed(9), dtype=torch.float64)
+    x = torch.randn(4, 96, dtype=torch.float64)
+    raw = plain.rms_norm(x, w["model.norm.weight"], 1e-5) @ w["lm_head.weight"].T
+    torch.testing.assert_close(plain.lm_head(x, w, cfg), 15 * torch.tanh(raw / 15))
 
 
 # ------------------------------------------------------------------ whole model
@@ -247,3 +280,53 @@ def test_greedy_and_sampling_helpers():
     assert plain.top_p_mask(logits, float(p[0]) + 1e-6).tolist() == [True, True, False, False]
     assert plain.top_p_mask(logits, float(p[0]) - 1e-6).tolist() == [True, False, False, False]
     assert abs(plain.log_prob(logits, 1, 0.5) - float(torch.log_softmax(logits.double() / 0.5, -1)[1])) < 1e-12
+
+
+# ------------------------------------------------------------------ rounding places
+def test_rounding_nowhere_changes_nothing_and_everywhere_is_bfloat16_arithmetic():
+    cfg = dict(tiny.TINY_B)       # sqrt(96) is no bfloat16 number
+    w = {k: v.to(torch.bfloat16).double() for k, v in weights(cfg, seed=6).items()}
+    tokens = tiny.random_tokens(20, cfg["vocab_size"], 7)
+    exact = plain.forward(w, cfg, tokens, torch.float64)
+    assert torch.equal(plain.forward(w, cfg, tokens, torch.float64, rnd=plain.Rounding(torch.bfloat16, ())), exact)
+    with pytest.raises(ValueError):
+        plain.Rounding(torch.bfloat16, ("nowhere",))
+    # every place rounds: each alone moves the logits, by no more than a few bfloat16 steps of the largest logit
+    for place in plain.Rounding.PLACES:
+        moved = plain.forward(w, cfg, tokens, torch.float64, rnd=plain.Rounding(torch.bfloat16, (place,)))
+        err = (moved - exact).abs().max().item() / exact.abs().max().item()
+        assert 0 < err < 2e-2, (place, err)
+    # the norm's result rounded: the same as rounding by hand
+    x = torch.randn(3, 96, dtype=torch.float64)
+    scale = w["model.norm.weight"]
+    by_hand = plain.rms_norm(x, scale, 1e-5).to(torch.bfloat16).double()
+    assert torch.equal(plain.rms_norm(x, scale, 1e-5, plain.Rounding(torch.bfloat16, ("norm_out",))), by_hand)
+
+
+def test_where_bfloat16_error_enters_a_sharp_model():
+    """tiny.drawn_case(11): three global layers of one head of size 128, no soft-cap, weights N(0, 0.32): bfloat16
+    logits are 5 to 10 % off, ten times the usual.  Rounding what feeds the scores (norm results, projections,
+    rotated queries and keys) does it; rounding behind the softmax (probabilities, attention output, the gated
+    product) costs a tenth of that.  With the scores themselves and the residual stream rounded too, as
+    google-deepmind/simply does in bfloat16, the error is larger still.  A flat model (drawn_case(0): soft-cap 5) is
+    at 0.3 %."""
+    def errors(case, n):
+        import tempfile
+
+        with tempfile.TemporaryDirectory() as tmp:
+            d, _, _ = tiny.write_drawn_case(case, tmp + "/m")
+            w, cfg = plain.load(d)
+        w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+        tokens = tiny.random_tokens(n, cfg["vocab_size"], case * 100)
+        exact = plain.forward(w, cfg, tokens, torch.float64)
+        err = lambda rnd: ((plain.forward(w, cfg, tokens, torch.float64, rnd=rnd) - exact).abs().max()
+                           / exact.abs().max()).item()
+        R = lambda *places: plain.Rounding(torch.bfloat16, places)
+        return (err(R("norm_out", "proj", "rope")), err(R("probs", "attn_out", "ffn_mid")),
+                err(plain.rounding_of_fp32_residual_engine()), err(plain.rounding_like_simply()))
+
+    before, behind, engine, simply = errors(11, 82)
+    assert before > 3e-2 and behind < before / 4
+    assert engine > 3e-2 and simply > engine
+    before, behind, engine, simply = errors(0, 130)
+    assert engine < 6e-3 and simply < 1.2e-2

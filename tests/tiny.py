@@ -88,3 +88,60 @@ def write_random_config_model(seed: int, out_dir: str) -> str:
     d = random_config(seed)
     std = 0.15 * (64.0 / d["hidden_size"]) ** 0.5
     return write_random_model(config_from_dict(d), out_dir, seed, torch.float32, std=std, norm_std=0.2)
+
+
+def drawn_case(case: int) -> tuple[dict, int, float, list[int]]:
+    """Another family of configurations drawn at random, with larger weights: (config, page size, std of the
+    weights, lengths of the requests).  Cases 4, 11, 21, 36, 94 and 135 are the ones whose bfloat16 logits lie
+    furthest from the float64 ones (4 to 8 % of the largest logit: sharp softmaxes without a soft-cap, or four
+    layers of head size 256 over a width of 136)."""
+    import numpy as np
+
+    rng = np.random.default_rng(case)
+    kv, group = int(rng.choice([1, 2, 3, 4])), int(rng.choice([1, 2, 3, 4, 8]))
+    hd = int(rng.choice([16, 32, 48, 64, 80, 96, 128, 256]))
+    if hd >= 128:
+        kv, group = min(kv, 2), min(group, 2)
+    hidden = int(rng.choice([64, 96, 120, 128, 136, 200, 100, 264]))
+    inter = int(rng.choice([128, 200, 320, 264, 72, 500]))
+    layers = int(rng.integers(1, 5))
+    vocab = int(rng.choice([256, 333, 512, 1000, 1001, 4099]))
+    window = int(rng.integers(3, 60))
+    types = [str(rng.choice(["full_attention", "sliding_attention"])) for _ in range(layers)]
+    d = dict(
+        architectures=["Gemma2ForCausalLM"], hidden_size=hidden, num_hidden_layers=layers,
+        num_attention_heads=kv * group, num_key_value_heads=kv, head_dim=hd, intermediate_size=inter, vocab_size=vocab,
+        rms_norm_eps=float(rng.choice([1e-6, 1e-5])), rope_theta=float(rng.choice([10000.0, 1e6, 500.0])),
+        sliding_window=window, query_pre_attn_scalar=int(rng.choice([hd, 24, 144])),
+        attn_logit_softcapping=None if rng.random() < 0.3 else float(rng.choice([50.0, 20.0, 5.0])),
+        final_logit_softcapping=None if rng.random() < 0.3 else float(rng.choice([30.0, 15.0])),
+        tie_word_embeddings=True, max_position_embeddings=1024, layer_types=types,
+        hidden_activation="gelu_pytorch_tanh", initializer_range=0.05)
+    page = int(rng.choice([4, 8, 16, 16, 32]))
+    std = float(rng.choice([0.1, 0.2, 0.3])) * (64.0 / hidden) ** 0.5 * 1.5
+    lens = [int(rng.integers(2, 160)) for _ in range(int(rng.integers(3, 7)))]
+    return d, page, std, lens
+
+
+# the smallest sizes anything takes, a window of one key: its bfloat16 logits were 8.7 % off on a 130-token request
+SMALLEST = dict(
+    architectures=["Gemma2ForCausalLM"], hidden_size=8, num_hidden_layers=3, num_attention_heads=1,
+    num_key_value_heads=1, head_dim=16, intermediate_size=24, vocab_size=17, rms_norm_eps=1e-6, rope_theta=10000.0,
+    sliding_window=1, query_pre_attn_scalar=16, attn_logit_softcapping=50.0, final_logit_softcapping=30.0,
+    tie_word_embeddings=True, max_position_embeddings=1024,
+    layer_types=["full_attention", "sliding_attention", "full_attention"], hidden_activation="gelu_pytorch_tanh",
+    initializer_range=0.05)
+
+
+def write_drawn_case(case, out_dir: str) -> tuple[str, int, list[int]]:
+    """Writes `drawn_case(case)` (or, for case "smallest", SMALLEST) as a model folder; returns (folder, page size,
+    request lengths)."""
+    from simply_amd.config import config_from_dict
+    from simply_amd.weights import write_random_model
+
+    if case == "smallest":
+        d, page, std, lens, seed = SMALLEST, 4, 0.3 * (64.0 / 8) ** 0.5 * 1.5, [19, 49, 67, 130], 2
+    else:
+        d, page, std, lens = drawn_case(case)
+        seed = case
+    return write_random_model(config_from_dict(d), out_dir, seed, torch.float32, std=std, norm_std=0.2), page, lens
