@@ -41,7 +41,8 @@ class Executor:
             pages = config.batch_size * -(-config.max_seq_len // config.page_size)
         self.cache = CacheManager(model.cache_needs(), page_size=config.page_size, num_pages=pages,
                                   num_slots=config.batch_size, max_seq_len=config.max_seq_len, dtype=self.dtype,
-                                  device=self.device, poison=config.poison_freed_pages)
+                                  device=self.device, poison=config.poison_freed_pages,
+                                  max_step_tokens=max(config.issue_budget, config.batch_size))
         self.num_computed: dict[Hashable, tuple[int, int]] = {}  # request -> (admission, tokens run)
         self.vocab_size = model.spec.vocab_size
         # one pinned staging buffer and one device buffer for all of a step's integers
@@ -56,8 +57,10 @@ class Executor:
         self._copied = torch.cuda.Event() if self._on_gpu else None
         # decode-only steps (one token per request) are captured once per number of requests and order of magnitude
         # of the context (the attention kernels choose their cut of the keys when they are recorded) and replayed
-        self._graphs: dict[tuple, tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
         self._graph_pool = None
+        # where every recorded step writes its logits, [batch_size, vocab] float32: made at the first such step
+        self._graph_logits: torch.Tensor | None = None
         # several decode steps in a row without the host (decode_many): what was drawn in each, and the step count
         self._records: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None
 
@@ -86,24 +89,37 @@ class Executor:
     def _replay(self, T: int, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
         """A decode-only step through a captured HIP graph.  Everything that differs between two such steps
         with the same number of requests (tokens, positions, slots, block tables) lies in buffers at fixed
-        addresses that the kernels read, so the launches can be recorded once.  The returned logits are
-        overwritten by the next replay with as many requests."""
+        addresses that the kernels read, so the launches can be recorded once.  The returned logits lie in a buffer
+        that all recorded steps share: the next decode-only step overwrites them.  A step runs exactly once: the
+        first step with a new key runs eagerly (kernels choose their plans, scratch buffers get allocated) and is
+        this call's result; the recording that follows executes nothing (a mixer that keeps a state of its own would
+        otherwise advance it twice)."""
         key = (T, self._context_bucket(ctx))
-        entry = self._graphs.get(key)
-        if entry is None:
-            # once eagerly (kernels compile their plans, scratch buffers get allocated; the step's writes to the
-            # cache are the same when repeated), then record
-            self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
-            torch.cuda.synchronize(self.device)
-            graph = torch.cuda.CUDAGraph()
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits = self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
-            entry = (graph, logits)
-            self._graphs[key] = entry
-        entry[0].replay()
-        return entry[1]
+        out = self._shared_logits()[:T]
+        graph = self._graphs.get(key)
+        if graph is not None:
+            graph.replay()
+            return out
+        logits = self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows, logits_out=out)
+        self._graphs[key] = self._record(
+            lambda: self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows, logits_out=out))
+        return logits
+
+    def _shared_logits(self) -> torch.Tensor:
+        if self._graph_logits is None:
+            self._graph_logits = torch.empty((self.config.batch_size, self.vocab_size), dtype=torch.float32,
+                                             device=self.device)
+        return self._graph_logits
+
+    def _record(self, run) -> "torch.cuda.CUDAGraph":
+        """Records the launches of `run()` in a HIP graph, executing none of them."""
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            run()
+        return graph
 
     @staticmethod
     def _context_bucket(ctx: StepContext) -> int:
@@ -125,6 +141,7 @@ class Executor:
             logits = self.model.forward(self._dev[:T], ctx, self.cache.views, logit_rows)
         for rid, start, q in wants:
             self.num_computed[rid] = (self.cache.admission[rid], start + q)
+        self.cache.mark_issued(wants)
         return logits
 
     def decode_many(self, entries: Sequence[StepEntry], num_steps: int, sampler) -> tuple[list[list[int]], list[list[float]]]:
@@ -164,8 +181,10 @@ class Executor:
         out_tok, out_lp = rec_tok[:max_steps * B].view(max_steps, B), rec_lp[:max_steps * B].view(max_steps, B)
         from ..kernels import ops
 
+        shared = self._shared_logits()[:T]
+
         def one_step():
-            logits = self.model.forward(dev[:T], ctx, self.cache.views, logit_rows)
+            logits = self.model.forward(dev[:T], ctx, self.cache.views, logit_rows, logits_out=shared)
             toks, lps = sampler.launch(logits)
             ops.decode_advance(counter, toks, lps, dev[:T], dev[cap:cap + T], ctx.seq_meta, sampler.draw_counters,
                                out_tok, out_lp)
@@ -175,25 +194,19 @@ class Executor:
 
         ops.fill_(counter, 0)
         key = ("many", B, self._context_bucket(ctx), max_steps, id(sampler), sampler.modes)
-        entry = self._graphs.get(key)
+        graph = self._graphs.get(key)
         done = 0
-        if entry is None:
+        if graph is None:
             one_step()   # once eagerly (it counts as the first step), then recorded
             done = 1
-            torch.cuda.synchronize(self.device)
-            graph = torch.cuda.CUDAGraph()
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                one_step()
-            entry = (graph, None)
-            self._graphs[key] = entry
+            graph = self._graphs[key] = self._record(one_step)
         for _ in range(done, num_steps):
-            entry[0].replay()
+            graph.replay()
         tokens = out_tok[:num_steps].tolist()      # waits for the steps
         logprobs = out_lp[:num_steps].tolist()
         for rid, start, _ in wants:
             self.num_computed[rid] = (self.cache.admission[rid], start + num_steps)
+        self.cache.mark_issued([(rid, start, num_steps) for rid, start, _ in wants])
         return tokens, logprobs
 
     def _prepare(self, entries: Sequence[StepEntry], reserve_ahead: int = 1):
@@ -225,13 +238,7 @@ class Executor:
             raise ValueError(f"{len(entries)} requests in one step, batch_size is {self.config.batch_size}")
         # make room for every entry first: nothing is reserved unless all of it fits
         wants = [(e.request_id, self._start_of(e), max(len(e.tokens), reserve_ahead)) for e in entries]
-        if not cache.can_reserve(wants):
-            from ..cache import OutOfPages
-
-            raise OutOfPages("the cache cannot hold this step's tokens: " + ", ".join(
-                f"{rid!r}+{q}" for rid, _, q in wants))
-        for rid, start, q in wants:
-            cache.reserve(rid, start, q, fits=True)
+        cache.reserve_all(wants)
 
         if self._copied is not None:
             self._copied.synchronize()  # the last step's copy out of the staging buffer has finished

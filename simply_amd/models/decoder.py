@@ -14,8 +14,7 @@ from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.spec import LayerSpec, ModelSpec, PartSpec
 from ..kernels import ops
 from ..parts.base import Block, ParamSpec, Part, PendingNorm
-from ..parts.embedding import EMBEDDINGS, HEADS
-from ..registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
 
 
 def _build_layer(spec: LayerSpec) -> Block:
@@ -29,12 +28,8 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec):
         spec.validate()
         self.spec = spec
-        if spec.embedding.kind not in EMBEDDINGS:
-            raise ValueError(f"unknown embedding {spec.embedding.kind!r}; known: {sorted(EMBEDDINGS)}")
-        if spec.head.kind not in HEADS:
-            raise ValueError(f"unknown head {spec.head.kind!r}; known: {sorted(HEADS)}")
-        self.embedding = EMBEDDINGS[spec.embedding.kind](**spec.embedding.params)
-        self.head = HEADS[spec.head.kind](**spec.head.params)
+        self.embedding = EMBEDDINGS.build(spec.embedding.kind, **spec.embedding.params)
+        self.head = HEADS.build(spec.head.kind, **spec.head.params)
         self.final_norm = NORMS.build(spec.final_norm.kind, **spec.final_norm.params)
         self.layers: list[Block] = [_build_layer(ls) for ls in spec.layers]
         self.loaded = False
@@ -81,9 +76,11 @@ class DecoderModel:
         return [(self.layers[e.layer].mixer.cache_need(), e.cache_from) for e in self.spec.schedule]
 
     # ------------------------------------------------------------------ forward
-    def forward(self, tokens: torch.Tensor, ctx, cache_views, logit_rows: torch.Tensor | None) -> torch.Tensor | None:
+    def forward(self, tokens: torch.Tensor, ctx, cache_views, logit_rows: torch.Tensor | None,
+                logits_out: torch.Tensor | None = None) -> torch.Tensor | None:
         """Runs this step's tokens through the schedule.  Returns float32 logits [R, V] at the rows of
-        the step that `logit_rows` (int32 [R]) names, or None if it is None or empty."""
+        the step that `logit_rows` (int32 [R]) names (in `logits_out` if that is given), or None if it is None or
+        empty."""
         h = self.embedding.forward(tokens)
         schedule = self.spec.schedule
         normed = None
@@ -96,4 +93,4 @@ class DecoderModel:
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         rows = ops.gather_rows(h, logit_rows)
-        return self.head.forward(PendingNorm(rows, None, None, self.final_norm, ctx.dtype))
+        return self.head.forward(PendingNorm(rows, None, None, self.final_norm, ctx.dtype), out=logits_out)

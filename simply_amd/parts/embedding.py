@@ -9,9 +9,11 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..registry import EMBEDDINGS, HEADS
 from .base import ParamSpec, Part, as_product_weight, project
 
 
+@EMBEDDINGS.register("scaled_embedding")
 class ScaledEmbedding(Part):
     def __init__(self, vocab_size: int, dim: int, scale: float):
         self.vocab_size, self.dim, self.scale = int(vocab_size), int(dim), float(scale)
@@ -31,6 +33,7 @@ class ScaledEmbedding(Part):
         return ops.embed(self.table, tokens, scale)
 
 
+@HEADS.register("linear_head")
 class LinearHead(Part):
     def __init__(self, vocab_size: int, dim: int, soft_cap: float | None):
         self.vocab_size, self.dim = int(vocab_size), int(dim)
@@ -43,10 +46,7 @@ class LinearHead(Part):
     def load(self, tensors):
         self.weight = as_product_weight(tensors["weight"], shared=True)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """x [R, D] activations (or a `PendingNorm` of them) -> float32 logits [R, V]."""
-        return project(x, self.weight, soft_cap=self.soft_cap, out_dtype=torch.float32)
+    def forward(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """x [R, D] activations (or a `PendingNorm` of them) -> float32 logits [R, V] (written into `out` if given)."""
+        return project(x, self.weight, soft_cap=self.soft_cap, out_dtype=torch.float32, out=out)
 
-
-EMBEDDINGS = {"scaled_embedding": ScaledEmbedding}
-HEADS = {"linear_head": LinearHead}

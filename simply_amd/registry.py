@@ -1,8 +1,8 @@
 """Name -> factory registries.
 
 One `Registry` object per kind of thing that a configuration can name: whole
-architectures, mixers, feed-forwards, norms, position encodings and block
-arrangements.  A registry is a plain dictionary with two rules taken from
+architectures, mixers, feed-forwards, norms, position encodings, block
+arrangements, embeddings, heads and activations.  A registry is a plain dictionary with two rules taken from
 simply/utils/registry.py:60-96: registering a name twice is an error, and asking
 for an unknown name is an error that lists the known names.
 """
@@ -63,4 +63,7 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("head")
+#: activation name -> code of the gated product's epilogue (simply_amd/csrc/activations.h)
 ACTIVATIONS = Registry("activation")

@@ -14,6 +14,7 @@ from simply_amd.cache import CacheManager
 from simply_amd.config import EngineConfig, LayerSpec, ModelSpec, PartSpec, ScheduleEntry, config_from_dict
 from simply_amd.engine import Executor, StepEntry
 from simply_amd.engine.context import GroupStep, StepContext
+from simply_amd.kernels import ops
 from simply_amd.models import DecoderModel
 from simply_amd.parts.base import FeedForward, Mixer, PagedKVNeed, ParamSpec, PositionEncoding, StateNeed
 from simply_amd.weights import init_random
@@ -95,6 +96,26 @@ def test_feed_forward_part(dtype):
     torch.testing.assert_close(part.forward(x).double().cpu(), want, rtol=tol, atol=tol * want.abs().max().item())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("activation", ["silu", "squared_relu"])
+def test_feed_forward_part_with_another_activation(dtype, activation):
+    """The gated feed-forward takes its activation by name from the registry; the ones beside Gemma 2's own."""
+    D, F = 96, 200
+    part = registry.FEED_FORWARDS.build("gated_dense", hidden_size=D, intermediate_size=F, activation=activation)
+    w = {n: rand(s, 10 + i, 0.1).to(dtype) for i, (n, s) in enumerate((("gate_proj", (F, D)), ("up_proj", (F, D)),
+                                                                       ("down_proj", (D, F))))}
+    part.load(w)
+    x = rand((11, D), 13).to(dtype)
+    g, u, d = (w[n].double().cpu() for n in ("gate_proj", "up_proj", "down_proj"))
+    xd = x.double().cpu()
+    act = {"silu": torch.nn.functional.silu, "squared_relu": lambda v: torch.relu(v) ** 2}[activation]
+    want = (act(xd @ g.T) * (xd @ u.T)) @ d.T
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    torch.testing.assert_close(part.forward(x).double().cpu(), want, rtol=tol, atol=tol * want.abs().max().item())
+    with pytest.raises(ValueError, match="unknown activation"):
+        registry.FEED_FORWARDS.build("gated_dense", hidden_size=D, intermediate_size=F, activation="swish7")
+
+
 @pytest.mark.parametrize("dtype,hd,page", [(torch.float32, 16, 4), (torch.bfloat16, 16, 4), (torch.bfloat16, 64, 16)])
 @pytest.mark.parametrize("window", [None, 8])
 def test_attention_part(dtype, hd, page, window):
@@ -140,7 +161,8 @@ def test_embedding_and_head_parts(dtype):
 class RunningMeanMixer(Mixer):
     """A toy mixer with a state of fixed size per request: y_t = W (decay * s_{t-1} + x_t), s_t = decay * s_{t-1} + x_t.
     It keeps no keys: its state lives in the request's state slot, from which a portion continues and into which
-    the portion's last state is written back."""
+    the portion's last state is written back.  Steps in which every request brings one token take the slots from
+    the device (`ctx.token_seq`), so that such a step can be recorded once and replayed for other requests."""
 
     def __init__(self, hidden_size: int, decay: float):
         self.hidden_size, self.decay = hidden_size, decay
@@ -153,6 +175,11 @@ class RunningMeanMixer(Mixer):
         return StateNeed((self.hidden_size,), torch.float32)
 
     def forward(self, x, ctx, cache):
+        if ctx.max_q_len == 1:
+            slots = ctx.token_seq.long()
+            s = self.decay * cache.state.index_select(0, slots) + x.float()
+            cache.state.index_copy_(0, slots, s)
+            return ops.gemm(s, self.proj.float()).to(x.dtype)
         out = torch.empty_like(x)
         for slot, a, b in zip(ctx.seq_slots, ctx.cu_q_lens[:-1], ctx.cu_q_lens[1:]):
             s = cache.state[slot]
@@ -263,6 +290,52 @@ def test_toy_parts_are_registered_built_and_stepped(toy_registry):
     # a new request in a slot that was used before starts from a zero state
     ex.finish_request("x")
     torch.testing.assert_close(run("z", [30]), whole, rtol=1e-4, atol=1e-4)
+
+
+def test_toy_state_advances_once_per_step_under_graphs(toy_registry):
+    """Decode-only steps are recorded in HIP graphs and replayed.  A mixer with a state of its own shows whether a
+    step runs exactly once (the step that is recorded included) and whether a replay serves other requests in
+    other slots than those it was recorded with: three requests decode together, finish at different times (so
+    the number of rows changes and new graphs are recorded on the way), a fourth takes over a freed slot; every
+    logit equals the request run whole."""
+    model = DecoderModel(toy_spec())
+    init_random(model, 0, torch.float32, torch.device(DEV), std=0.2)
+    reqs = {r: tiny.random_tokens(n, 128, 30 + i) for i, (r, n) in enumerate((("a", 24), ("b", 17), ("c", 30), ("d", 21)))}
+
+    def run(graphs):
+        cfg = EngineConfig(activation_dtype="float32", page_size=4, batch_size=3, max_seq_len=64,
+                           max_num_issue_tokens=64, total_num_pages=36, device=DEV, use_graphs=graphs)
+        ex = Executor(model, cfg)
+        got = {r: [] for r in reqs}
+        live, pending, pos = [], list(reqs), {}
+        while live or pending:
+            while pending and len(live) < 3:
+                r = pending.pop(0)
+                ex.add_request(r)
+                got[r].append(ex.step([StepEntry(r, reqs[r][:5], [0, 1, 2, 3, 4])]).cpu())   # its first portion, alone
+                pos[r] = 5
+                live.append(r)
+            logits = ex.step([StepEntry(r, [reqs[r][pos[r]]], [0]) for r in live]).cpu()
+            torch.cuda.synchronize()
+            for i, r in enumerate(live):
+                got[r].append(logits[i:i + 1])
+                pos[r] += 1
+            for r in [r for r in live if pos[r] == len(reqs[r])]:
+                ex.finish_request(r)
+                live.remove(r)
+        return {r: torch.cat(v) for r, v in got.items()}, ex
+
+    eager, _ = run(False)
+    replayed, ex = run(True)
+    assert {k[0] for k in ex._graphs} == {1, 2, 3}
+    whole_ex = Executor(model, EngineConfig(activation_dtype="float32", page_size=4, batch_size=3, max_seq_len=64,
+                                            max_num_issue_tokens=64, total_num_pages=36, device=DEV, use_graphs=False))
+    for r, t in reqs.items():
+        whole_ex.add_request(r)
+        whole = whole_ex.step([StepEntry(r, t, list(range(len(t))))]).cpu()
+        whole_ex.finish_request(r)
+        torch.testing.assert_close(eager[r], whole, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(replayed[r], whole, rtol=1e-4, atol=1e-4)
 
 
 def test_unknown_part_names_are_refused():
