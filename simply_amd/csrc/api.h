@@ -53,8 +53,9 @@ int sa_decode_advance(int B, int* step_counter, const int* sampled_tokens, const
 int sa_decode_slots(int B, const int* positions, const int* token_seq, const int* block_table, int table_stride,
                     int page_size, int64_t* slot_mapping, hipStream_t stream);
 
-// C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1: gelu_tanh(A.W^T) * (A.W2^T);
-// 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
+// C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1 + 16 * a: act(A.W^T) * (A.W2^T) with the activation
+// a of activations.h (0: tanh-approximated gelu, 1: silu, 2: squared relu), both products rounded to the output
+// type first; 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
 // few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel; 4: the wide-tile bfloat16 MFMA kernel for very
 // many rows (2, 3 and 4 refuse what they do not take).
 // packed: W (and W2) are tiled instead of row-major: [ceil(N / 16)][ceil(K / 32)][64][8] bfloat16, block (i, j)
@@ -71,7 +72,8 @@ int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* 
             void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // For 1..16 rows of bfloat16: h_out = h_in + norm(y; w_post) (y null: h_out is h_in and is not written; w_post null:
-// h_out = h_in + y), a = norm(h_out; w_next), C = epilogue(a . W^T) with W tiled (paired tiles for epilogue 1).
+// h_out = h_in + y), a = norm(h_out; w_next), C = epilogue(a . W^T) with W tiled (paired tiles for the gated
+// epilogue; epilogue codes as for sa_gemm).
 // h_in, h_out: float32 [M, K], different buffers; y: bfloat16 [M, K]; norm weights float32 or bfloat16 [K].
 int sa_gemm_normed_takes(int M, int N, int K);
 
@@ -164,10 +166,11 @@ void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* 
 
 namespace sa {
 int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
-                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, int packed, hipStream_t stream);
+                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, int act, float cap, int packed,
+                 hipStream_t stream);
 bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2);
 int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
-                int N, int K, int epi, float cap, int packed, int shape, hipStream_t stream);
+                int N, int K, int epi, int act, float cap, int packed, int shape, hipStream_t stream);
 bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q);
 int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
@@ -184,12 +187,12 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             hipStream_t stream);
 bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
                      const void* C, int c_dtype, int epi, int packed);
-int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
-              hipStream_t stream);
+int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
+              int shape, hipStream_t stream);
 bool gemm_streams_weights(int M, int NW, int K);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
-               int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream);
+               int epi, int act, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream);
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,

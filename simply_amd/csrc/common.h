@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "activations.h"
+
 namespace sa {
 
 // Element type codes used across the C interface.
@@ -76,14 +78,6 @@ __device__ inline float block_sum(float v, float* scratch /* >= 16 floats */) {
   float total = 0.f;
   for (int w = 0; w < nwaves; ++w) total += scratch[w];
   return total;
-}
-
-// tanh-approximated GELU for the bfloat16 kernels: tanh(u) = 1 - 2 / (exp(2 u) + 1) with the hardware's exponential and
-// reciprocal (relative error about 1e-6, far below a bfloat16 step); exact at both ends.  simply/model_lib.py:94-104.
-__device__ inline float gelu_tanh_fast(float x) {
-  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  const float t = 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * u) + 1.f);
-  return 0.5f * x * (1.f + t);
 }
 
 // Layout of a page of keys [page_size keys][hd]: row-major, or, when the sizes allow it, in 16-key x 32-dimension

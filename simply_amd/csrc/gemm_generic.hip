@@ -11,12 +11,6 @@ namespace sa {
 
 constexpr int BM = 64, BN = 64, BK = 16, TM = 4, TN = 4;
 
-__device__ inline float gelu_tanh(float x) {
-  // simply/model_lib.py:94-96
-  const float k = 0.7978845608028654f;  // sqrt(2/pi)
-  return 0.5f * x * (1.f + tanhf(k * (x + 0.044715f * x * x * x)));
-}
-
 // Index of W[n][k] in memory: row-major, or tiled [N / 16][chunks][kq 4][row 16][8] (chunks = ceil(K / 32)).  With
 // `paired` (the gated epilogue on tiled weights) the tiles of the gate and of the other factor alternate: the gate's
 // tile n / 16 is tile 2 (n / 16), the factor's follows it.
@@ -27,12 +21,12 @@ __device__ inline size_t w_index(int n, int k, int K, int chunks, int paired = 0
   return ((tile * chunks + k / 32) * 64 + ((k % 32) / 8) * 16 + n % 16) * 8 + k % 8;
 }
 
-// EPI: 0 plain, 1 gated (C = gelu(A.W^T) * (A.W2^T)), 2 soft-cap (C = cap * tanh(A.W^T / cap))
+// EPI: 0 plain, 1 gated (C = act(A.W^T) * (A.W2^T)), 2 soft-cap (C = cap * tanh(A.W^T / cap))
 template <typename TA, typename TW, typename TC, int EPI, bool PACKED>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, int64_t lda,
                                                            const TW* __restrict__ W, const TW* __restrict__ W2,
                                                            TC* __restrict__ C, int64_t ldc, int M, int N, int K,
-                                                           float cap) {
+                                                           float cap, int act) {
   __shared__ float As[BK][BM + 4];
   __shared__ float Ws[BK][BN + 4];
   __shared__ float W2s[EPI == 1 ? BK : 1][BN + 4];
@@ -87,7 +81,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
       float v = acc[i][j];
       if (EPI == 1) {
         // both products are rounded to the activation type first, as separate matrix products would be
-        v = gelu_tanh(to_float(from_float<TC>(v))) * to_float(from_float<TC>(acc2[i][j]));
+        v = gated_activation_exact(act, to_float(from_float<TC>(v))) * to_float(from_float<TC>(acc2[i][j]));
       } else if (EPI == 2) {
         v = cap * tanhf(v / cap);
       }
@@ -98,32 +92,33 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
 
 template <typename TA, typename TW, typename TC, bool PACKED>
 static void launch_generic(const void* A, int64_t lda, const void* W, const void* W2, void* C, int64_t ldc, int M, int N,
-                           int K, int epi, float cap, hipStream_t stream) {
+                           int K, int epi, int act, float cap, hipStream_t stream) {
   const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   const TA* a = static_cast<const TA*>(A);
   const TW* w = static_cast<const TW*>(W);
   const TW* w2 = static_cast<const TW*>(W2);
   TC* c = static_cast<TC*>(C);
   if (epi == 0)
-    gemm_generic_kernel<TA, TW, TC, 0, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
+    gemm_generic_kernel<TA, TW, TC, 0, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap, act);
   else if (epi == 1)
-    gemm_generic_kernel<TA, TW, TC, 1, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
+    gemm_generic_kernel<TA, TW, TC, 1, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap, act);
   else
-    gemm_generic_kernel<TA, TW, TC, 2, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap);
+    gemm_generic_kernel<TA, TW, TC, 2, PACKED><<<grid, 256, 0, stream>>>(a, lda, w, w2, c, ldc, M, N, K, cap, act);
 }
 
 int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
-                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, float cap, int packed, hipStream_t stream) {
+                 int c_dtype, int64_t ldc, int M, int N, int K, int epi, int act, float cap, int packed,
+                 hipStream_t stream) {
   if (a_dtype == kF32 && w_dtype == kF32 && c_dtype == kF32 && !packed)
-    launch_generic<float, float, float, false>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+    launch_generic<float, float, float, false>(A, lda, W, W2, C, ldc, M, N, K, epi, act, cap, stream);
   else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kBF16 && !packed)
-    launch_generic<bf16, bf16, bf16, false>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+    launch_generic<bf16, bf16, bf16, false>(A, lda, W, W2, C, ldc, M, N, K, epi, act, cap, stream);
   else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32 && !packed)
-    launch_generic<bf16, bf16, float, false>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+    launch_generic<bf16, bf16, float, false>(A, lda, W, W2, C, ldc, M, N, K, epi, act, cap, stream);
   else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kBF16 && packed)
-    launch_generic<bf16, bf16, bf16, true>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+    launch_generic<bf16, bf16, bf16, true>(A, lda, W, W2, C, ldc, M, N, K, epi, act, cap, stream);
   else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32 && packed)
-    launch_generic<bf16, bf16, float, true>(A, lda, W, W2, C, ldc, M, N, K, epi, cap, stream);
+    launch_generic<bf16, bf16, float, true>(A, lda, W, W2, C, ldc, M, N, K, epi, act, cap, stream);
   else {
     set_error("gemm: unsupported element types a=%d w=%d c=%d (tiled weights: bfloat16 only)", a_dtype, w_dtype,
               c_dtype);

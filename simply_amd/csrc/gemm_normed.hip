@@ -49,7 +49,7 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_post,
     const void* __restrict__ w_next, int w_next_dtype, float eps_next, float plus_next, const bf16* __restrict__ W,
     void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N, int K, int chunks, int act_rows, float cap,
-    RotaryArgs rot) {
+    int activation, RotaryArgs rot) {
   constexpr int NP = (EPI == 1 || EPI == 3) ? 2 : 1;  // tiles of W that a workgroup multiplies side by side
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int pitch = K + 8;                               // elements per row of activations in LDS
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
           sum[p] = t;
         }
         float v = sum[0];
-        if (EPI == 1) v = gelu_tanh_fast(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
+        if (EPI == 1) v = gated_activation(activation, to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
         else if (EPI == 2) v = cap * tanhf(v / cap);
         store_f(C, c_dtype, static_cast<size_t>(ml) * ldc + n, v);
       }
@@ -285,8 +285,8 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
 template <int EPI, int NCH>
 static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype, float eps_post,
                   float plus_post, const void* w_next, int w_next_dtype, float eps_next, float plus_next, const bf16* W,
-                  void* C, int c_dtype, int64_t ldc, int M, int N, int K, float cap, const RotaryArgs& rot,
-                  hipStream_t stream) {
+                  void* C, int c_dtype, int64_t ldc, int M, int N, int K, float cap, int activation,
+                  const RotaryArgs& rot, hipStream_t stream) {
   const int act_rows = M <= 8 ? 8 : 16;
   const size_t lds = static_cast<size_t>(act_rows) * (K + 8) * sizeof(bf16) +
                      static_cast<size_t>(kWaves) * ((EPI == 1 || EPI == 3) ? 2 : 1) * 16 * 17 * sizeof(float);
@@ -307,7 +307,7 @@ static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_
   const int grid = (ntiles + (ntiles + kMaxGroups - 1) / kMaxGroups - 1) / ((ntiles + kMaxGroups - 1) / kMaxGroups);
   kernel<<<grid, kWaves * kWave, lds, stream>>>(y, h_in, h_out, w_post, w_post_dtype, eps_post, plus_post, w_next,
                                                          w_next_dtype, eps_next, plus_next, W, C, c_dtype, ldc, M, N, K,
-                                                         (K + 31) / 32, act_rows, cap, rot);
+                                                         (K + 31) / 32, act_rows, cap, activation, rot);
   return check_launch("gemm_normed");
 }
 
@@ -332,13 +332,17 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
              "gemm_normed: the norm weights must be bfloat16");
   SA_REQUIRE(y == nullptr || (h_out != nullptr && h_out != h_in),
              "gemm_normed: with y the updated residual goes to a buffer other than the input");
+  const int activation = epilogue_activation(epilogue);
+  epilogue = epilogue_kind(epilogue);
   SA_REQUIRE(epilogue >= 0 && epilogue <= 2 && (epilogue != 2 || cap > 0.f), "gemm_normed: bad epilogue");
+  SA_REQUIRE(activation >= 0 && activation < kNumActivations && (epilogue == 1 || activation == 0),
+             "gemm_normed: unknown activation %d", activation);
   const bf16* yb = static_cast<const bf16*>(y);
   const bf16* w = static_cast<const bf16*>(W);
   const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
 #define SA_NORMED(EPI, NCH)                                                                                      \
   return normed::launch<EPI, NCH>(yb, h_in, h_out, w_post, w_post_dtype, eps_post, pp, w_next, w_next_dtype, eps_next, \
-                                  pn, w, C, c_dtype, ldc, M, N, K, cap, normed::RotaryArgs{}, stream)
+                                  pn, w, C, c_dtype, ldc, M, N, K, cap, activation, normed::RotaryArgs{}, stream)
 #define SA_NORMED_K(EPI)          \
   do {                            \
     if (K <= 2560) SA_NORMED(EPI, 10); \
@@ -382,7 +386,7 @@ extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_
 #define SA_ROTARY(NCH)                                                                                              \
   return normed::launch<3, NCH>(static_cast<const bf16*>(y), h_in, h_out, w_post, w_post_dtype, eps_post,             \
                                 plus_one_post ? 1.f : 0.f, w_next, w_next_dtype, eps_next, plus_one_next ? 1.f : 0.f, \
-                                static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, 0.f, rot, stream)
+                                static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, 0.f, 0, rot, stream)
   if (K <= 2560) SA_ROTARY(10);
   if (K <= 3584) SA_ROTARY(14);
   SA_ROTARY(18);

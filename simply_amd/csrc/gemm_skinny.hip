@@ -31,7 +31,7 @@ template <int MB, int EPI, bool PACKED>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restrict__ A, int64_t lda,
                                                            const bf16* __restrict__ W, const bf16* __restrict__ W2,
                                                            void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N,
-                                                           int K, int chunks, int tile_rows, float cap) {
+                                                           int K, int chunks, int tile_rows, float cap, int act) {
   constexpr int NP = EPI == 1 ? 2 : 1;  // planes: gate and up for the gated epilogue
   extern __shared__ float red[];        // [NW][NP][MB][16 * 17]
   const int tid = threadIdx.x, lane = tid % kWave;
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
     float v = sum[0];
     if (EPI == 1) {
       // both products are rounded to bfloat16 first, as separate matrix products would be
-      v = gelu_tanh_fast(to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
+      v = gated_activation(act, to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
     } else if (EPI == 2) {
       v = cap * tanhf(v / cap);
     }
@@ -151,20 +151,21 @@ static void choose_shape(int N, int chunks, int planes, int MB, int* tile_rows, 
 
 template <int MB, bool PACKED>
 static void launch_skinny(const bf16* A, int64_t lda, const bf16* W, const bf16* W2, void* C, int c_dtype, int64_t ldc,
-                          int M, int N, int K, int epi, float cap, int tile_rows, int waves, hipStream_t stream) {
+                          int M, int N, int K, int epi, int act, float cap, int tile_rows, int waves,
+                          hipStream_t stream) {
   const int chunks = (K + 31) / 32;
   const dim3 grid((N + tile_rows - 1) / tile_rows);
   const int threads = waves * kWave;
   const size_t lds = static_cast<size_t>(waves) * (epi == 1 ? 2 : 1) * MB * 16 * 17 * sizeof(float);
   if (epi == 0)
     gemm_skinny_kernel<MB, 0, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
-                                                                      tile_rows, cap);
+                                                                      tile_rows, cap, act);
   else if (epi == 1)
     gemm_skinny_kernel<MB, 1, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
-                                                                      tile_rows, cap);
+                                                                      tile_rows, cap, act);
   else
     gemm_skinny_kernel<MB, 2, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
-                                                                      tile_rows, cap);
+                                                                      tile_rows, cap, act);
 }
 
 bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2) {
@@ -175,7 +176,7 @@ bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const vo
 
 // shape > 0 fixes the cut: tile_rows * 100 + waves (for instance 816: 8 rows, 16 waves)
 int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
-                int N, int K, int epi, float cap, int packed, int shape, hipStream_t stream) {
+                int N, int K, int epi, int act, float cap, int packed, int shape, hipStream_t stream) {
   const int chunks = (K + 31) / 32, planes = epi == 1 ? 2 : 1;
   const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   int tile_rows, waves;
@@ -194,8 +195,10 @@ int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void*
   const bf16* w2 = static_cast<const bf16*>(W2);
 #define SA_SKINNY(MBV)                                                                                              \
   do {                                                                                                              \
-    if (packed) launch_skinny<MBV, true>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, tile_rows, waves, stream); \
-    else launch_skinny<MBV, false>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, cap, tile_rows, waves, stream);     \
+    if (packed)                                                                                                     \
+      launch_skinny<MBV, true>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream);    \
+    else                                                                                                            \
+      launch_skinny<MBV, false>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream);   \
   } while (0)
   if (MB == 1) SA_SKINNY(1);
   else if (MB == 2) SA_SKINNY(2);

@@ -39,7 +39,7 @@ constexpr int PITCH = BK + 8;   // elements per LDS row: 144 bytes
 template <int WM, int EPI, int WAVES_N, bool TAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __restrict__ W, void* __restrict__ C,
-                       int c_dtype, int64_t ldc, int M, int N, int K, int chunks, float cap,
+                       int c_dtype, int64_t ldc, int M, int N, int K, int chunks, float cap, int act,
                        float* __restrict__ partials) {
   constexpr int WAVES_M = 4 / WAVES_N;
   constexpr int BM = WAVES_M * WM * 16;
@@ -201,7 +201,8 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
         const int n = EPI == 1 ? (nt0 / 2 + j) * 16 + r : (nt0 + j) * 16 + r;
         if (n >= N) continue;
         float x;
-        if (EPI == 1) x = gelu_tanh_fast(to_float(float_to_bf16(acc[i][2 * j][v]))) * to_float(float_to_bf16(acc[i][2 * j + 1][v]));
+        if (EPI == 1)
+          x = gated_activation(act, to_float(float_to_bf16(acc[i][2 * j][v]))) * to_float(float_to_bf16(acc[i][2 * j + 1][v]));
         else if (EPI == 2) x = cap * tanhf(acc[i][j][v] / cap);
         else x = acc[i][j][v];
         store_f(C, c_dtype, static_cast<size_t>(m) * ldc + n, x);
@@ -214,7 +215,7 @@ void gemm_tiled_kernel(const bf16* __restrict__ A, int64_t lda, const bf16* __re
 // factor 16 further.
 template <int EPI>
 __global__ void gemm_reduce_kernel(const float* __restrict__ partials, int KS, void* __restrict__ C, int c_dtype,
-                                   int64_t ldc, int M, int N, int NW, float cap) {
+                                   int64_t ldc, int M, int N, int NW, float cap, int act) {
   const size_t total = static_cast<size_t>(M) * N, plane = static_cast<size_t>(M) * NW;
   for (size_t e = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; e < total;
        e += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -236,7 +237,7 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partials, int KS, v
         y += py[j];
       }
     }
-    if (EPI == 1) x = gelu_tanh_fast(to_float(float_to_bf16(x))) * to_float(float_to_bf16(y));
+    if (EPI == 1) x = gated_activation(act, to_float(float_to_bf16(x))) * to_float(float_to_bf16(y));
     else if (EPI == 2) x = cap * tanhf(x / cap);
     store_f(C, c_dtype, m * ldc + n, x);
   }
@@ -244,20 +245,20 @@ __global__ void gemm_reduce_kernel(const float* __restrict__ partials, int KS, v
 
 template <int WM, int EPI, int WAVES_N>
 static void launch(const bf16* A, int64_t lda, const bf16* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
-                   float cap, int ks, float* partials, hipStream_t stream) {
+                   float cap, int act, int ks, float* partials, hipStream_t stream) {
   constexpr int BM = (4 / WAVES_N) * WM * 16, BNW = WAVES_N * 64;
   const int NW = EPI == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM, ks);
   if (K % BK == 0)
     gemm_tiled_kernel<WM, EPI, WAVES_N, false><<<grid, 256, 0, stream>>>(A, lda, W, C, c_dtype, ldc, M, N, K, (K + 31) / 32,
-                                                                         cap, partials);
+                                                                         cap, act, partials);
   else
     gemm_tiled_kernel<WM, EPI, WAVES_N, true><<<grid, 256, 0, stream>>>(A, lda, W, C, c_dtype, ldc, M, N, K, (K + 31) / 32,
-                                                                        cap, partials);
+                                                                        cap, act, partials);
   if (ks > 1) {
     const size_t total = static_cast<size_t>(M) * N;
     const int blocks = static_cast<int>((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
-    gemm_reduce_kernel<EPI><<<blocks, 256, 0, stream>>>(partials, ks, C, c_dtype, ldc, M, N, NW, cap);
+    gemm_reduce_kernel<EPI><<<blocks, 256, 0, stream>>>(partials, ks, C, c_dtype, ldc, M, N, NW, cap, act);
   }
 }
 
@@ -281,7 +282,7 @@ bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const voi
 
 // ksplit > 0 fixes the number of cuts of K.
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,
-               int epi, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+               int epi, int act, float cap, int ksplit, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   const bf16* a = static_cast<const bf16*>(A);
   const bf16* w = static_cast<const bf16*>(W);
   float* ws = static_cast<float*>(workspace);
@@ -306,9 +307,9 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
   while (ks > 1 && (ws == nullptr || static_cast<size_t>(ks) * M * NW * sizeof(float) > workspace_bytes)) --ks;
 #define SA_TILED(WM, WN)                                                                                      \
   do {                                                                                                        \
-    if (epi == 1) tiled::launch<WM, 1, WN>(a, lda, w, C, c_dtype, ldc, M, N, K, cap, ks, ws, stream);          \
-    else if (epi == 2) tiled::launch<WM, 2, WN>(a, lda, w, C, c_dtype, ldc, M, N, K, cap, ks, ws, stream);     \
-    else tiled::launch<WM, 0, WN>(a, lda, w, C, c_dtype, ldc, M, N, K, cap, ks, ws, stream);                   \
+    if (epi == 1) tiled::launch<WM, 1, WN>(a, lda, w, C, c_dtype, ldc, M, N, K, cap, act, ks, ws, stream);      \
+    else if (epi == 2) tiled::launch<WM, 2, WN>(a, lda, w, C, c_dtype, ldc, M, N, K, cap, act, ks, ws, stream); \
+    else tiled::launch<WM, 0, WN>(a, lda, w, C, c_dtype, ldc, M, N, K, cap, act, ks, ws, stream);               \
   } while (0)
   if (few) SA_TILED(4, 4);
   else SA_TILED(4, 2);

@@ -61,7 +61,7 @@ __device__ __forceinline__ void load_to_lds(const bf16* base, uint32_t offset, u
 template <int WM, int WN, int WAVES_M, int EPI, int NSTAGE, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __restrict__ A, int64_t lda,
                                                         const bf16* __restrict__ W, bf16* __restrict__ C, int64_t ldc,
-                                                        int M, int N, int K, int chunks) {
+                                                        int M, int N, int K, int chunks, int act) {
   constexpr int WAVES_N = WAVES / WAVES_M;
   constexpr int MT = WAVES_M * WM, NT = WAVES_N * WN;  // 16-row tiles of A and of W per workgroup
   constexpr int BM = MT * 16;
@@ -234,7 +234,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         if (EPI == 1)
-          x[v] = gelu_tanh_fast(to_float(float_to_bf16(acc[i][2 * j][v]))) * to_float(float_to_bf16(acc[i][2 * j + 1][v]));
+          x[v] = gated_activation(act, to_float(float_to_bf16(acc[i][2 * j][v]))) *
+                 to_float(float_to_bf16(acc[i][2 * j + 1][v]));
         else
           x[v] = acc[i][j][v];
       }
@@ -248,14 +249,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
 
 template <int WM, int WN, int WAVES_M, int NSTAGE, int WAVES = 8>
 static void launch(const bf16* A, int64_t lda, const bf16* W, bf16* C, int64_t ldc, int M, int N, int K, int epi,
-                   hipStream_t stream) {
+                   int act, hipStream_t stream) {
   constexpr int BM = WAVES_M * WM * 16, BNW = (WAVES / WAVES_M) * WN * 16;
   const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM);
   if (epi == 1)
-    gemm_wide_kernel<WM, WN, WAVES_M, 1, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
+    gemm_wide_kernel<WM, WN, WAVES_M, 1, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32,
+                                                                                         act);
   else
-    gemm_wide_kernel<WM, WN, WAVES_M, 0, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32);
+    gemm_wide_kernel<WM, WN, WAVES_M, 0, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32,
+                                                                                         act);
 }
 
 }  // namespace wide
@@ -270,8 +273,8 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
 
 // shape: 0: chosen here; else stages * 1000000 + rows * 1000 + weight rows of a workgroup's tile (2256192, 3256128,
 // 3128256, 3192128; 2128192: workgroups of four waves, two to a CU).
-int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int shape,
-              hipStream_t stream) {
+int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
+              int shape, hipStream_t stream) {
   const bf16* a = static_cast<const bf16*>(A);
   const bf16* w = static_cast<const bf16*>(W);
   bf16* c = static_cast<bf16*>(C);
@@ -296,11 +299,11 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     }
   }
   switch (shape) {
-    case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
-    case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
-    case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
-    case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, stream); break;
-    case 2128192: wide::launch<4, 6, 2, 2, 4>(a, lda, w, c, ldc, M, N, K, epi, stream); break;  // two workgroups per CU
+    case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 2128192: wide::launch<4, 6, 2, 2, 4>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;  // two workgroups per CU
     default:
       set_error("gemm: unknown wide tile %d", shape);
       return 1;

@@ -39,7 +39,10 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
   SA_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld are below K=%d, N=%d", (long long)lda,
              (long long)ldc, K, N);
+  const int act = epilogue_activation(epilogue);
+  epilogue = epilogue_kind(epilogue);
   SA_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm: unknown epilogue %d", epilogue);
+  SA_REQUIRE(act >= 0 && act < kNumActivations && (epilogue == 1 || act == 0), "gemm: unknown activation %d", act);
   SA_REQUIRE(epilogue != 1 || (W2 != nullptr) != (packed != 0),
              "gemm: the gated epilogue takes two row-major weights, or one tiled weight that holds both");
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
@@ -62,7 +65,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
                "operands; got M=%d K=%d lda=%lld", M, K, (long long)lda);
     if (takes)
-      return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, shape, stream);
+      return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, shape, stream);
   }
   // once the product is no longer bound by streaming the weights: the wide tiles (both operands through LDS); and
   // the gated product from 17 rows on, whose very many weight rows fill the GPU with the wide kernel's workgroups
@@ -76,7 +79,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "gemm: the wide MFMA kernel takes bfloat16 in and out with tiled weights, no soft-cap, K a multiple of "
                "64, N and ldc of 4, lda of 8; got N=%d K=%d lda=%lld ldc=%lld tiled=%d", N, K, (long long)lda,
                (long long)ldc, packed);
-    if (takes) return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, algo == 4 ? shape : 0, stream);
+    if (takes) return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape : 0, stream);
   }
   if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || tiled_first))) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
@@ -84,10 +87,10 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
                "aligned operands; got K=%d lda=%lld tiled=%d", K, (long long)lda, packed);
     if (takes)
-      return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, cap, shape, workspace,
+      return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, act, cap, shape, workspace,
                         static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
   }
-  return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, packed, stream);
+  return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, stream);
 }
 
 extern "C" int sa_paged_attention(const void* q, int dtype, int64_t q_stride, const void* k_pages,

@@ -264,7 +264,16 @@ def decode_slots(positions: torch.Tensor, token_seq: torch.Tensor, block_table: 
 
 # --------------------------------------------------------------------------- matrix products
 
-EPILOGUE_NONE, EPILOGUE_GATED_GELU, EPILOGUE_SOFT_CAP = 0, 1, 2
+EPILOGUE_NONE, EPILOGUE_GATED, EPILOGUE_SOFT_CAP = 0, 1, 2
+#: activations of the gated epilogue (simply_amd/csrc/activations.h); the epilogue argument is 1 + 16 * activation
+ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU = 0, 1, 2
+
+
+def _gated(activation: int) -> int:
+    if activation not in (ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU):
+        raise KernelError(f"unknown activation code {activation!r}")
+    return EPILOGUE_GATED + 16 * activation
+
 
 #: scratch memory for partial results (attention over key ranges, products with K cut over workgroups), one per
 #: device, allocated at first use; kernels on one stream use it one after the other
@@ -296,9 +305,9 @@ def library_gemm_min_rows() -> int:
 
 def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
          soft_cap: float | None = None, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
-         algo: int = ALGO_AUTO, shape: int = 0) -> torch.Tensor:
-    """a[M, K] . w[N, K]^T.  With w2 (row-major weights) or a paired `TiledWeight`: gelu_tanh(a.wg^T) * (a.wu^T).
-    With soft_cap: cap * tanh(. / cap).  w is a row-major tensor or a `TiledWeight`."""
+         algo: int = ALGO_AUTO, shape: int = 0, activation: int = ACT_GELU_TANH) -> torch.Tensor:
+    """a[M, K] . w[N, K]^T.  With w2 (row-major weights) or a paired `TiledWeight`: act(a.wg^T) * (a.wu^T) with
+    the activation of that code.  With soft_cap: cap * tanh(. / cap).  w is a row-major tensor or a `TiledWeight`."""
     packed = isinstance(w, TiledWeight)
     wd = w.data if packed else w
     w2d = None
@@ -319,13 +328,13 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
         raise KernelError(f"gemm: a is {a.dtype} but the weight is {wd.dtype}")
     epi, cap = EPILOGUE_NONE, 0.0
     if paired:
-        epi = EPILOGUE_GATED_GELU
+        epi = _gated(activation)
     elif w2 is not None:
         if soft_cap:
             raise KernelError("gemm: the gated and the soft-cap epilogue do not combine")
         if tuple(w2.shape) != tuple(w.shape) or w2d.dtype != wd.dtype or not w2d.is_contiguous():
             raise KernelError("gemm: the second weight must match the first")
-        epi = EPILOGUE_GATED_GELU
+        epi = _gated(activation)
     elif soft_cap:
         epi, cap = EPILOGUE_SOFT_CAP, float(soft_cap)
     if out is None:
@@ -353,7 +362,8 @@ def gemm_normed_takes(M: int, w) -> bool:
 def gemm_normed(y: torch.Tensor | None, h_in: torch.Tensor, h_out: torch.Tensor | None, w: TiledWeight, *,
                 post_weight: torch.Tensor | None, post_eps: float, post_plus_one: bool, next_weight: torch.Tensor,
                 next_eps: float, next_plus_one: bool, soft_cap: float | None = None,
-                out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+                out_dtype: torch.dtype = torch.bfloat16, out: torch.Tensor | None = None,
+                activation: int = ACT_GELU_TANH) -> torch.Tensor:
     """h_out = h_in + norm(y; post) (y None: the residual stays h_in); returns epilogue(norm(h_out; next) . w^T),
     in one kernel, for up to 16 rows.  The residual buffers are float32 [M, K] and must differ."""
     _dev(y, h_in, h_out, post_weight, next_weight, w.data)
@@ -371,10 +381,13 @@ def gemm_normed(y: torch.Tensor | None, h_in: torch.Tensor, h_out: torch.Tensor 
             raise KernelError("gemm_normed: a norm weight does not match the width")
     epi, cap = EPILOGUE_NONE, 0.0
     if w.paired:
-        epi = EPILOGUE_GATED_GELU
+        epi = _gated(activation)
     elif soft_cap:
         epi, cap = EPILOGUE_SOFT_CAP, float(soft_cap)
-    out = torch.empty((M, w.rows), dtype=out_dtype, device=h_in.device)
+    if out is None:
+        out = torch.empty((M, w.rows), dtype=out_dtype, device=h_in.device)
+    if tuple(out.shape) != (M, w.rows) or out.stride(1) != 1 or out.device != h_in.device:
+        raise KernelError(f"gemm_normed: the output must be [{M}, {w.rows}] with contiguous rows on the inputs' device")
     _lib.call("sa_gemm_normed", _ptr(y), _ptr(h_in), _ptr(h_out), _ptr(post_weight),
               _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one),
               _ptr(next_weight), _code(next_weight), float(next_eps), int(next_plus_one), _ptr(w.data), _ptr(out),

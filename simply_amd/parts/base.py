@@ -150,9 +150,12 @@ def pending_product(x: PendingNorm, run) -> torch.Tensor:
     return out
 
 
-def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | None = None,
+            out: torch.Tensor | None = None, activation: int = 0) -> torch.Tensor:
     """x . w^T (gated if w is a paired tiled weight) for activations x or a `PendingNorm`.  A pending norm is done
-    inside the product's kernel when that kernel takes the sizes; otherwise it is materialized first."""
+    inside the product's kernel when that kernel takes the sizes; otherwise it is materialized first.  `out`: where
+    the result goes (a buffer of the caller's), else a new tensor.  `activation`: the gated product's (a code of
+    the ACTIVATIONS registry)."""
     import functools
 
     from ..kernels import ops
@@ -160,9 +163,10 @@ def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | Non
     if isinstance(x, PendingNorm):
         if pending_fits_product(x, w):
             return pending_product(x, functools.partial(ops.gemm_normed, w=w, soft_cap=soft_cap,
-                                                        out_dtype=out_dtype or x.dtype))
+                                                        out_dtype=out_dtype or x.dtype, out=out,
+                                                        activation=activation))
         x = x.materialize()
-    return ops.gemm(x, w, soft_cap=soft_cap, out_dtype=out_dtype)
+    return ops.gemm(x, w, soft_cap=soft_cap, out_dtype=out_dtype, out=out, activation=activation)
 
 
 class Part:

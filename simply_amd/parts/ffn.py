@@ -1,5 +1,6 @@
 """Dense gated feed-forward: down(act(gate(x)) * up(x))  (simply/model_lib.py:643-730 with
-use_gated_activation_in_ffn=True, ffn_use_bias=False)."""
+use_gated_activation_in_ffn=True, ffn_use_bias=False; `act` by its name in the registry, as
+simply/model_lib.py:723 looks `ffn_activation` up)."""
 from __future__ import annotations
 
 import torch
@@ -8,8 +9,10 @@ from ..kernels import ops
 from ..registry import ACTIVATIONS, FEED_FORWARDS
 from .base import FeedForward, ParamSpec, PendingNorm, as_product_weight, project
 
-# activation name -> epilogue of the fused gate/up product
-ACTIVATIONS.register("gelu_tanh", ops.EPILOGUE_GATED_GELU)
+# activation name -> its code in the gated product's epilogue (simply/model_lib.py:93-104 registers these three)
+ACTIVATIONS.register("gelu_tanh", ops.ACT_GELU_TANH)
+ACTIVATIONS.register("silu", ops.ACT_SILU)
+ACTIVATIONS.register("squared_relu", ops.ACT_SQUARED_RELU)
 
 
 @FEED_FORWARDS.register("gated_dense")
@@ -18,9 +21,8 @@ class GatedDense(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh"):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
-        if ACTIVATIONS.get(activation) != ops.EPILOGUE_GATED_GELU:
-            raise ValueError(f"gated_dense: activation {activation!r} has no fused kernel")
         self.activation = activation
+        self.activation_code = int(ACTIVATIONS.get(activation))   # an unknown name is refused with the known ones
         self.gate_proj = self.up_proj = self.down_proj = self.gate_up = None
 
     def param_specs(self):
@@ -41,9 +43,9 @@ class GatedDense(FeedForward):
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         # gelu(x.Wg^T) * (x.Wu^T), one kernel
         if self.gate_up is not None:
-            z = project(x, self.gate_up)
+            z = project(x, self.gate_up, activation=self.activation_code)
         else:
             if isinstance(x, PendingNorm):
                 x = x.materialize()
-            z = ops.gemm(x, self.gate_proj, w2=self.up_proj)
+            z = ops.gemm(x, self.gate_proj, w2=self.up_proj, activation=self.activation_code)
         return ops.gemm(z, self.down_proj)

@@ -562,6 +562,45 @@ def test_score(V):
     assert got[4] == ops.SCORE_MASKED and got[8] == ops.SCORE_MASKED and got[5] > -1e3   # greedy rows; a plain draw
 
 
+@pytest.mark.parametrize("activation", [0, 1, 2])
+@pytest.mark.parametrize("M", [5, 16, 40, 300])
+def test_gated_activations_in_every_product_kernel(M, activation):
+    """act(a.Wg^T) * (a.Wu^T) for the three activations that the reference registers (tanh-gelu, silu, squared relu:
+    simply/model_lib.py:93-104), in each kernel that has the gated epilogue: the 32-bit one, the few-rows one, the
+    one with the norms in front, the tiled one with and without its sum kernel, the wide one."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_gate_up
+    N, K = 200, 256
+    a = rand((M, K), torch.bfloat16, 130, 1.5)
+    w, w2 = rand((N, K), torch.bfloat16, 131, 0.08), rand((N, K), torch.bfloat16, 132, 0.08)
+    tg = pack_gate_up(w, w2)
+    want = ref.gemm(a, w, w2=w2, activation=activation).float()
+    assert want.abs().max() > 0.5
+    if activation:
+        assert not torch.allclose(want, ref.gemm(a, w, w2=w2).float(), rtol=2e-2, atol=2e-2)   # the activations differ
+    t = dict(rtol=2e-2, atol=2e-2)
+    a32, w32, w232 = a.float(), w.float(), w2.float()
+    torch.testing.assert_close(ops.gemm(a32, w32, w2=w232, activation=activation),
+                               ref.gemm(a32, w32, w2=w232, activation=activation), rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(ops.gemm(a, w, w2=w2, activation=activation, algo=ops.ALGO_GENERIC).float(), want, **t)
+    torch.testing.assert_close(ops.gemm(a, tg, activation=activation).float(), want, **t)      # the dispatcher's choice
+    if M <= 16:
+        torch.testing.assert_close(ops.gemm(a, tg, activation=activation, algo=ops.ALGO_SKINNY).float(), want, **t)
+        h = a.float() * 3.0
+        wn = rand((K,), torch.bfloat16, 133, 0.3)
+        normed = ref.rmsnorm(h, wn, 1e-6, True, torch.bfloat16)
+        got = ops.gemm_normed(None, h, None, tg, post_weight=None, post_eps=0.0, post_plus_one=True, next_weight=wn,
+                              next_eps=1e-6, next_plus_one=True, activation=activation)
+        torch.testing.assert_close(got.float(), ref.gemm(normed, w, w2=w2, activation=activation).float(), **t)
+    for cuts in (1, 2):
+        got = ops.gemm(a, tg, activation=activation, algo=ops.ALGO_TILED, shape=cuts)
+        torch.testing.assert_close(got.float(), want, **t)
+    torch.testing.assert_close(ops.gemm(a, tg, activation=activation, algo=ops.ALGO_WIDE).float(), want, **t)
+    from simply_amd.kernels.lib import KernelError
+    with pytest.raises(KernelError, match="activation"):
+        ops.gemm(a, tg, activation=3)
+
+
 @pytest.mark.parametrize("M", [1, 8, 13, 16])
 @pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (3584, 512), (4608, 64), (4640, 64), (96, 40),
                                  (72, 64)])

@@ -106,7 +106,18 @@ def gelu_tanh(x):
     return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
 
 
-def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0):
+def silu(x):
+    return x * torch.sigmoid(x)
+
+
+def squared_relu(x):
+    return torch.relu(x) ** 2
+
+
+ACTIVATIONS = (gelu_tanh, silu, squared_relu)   # by the kernels' activation codes
+
+
+def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0, activation=0):
     out_dtype = out_dtype or a.dtype
     if getattr(w, "paired", False):
         from simply_amd.kernels.packing import unpack_gate_up
@@ -114,7 +125,7 @@ def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shap
     c = _f(a) @ _f(w).T
     if w2 is not None:
         up = _f(a) @ _f(w2).T
-        c = gelu_tanh(_f(c.to(out_dtype))) * _f(up.to(out_dtype))
+        c = ACTIVATIONS[activation](_f(c.to(out_dtype))) * _f(up.to(out_dtype))
     elif soft_cap:
         c = soft_cap * torch.tanh(c / soft_cap)
     c = c.to(out_dtype)
