@@ -8,6 +8,9 @@ with the same (pages, page size, window) share the bookkeeping (:865-917).  Diff
 bookkeeping lives on the host, a block table is indexed by the absolute block number of a key
 (position // page_size) so that a windowed group leaves holes instead of shifting its table, and
 running out of pages is reported to the caller instead of being excluded by construction.
+Every group has a pool of its own size: a windowed group's holds what its requests can hold at
+once (`windowed_pool_pages`), as the reference sizes its local pool by the window (:95-110,
+simply/serving/page_server.py:180-196).
 
 Bookkeeping is separate from storage: `CacheManager(device=None)` keeps no tensors and runs
 anywhere.
@@ -34,6 +37,15 @@ class OutOfPages(CacheError):
 
 def ceil_div(a: int, b: int) -> int:
     return -(-a // b)
+
+
+def windowed_pool_pages(window: int, page_size: int, num_slots: int, max_step_tokens: int) -> int:
+    """The most pages that `num_slots` requests of a group with this window hold at once.  A request that has run
+    c tokens and brings q more holds blocks floor((c - window + 1) / P) .. ceil((c + q) / P) - 1, at most
+    (window - 1 + q) / P + 2 of them; the q of one step add up to max_step_tokens at most.  (The reference,
+    whose steps never hold more than the window, has ceil(window / P) + 1 per request:
+    simply/utils/ragged_paged_attention.py:95-110.)"""
+    return num_slots * (ceil_div(max(window - 1, 0), page_size) + 2) + ceil_div(max_step_tokens, page_size)
 
 
 class PagePool:
@@ -111,6 +123,16 @@ class CacheGroup:
         if rid in self.seqs:
             raise CacheError(f"request {rid!r} is already in group {self.group_id}")
         self.seqs[rid] = _Sequence(slot)
+
+    def new_blocks(self, rid: Hashable, new_num_tokens: int) -> int:
+        """Pages that `extend(rid, new_num_tokens)` would take."""
+        s = self.seqs[rid]
+        return max(ceil_div(new_num_tokens, self.page_size) - ceil_div(s.num_tokens, self.page_size), 0)
+
+    def releasable(self, rid: Hashable, num_computed: int | None) -> int:
+        """Pages that `release_window(rid, num_computed)` would give back."""
+        s = self.seqs[rid]
+        return max(min(self.dead_blocks(num_computed), ceil_div(s.num_tokens, self.page_size)) - s.first_block, 0)
 
     def release_window(self, rid: Hashable, num_computed: int) -> list[int]:
         s = self.seqs[rid]
@@ -217,7 +239,12 @@ class CacheManager:
     """
 
     def __init__(self, needs, *, page_size: int, num_pages: int, num_slots: int, max_seq_len: int,
-                 dtype: torch.dtype = torch.float32, device=None, poison: bool = False):
+                 dtype: torch.dtype = torch.float32, device=None, poison: bool = False,
+                 max_step_tokens: int | None = None, group_pages=None):
+        """num_pages: pages of a group that keeps every key.  A windowed group gets the fewer pages that its
+        requests can hold at once when a step brings at most `max_step_tokens` tokens (None: as many as the
+        others).  group_pages: a function (need, default number) -> number, for a group with a pool of another
+        size."""
         self.page_size, self.num_pages, self.num_slots = int(page_size), int(num_pages), int(num_slots)
         self.max_seq_len, self.dtype, self.device, self.poison = int(max_seq_len), dtype, device, bool(poison)
         self.slots = StateSlots(num_slots)
@@ -226,6 +253,9 @@ class CacheManager:
         #: a number that is new for every admission (a request that comes back after giving up its pages gets another)
         self.admission: dict[Hashable, int] = {}
         self._admissions = 0
+        #: per request the number of its tokens whose step has been handed to the GPU (`mark_issued`): the queries
+        #: still to come start there, so a window's pages below what they see can go
+        self.issued: dict[Hashable, int] = {}
         self.views: list[CacheView] = []
         self._group_entries: dict[int, list[int]] = {}
         self._device_tables: dict[int, torch.Tensor] = {}
@@ -244,17 +274,24 @@ class CacheManager:
             elif isinstance(need, PagedKVNeed):
                 group = by_need.get(need)
                 if group is None:
-                    group = CacheGroup(len(self.groups), need, self.page_size, self.num_pages, self.num_slots, max_blocks)
+                    pages = self.num_pages
+                    if need.window is not None and max_step_tokens is not None:
+                        pages = min(pages, windowed_pool_pages(need.window, self.page_size, self.num_slots,
+                                                               int(max_step_tokens)))
+                    if group_pages is not None:
+                        pages = int(group_pages(need, pages))
+                    group = CacheGroup(len(self.groups), need, self.page_size, pages, self.num_slots, max_blocks)
                     by_need[need] = group
                     self.groups.append(group)
                     self._group_entries[group.group_id] = []
                 view = CacheView(need, group.group_id)
                 if device is not None:
                     fill = float("nan") if poison else 0.0
-                    view.k_pages = torch.full((self.num_pages, need.num_kv_heads, self.page_size, need.head_dim), fill,
+                    n = group.pool.num_pages
+                    view.k_pages = torch.full((n, need.num_kv_heads, self.page_size, need.head_dim), fill,
                                               dtype=dtype, device=device)
                     # values are stored transposed, so that the keys of a page are contiguous for each dimension
-                    view.v_pages = torch.full((self.num_pages, need.num_kv_heads, need.head_dim, self.page_size), fill,
+                    view.v_pages = torch.full((n, need.num_kv_heads, need.head_dim, self.page_size), fill,
                                               dtype=dtype, device=device)
                 self._group_entries[group.group_id].append(i)
                 self.views.append(view)
@@ -282,6 +319,7 @@ class CacheManager:
         self.requests[rid] = slot
         self._admissions += 1
         self.admission[rid] = self._admissions
+        self.issued[rid] = 0
         for g in self.groups:
             g.add(rid, slot)
         for v in self.views:
@@ -295,33 +333,82 @@ class CacheManager:
     def pages_needed(self, rid: Hashable, num_computed: int, q_len: int) -> dict[int, int]:
         return {g.group_id: g.pages_needed(rid, num_computed, q_len) for g in self.groups}
 
+    def _release_points(self, wants: Sequence[tuple[Hashable, int, int]]) -> dict[Hashable, int]:
+        """For every live request the position from which its next queries look back: where its tokens of this
+        step begin, or, for a request that this step leaves out, the end of what has been handed to the GPU."""
+        points = dict(self.issued)
+        for rid, nc, _ in wants:
+            points[rid] = nc
+        return points
+
+    def mark_issued(self, wants: Sequence[tuple[Hashable, int, int]]) -> None:
+        """The step that `reserve_all(wants)` made room for has been handed to the GPU (in stream order before
+        anything that a later step writes): the requests' next queries begin behind it."""
+        for rid, nc, q in wants:
+            if rid in self.issued:
+                self.issued[rid] = nc + q
+
     def can_reserve(self, wants: Sequence[tuple[Hashable, int, int]]) -> bool:
-        """Whether every group can hold all of `wants` = (request, num_computed, q_len) together."""
+        """Whether every group can hold all of `wants` = (request, num_computed, q_len) together, once every live
+        request, in the step or not, has given back the pages that its window has passed (`reserve_all` does it in
+        that order)."""
+        points = self._release_points(wants)
         for g in self.groups:
-            if sum(g.pages_needed(rid, nc, q) for rid, nc, q in wants) > g.pool.num_free:
+            free = g.pool.num_free
+            if g.need.window is not None:
+                free += sum(g.releasable(rid, at) for rid, at in points.items())
+            if sum(g.new_blocks(rid, nc + q) for rid, nc, q in wants) > free:
                 return False
         return True
 
-    def reserve(self, rid: Hashable, num_computed: int, q_len: int, *, fits: bool = False) -> None:
-        """Makes room for tokens [num_computed, num_computed + q_len) in every group: first gives back
-        the pages that the window has passed, then takes new ones.  Raises OutOfPages, with nothing
-        changed, if any group is short (fits: the caller has asked `can_reserve` for this and the rest of what it
-        reserves, so that is not asked again)."""
-        if num_computed + q_len > self.max_seq_len:
-            raise CacheError(f"request {rid!r}: {num_computed + q_len} tokens exceed max_seq_len {self.max_seq_len}")
-        for g in self.groups if not fits else ():
-            short = g.pages_needed(rid, num_computed, q_len) - g.pool.num_free
-            if short > 0:
-                raise OutOfPages(f"group {g.group_id} (window {g.need.window}): {short} pages short for request "
-                                 f"{rid!r}")
+    def can_hold(self, num_tokens: int, max_step_tokens: int) -> bool:
+        """Whether the free pages of every group hold a new request of `num_tokens` tokens that runs in steps of at
+        most `max_step_tokens`: all of its pages in a group that keeps every key, the most it ever holds at once
+        in a windowed one."""
+        points = self._release_points(())
         for g in self.groups:
-            self._poison(g, g.release_window(rid, num_computed))
-            g.extend(rid, num_computed + q_len)
+            peak = ceil_div(num_tokens, self.page_size)
+            free = g.pool.num_free
+            if g.need.window is not None:
+                step = min(num_tokens, max(int(max_step_tokens), 1))
+                peak = min(peak, ceil_div(g.need.window - 1 + step, self.page_size) + 1)
+                free += sum(g.releasable(rid, at) for rid, at in points.items())
+            if peak > free:
+                return False
+        return True
+
+    def reserve_all(self, wants: Sequence[tuple[Hashable, int, int]]) -> None:
+        """Makes room for the tokens [num_computed, num_computed + q_len) of every (request, num_computed, q_len) in
+        every group: all of it or, with OutOfPages, nothing.  The pages that windows have passed are given back
+        first, by every live request (also those that the step leaves out: what they hold beyond their window
+        is of no use to anyone), then the new ones are taken: a request whose window frees pages makes room for
+        another wherever the two stand in `wants`."""
+        for rid, nc, q in wants:
+            if nc + q > self.max_seq_len:
+                raise CacheError(f"request {rid!r}: {nc + q} tokens exceed max_seq_len {self.max_seq_len}")
+        if not self.can_reserve(wants):
+            raise OutOfPages("the cache cannot hold this step's tokens: " + ", ".join(
+                f"{rid!r}+{q}" for rid, _, q in wants) + "; free pages per group: " + ", ".join(
+                str(g.pool.num_free) for g in self.groups))
+        points = self._release_points(wants)
+        for rid, nc, _ in wants:
+            self.issued[rid] = min(self.issued[rid], nc)    # its queries from nc on are still to come
+        for g in self.groups:
+            if g.need.window is not None:
+                for rid, at in points.items():
+                    self._poison(g, g.release_window(rid, at))
+            for rid, nc, q in wants:
+                g.extend(rid, nc + q)
+
+    def reserve(self, rid: Hashable, num_computed: int, q_len: int) -> None:
+        """`reserve_all` for one request."""
+        self.reserve_all([(rid, num_computed, q_len)])
 
     def free(self, rid: Hashable) -> None:
         """Gives back everything the request holds."""
         slot = self.requests.pop(rid)
         del self.admission[rid]
+        del self.issued[rid]
         for g in self.groups:
             self._poison(g, g.remove(rid))
         self.slots.give_back(slot)

@@ -175,11 +175,10 @@ class Scheduler:
         # 3. admission, in order of arrival, while a slot is free and the free pages hold the whole request
         while self.waiting and budget >= 1 and self.cache.has_slot() and not out.preempted:
             r = self.waiting[0]
+            if not self.cache.can_hold(r.num_tokens, self.budget):
+                break
             self.cache.admit(r.request_id)
             n = min(r.num_tokens, budget)
-            if not self.cache.can_reserve([(r.request_id, 0, r.num_tokens)]):
-                self.cache.free(r.request_id)
-                break
             self.waiting.popleft()
             r.status = Status.RUNNING
             self.running.append(r)

@@ -118,6 +118,72 @@ def test_windowed_group_holds_a_window_only():
     assert all(g.pool.num_free == 100 for g in m.groups)
 
 
+def test_windowed_group_has_a_pool_of_its_own_size():
+    """A windowed group's pool holds what its requests can hold at once (the reference sizes its local pool by the
+    window: simply/utils/ragged_paged_attention.py:95-110, simply/serving/page_server.py:180-196), not what the
+    group that keeps every key needs; and a long request still runs in it, portion by portion."""
+    from simply_amd.cache.manager import windowed_pool_pages
+    W, P, slots, step = 64, 16, 3, 128
+    m = CacheManager([(PagedKVNeed(1, 2, W), None), (GLOBAL, None)], page_size=P, num_pages=3 * 512, num_slots=slots,
+                     max_seq_len=8192, max_step_tokens=step)
+    assert m.groups[1].pool.num_pages == 3 * 512
+    assert m.groups[0].pool.num_pages == windowed_pool_pages(W, P, slots, step) == 3 * (4 + 2) + 8
+    # the group that keeps every key could hold each of three requests of 8192 tokens; the windowed pool is tight
+    rng = np.random.default_rng(0)
+    done = {r: 0 for r in "abc"}
+    for r in done:
+        assert m.can_hold(8192, step)
+        m.admit(r)
+    most = 0
+    while any(n < 8192 for n in done.values()):
+        # a step: every request brings something, together at most `step` tokens, cut anywhere
+        left = step
+        wants = []
+        for r in sorted(done, key=lambda _: rng.random()):
+            q = min(int(rng.integers(1, 100)), left, 8192 - done[r])
+            if q > 0:
+                wants.append((r, done[r], q))
+                left -= q
+        m.reserve_all(wants)                      # never short of pages
+        for r, start, q in wants:
+            m.check_readable(0, r, start, q)
+            done[r] += q
+        for r in done:                            # a request that the step left out can go on where it stands
+            m.check_readable(0, r, done[r], 0)
+        m.mark_issued(wants)                      # the step has been handed to the GPU
+        most = max(most, m.groups[0].pool.num_pages - m.groups[0].pool.num_free)
+        m.check()
+    assert most <= m.groups[0].pool.num_pages and most >= 3 * 4
+    # a function may give a group another size
+    m2 = CacheManager([(PagedKVNeed(1, 2, W), None), (GLOBAL, None)], page_size=P, num_pages=100, num_slots=2,
+                      max_seq_len=512, group_pages=lambda need, pages: 7 if need.window else pages)
+    assert [g.pool.num_pages for g in m2.groups] == [7, 100]
+
+
+def test_a_steps_reservations_give_back_before_they_take():
+    """Two requests in one step, no free page: the first needs two new pages, the second's window gives two back.
+    Whichever comes first in the list, the step fits; and when it does not fit, nothing has changed."""
+    W, P = 4, 2
+    for order in (("a", "b"), ("b", "a")):
+        m = manager([PagedKVNeed(1, 2, W)], P, 8, slots=2)
+        m.admit("a")
+        m.admit("b")
+        m.reserve("a", 0, 4)           # a: blocks 0, 1
+        m.reserve("b", 0, 12)          # b: all of its 12 tokens in one step, blocks 0..5
+        assert m.groups[0].pool.num_free == 0
+        wants = {"a": ("a", 4, 4), "b": ("b", 12, 1)}   # a: two new pages; b: blocks 0..3 are dead at position 12, one new
+        assert m.can_reserve([wants[r] for r in order])
+        m.reserve_all([wants[r] for r in order])
+        m.check()
+        assert len(m.groups[0].pages_of("a")) == 4 and len(m.groups[0].pages_of("b")) == 3
+        assert m.groups[0].pool.num_free == 1
+        # one more page than there is: refused, nothing changed
+        before = m.groups[0].table.copy(), m.groups[0].pool.free_list()
+        with pytest.raises(OutOfPages):
+            m.reserve_all([("a", 8, 10), ("b", 13, 1)])     # five new pages, four to be had
+        assert (before[0] == m.groups[0].table).all() and before[1] == m.groups[0].pool.free_list()
+
+
 def test_errors():
     pool = PagePool(3)
     pages = pool.take(2)

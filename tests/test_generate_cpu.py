@@ -34,6 +34,31 @@ def test_greedy_generation_matches_plain(tmp_path, cpu_ops):
     assert all(g.pool.num_free == 11 for g in small.executor.cache.groups)
 
 
+def test_windowed_layers_have_a_smaller_pool(tmp_path, cpu_ops):
+    """Prompts much longer than the window, in portions of 16: the windowed layers' pool holds a window and a portion
+    per request (simply/utils/ragged_paged_attention.py:95-110), a third of what the other layers' pool holds, and
+    generation equals the plain implementation's."""
+    d = tiny.write_model("A", str(tmp_path / "A"), std=0.5)      # window 8
+    w, cfg = plain.load(d)
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 90 + n) for n in (90, 61, 75)]
+    want = [plain.greedy(w, cfg, p, 6) for p in prompts]
+    m = lm(d, max_seq_len=128)
+    windowed, rest = sorted(m.executor.cache.groups, key=lambda g: g.need.window is None)
+    assert windowed.need.window == 8 and rest.need.window is None
+    assert rest.pool.num_pages == 3 * 32 and windowed.pool.num_pages == 3 * (2 + 2) + 4
+    most = 0
+    for i, p in enumerate(prompts):
+        m.add_request(i, p, SamplingParams(temperature=0.0, max_decode_steps=6))
+    done = []
+    while m.scheduler.has_work():
+        done += m.step()
+        most = max(most, windowed.pool.num_pages - windowed.pool.num_free)
+        m.executor.cache.check()
+    assert [r.output_token_ids for r in sorted(done, key=lambda r: r.request_id)] == want
+    assert m.stats["preemptions"] == 0 and 6 <= most <= windowed.pool.num_pages
+    assert windowed.pool.num_free == windowed.pool.num_pages
+
+
 def test_sampled_tokens_do_not_depend_on_the_batch(tmp_path, cpu_ops):
     d = tiny.write_model("B", str(tmp_path / "B"), std=0.1)
     _, cfg = plain.load(d)
