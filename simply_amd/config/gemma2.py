@@ -226,6 +226,8 @@ class Gemma2Config:
             max_position=self.max_position_embeddings,
             eos_token_ids=self.eos_token_ids,
             initializer_range=self.initializer_range,
+            # a folder of a tied model may store the head once more under its own name
+            copies={"lm_head.weight": "model.embed_tokens.weight"} if self.tie_word_embeddings else {},
         )
         spec.validate()
         return spec

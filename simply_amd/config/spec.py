@@ -57,6 +57,9 @@ class ModelSpec:
     max_position: int
     eos_token_ids: tuple[int, ...] = ()
     initializer_range: float = 0.02
+    #: tensor names that a model folder may hold beside the expected ones, each with the expected tensor whose
+    #: copy it must be (a tied head stored once more under its own name): checked for equality, then left unread
+    copies: Mapping[str, str] = dataclasses.field(default_factory=dict)
 
     def validate(self) -> None:
         n = len(self.layers)
@@ -70,3 +73,6 @@ class ModelSpec:
                 if self.schedule[e.cache_from].cache_from is not None:
                     raise ValueError(
                         f"schedule entry {i} reads the cache of entry {e.cache_from}, which itself has none")
+        for name, of in self.copies.items():
+            if name == of:
+                raise ValueError(f"tensor {name!r} is declared a copy of itself")

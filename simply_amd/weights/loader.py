@@ -2,8 +2,12 @@
 
 The reference restores an Orbax tree and renames keys per checkpoint format
 (simply/utils/checkpoint_lib.py:690-773); a shape mismatch is an error there
-(:754-758), a missing tensor only a warning (:769-773).  Here missing tensors,
-unexpected tensors and wrong shapes are all errors, reported together.
+(:754-758), a missing tensor only a warning (:769-773), an unknown stored key is
+ignored with a warning (:333).  Here missing tensors, unexpected tensors and wrong
+shapes are all errors, reported together; one kind of extra tensor is allowed by
+rule: a name that the model declares a copy of an expected tensor (the head of a
+model with a tied head, stored once more as `lm_head.weight`) must equal that
+tensor bit for bit and is then left unread.
 
 Element types: floating tensors of role 'matrix' are held in the activation dtype
 (wider parameters are cast down as simply/model_lib.py:2986-2998 does); 'vector'
@@ -66,11 +70,17 @@ def target_dtype(stored: torch.dtype, spec: ParamSpec, activation_dtype: torch.d
     return activation_dtype
 
 
-def check_names_and_shapes(where: str, expected: Mapping[str, ParamSpec], found: Mapping[str, tuple]) -> None:
+def check_names_and_shapes(where: str, expected: Mapping[str, ParamSpec], found: Mapping[str, tuple],
+                           copies: Mapping[str, str] | None = None) -> None:
+    """copies: stored name -> expected tensor that it must be a copy of; such a name is not unexpected, and its
+    shape must be that tensor's."""
+    copies = {n: of for n, of in (copies or {}).items() if of in expected and n not in expected}
     missing = [n for n in expected if n not in found]
-    unexpected = [n for n in found if n not in expected]
+    unexpected = [n for n in found if n not in expected and n not in copies]
     wrong = [(n, tuple(found[n]), tuple(expected[n].shape)) for n in expected
              if n in found and tuple(found[n]) != tuple(expected[n].shape)]
+    wrong += [(n, tuple(found[n]), tuple(expected[of].shape)) for n, of in copies.items()
+              if n in found and tuple(found[n]) != tuple(expected[of].shape)]
     if missing or unexpected or wrong:
         raise WeightsError(where, missing, unexpected, wrong)
 
@@ -95,7 +105,13 @@ def load_weights(model, model_dir: str, activation_dtype: torch.dtype, device) -
             shapes[name] = tuple(h.get_slice(name).get_shape())
     if duplicates:
         raise WeightsError(model_dir, [], [], [], [f"tensors stored in more than one file: {', '.join(duplicates)}"])
-    check_names_and_shapes(model_dir, expected, shapes)
+    copies = {n: of for n, of in getattr(model.spec, "copies", {}).items() if n in shapes and n not in expected}
+    check_names_and_shapes(model_dir, expected, shapes, copies)
+    differing = [f"{n} is stored beside {of}, of which the model makes it a copy, but the two differ"
+                 for n, of in copies.items()
+                 if not torch.equal(handles[where_of[n]].get_tensor(n), handles[where_of[of]].get_tensor(of))]
+    if differing:
+        raise WeightsError(model_dir, [], [], [], differing)
     tensors = {}
     for name, spec in expected.items():
         t = handles[where_of[name]].get_tensor(name)

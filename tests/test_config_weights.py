@@ -127,6 +127,34 @@ def test_weight_errors_list_everything(tmp_path):
         assert name in msg
 
 
+def test_tied_head_stored_once_more(tmp_path):
+    """A folder of a model with a tied head that also stores `lm_head.weight`: allowed if it equals the embedding
+    table (it is then left unread), refused if it differs or has another shape; in a model without the rule it is
+    an unexpected tensor like any other."""
+    d = tiny.write_model("A", str(tmp_path / "A"))
+    path = os.path.join(d, "model.safetensors")
+    t = load_file(path)
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    save_file(t, path)
+    model = DecoderModel(load_config(d).model_spec())
+    load_weights(model, d, torch.float32, "cpu")
+    assert model.head.weight is model.embedding.table
+    t["lm_head.weight"][3, 5] += 1.0
+    save_file(t, path)
+    with pytest.raises(WeightsError, match="lm_head.weight is stored beside model.embed_tokens.weight"):
+        load_weights(model, d, torch.float32, "cpu")
+    t["lm_head.weight"] = torch.zeros(7, 64)
+    save_file(t, path)
+    with pytest.raises(WeightsError) as e:
+        load_weights(model, d, torch.float32, "cpu")
+    assert e.value.wrong_shape == [("lm_head.weight", (7, 64), (256, 64))] and not e.value.unexpected
+    import dataclasses
+    no_rule = DecoderModel(dataclasses.replace(load_config(d).model_spec(), copies={}))
+    with pytest.raises(WeightsError) as e:
+        load_weights(no_rule, d, torch.float32, "cpu")
+    assert e.value.unexpected == ["lm_head.weight"]
+
+
 def test_missing_files(tmp_path):
     with pytest.raises(FileNotFoundError, match="config.json"):
         load_config(str(tmp_path))
@@ -158,3 +186,147 @@ def test_element_types():
     assert target_dtype(f32, v, bf) == f32 and target_dtype(bf, v, bf) == bf      # a 32-bit stored vector stays so
     assert target_dtype(bf, m, f32) == f32 and target_dtype(bf, v, f32) == f32    # the 32-bit path holds 32-bit
     assert target_dtype(torch.int64, tb, bf) == torch.int32 and target_dtype(torch.int32, m, f32) == torch.int32
+
+
+# ------------------------------------------------------------------ which axis goes where
+REFERENCE_TESTDATA = "/root/reference/simply/utils/testdata"
+
+
+def _tree(path):
+    import json
+
+    def arrays(x):
+        if not isinstance(x, dict):
+            return torch.tensor(x, dtype=torch.float64)
+        out = {}
+        for key, v in x.items():          # a key may be a path ("transformer/layer_0/attn")
+            at = out
+            *parents, last = key.split("/")
+            for part in parents:
+                at = at.setdefault(part, {})
+            at[last] = arrays(v)
+        return out
+
+    with open(path) as f:
+        return arrays(json.load(f))
+
+
+def flax_params_to_simply(params: dict) -> dict:
+    """The Gemma parameter tree in the reference's own layout, by the rules of
+    simply/utils/checkpoint_lib.py:256-335 (written out here for the parameters; the reference's test applies the
+    same rules to the optimizer's trees)."""
+    t = params["transformer"]
+    out = {"embed_linear": {"w": t["embedder"]["input_embedding"]}, "final_ln": {"scale": t["final_norm"]["scale"]}}
+    ln = {"pre_attention_norm": "pre_ln_0", "pre_ffw_norm": "pre_ln_1", "post_attention_norm": "post_ln_0",
+          "post_ffw_norm": "post_ln_1"}                                                  # :249-254
+    for name, layer in t.items():
+        if not name.startswith("layer_"):
+            continue
+        qkv = torch.einsum("kndh->kdnh", layer["attn"]["qkv_einsum"]["w"])             # :272-277, then split in three
+        block = {"attn": {"q_proj": {"w": qkv[0]}, "k_proj": {"w": qkv[1]}, "v_proj": {"w": qkv[2]},
+                          "o_proj": {"w": torch.einsum("nhd->dnh", layer["attn"]["attn_vec_einsum"]["w"])}},   # :283-287
+                 "ffn": {"ffn_0_gate": {"w": layer["mlp"]["gating_einsum"]["w"][0], "b": layer["mlp"]["gating_einsum"]["b"][0]},
+                         "ffn_0": {"w": layer["mlp"]["gating_einsum"]["w"][1], "b": layer["mlp"]["gating_einsum"]["b"][1]},
+                         "ffn_1": {"w": layer["mlp"]["linear"]["w"], "b": layer["mlp"]["linear"]["b"]}}}        # :300-323
+        for theirs, ours in ln.items():
+            block[ours] = {"scale": layer[theirs]["scale"]}
+        out["block_" + name[len("layer_"):]] = block
+    return out
+
+
+def simply_params_to_folder(params: dict) -> dict:
+    """The model folder's tensors ([out_features, in_features], heads flattened head-major) from the reference's
+    layout: the inverse of the rules by which the reference reads such a folder
+    (simply/utils/checkpoint_lib.py:432-458: q/k/v `nhd->dnh` of the rows split into heads, o the columns split into
+    heads, the feed-forward matrices transposed).  The names of the four norms are the folder's Gemma 2 names in the
+    roles that simply/utils/checkpoint_lib.py:249-254 gives their Flax counterparts; no file of the reference names
+    the Gemma 2 folder's norms, so that part of the mapping is not pinned by it."""
+    out = {"model.embed_tokens.weight": params["embed_linear"]["w"], "model.norm.weight": params["final_ln"]["scale"]}
+    norms = {"pre_ln_0": "input_layernorm", "post_ln_0": "post_attention_layernorm",
+             "pre_ln_1": "pre_feedforward_layernorm", "post_ln_1": "post_feedforward_layernorm"}
+    for name, b in params.items():
+        if not name.startswith("block_"):
+            continue
+        p = f"model.layers.{name[len('block_'):]}."
+        for proj in ("q_proj", "k_proj", "v_proj"):
+            w = b["attn"][proj]["w"]                                                     # [d, n, h]
+            out[p + f"self_attn.{proj}.weight"] = torch.einsum("dnh->nhd", w).reshape(-1, w.shape[0])
+        w = b["attn"]["o_proj"]["w"]
+        out[p + "self_attn.o_proj.weight"] = w.reshape(w.shape[0], -1)
+        out[p + "mlp.gate_proj.weight"] = b["ffn"]["ffn_0_gate"]["w"].T
+        out[p + "mlp.up_proj.weight"] = b["ffn"]["ffn_0"]["w"].T
+        out[p + "mlp.down_proj.weight"] = b["ffn"]["ffn_1"]["w"].T
+        for ours, theirs in norms.items():
+            out[p + theirs + ".weight"] = b[ours]["scale"]
+    return out
+
+
+def test_axis_order_against_the_reference_fixtures():
+    """The reference holds one pair of files that says which axis of a Gemma tensor goes where: arange-filled trees
+    before and after its own conversion (simply/utils/testdata/ckpt_gemma2_format.json ->
+    ckpt_expected_format.json, compared by simply/utils/checkpoint_lib_test.py).  The rules as read here reproduce
+    the second file from the first; the folder layout derived from them names the tensors that the model expects,
+    with its shapes; and the plain implementation's products on that layout equal the reference's einsums on its
+    own (`ihd,...i->...hd`, `ihd,...hd->...i`, `io,...i->...o`: simply/model_lib.py:2047-2068, :671-694), so that a
+    transposed matrix or heads flattened the other way round would show."""
+    if not os.path.isdir(REFERENCE_TESTDATA):
+        pytest.skip("the reference's test data is not mounted")
+    flax = _tree(os.path.join(REFERENCE_TESTDATA, "ckpt_gemma2_format.json"))
+    expected = _tree(os.path.join(REFERENCE_TESTDATA, "ckpt_expected_format.json"))
+    simply = flax_params_to_simply(flax["params"])
+
+    def same(a, b, path=""):
+        if isinstance(b, dict):
+            assert set(a) == set(b), (path, sorted(a), sorted(b))
+            for k in b:
+                same(a[k], b[k], path + "/" + k)
+        else:
+            assert torch.equal(a, b), path
+
+    same(simply, expected["params"])
+    # the folder: names and shapes are the model's (2 layers, width 4, 2 heads of size 4, feed-forward 8, 2 tokens)
+    folder = simply_params_to_folder(simply)
+    d = dict(tiny.TINY_A, hidden_size=4, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=2, head_dim=4,
+             intermediate_size=8, vocab_size=2)
+    # (the engine's attention wants head sizes in steps of 16; names and shapes do not depend on that)
+    import dataclasses
+    spec = config_from_dict(dict(d, head_dim=16)).model_spec()
+    names = set()
+    for layer in spec.layers:
+        names |= set(layer.mixer.tensors.values()) | set(layer.feed_forward.tensors.values())
+        names |= {n.tensors["scale"] for n in layer.norms.values()}
+    names |= {spec.embedding.tensors["table"], spec.final_norm.tensors["scale"]}
+    assert names == set(folder)
+    assert folder["model.layers.0.self_attn.q_proj.weight"].shape == (8, 4)
+    assert folder["model.layers.0.self_attn.o_proj.weight"].shape == (4, 8)
+    assert folder["model.layers.1.mlp.down_proj.weight"].shape == (4, 8)
+    # the plain implementation on the folder's layout against the reference's einsums on the reference's layout
+    x = torch.randn(5, 4, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
+    b = simply["block_1"]
+    p = "model.layers.1."
+    for proj in ("q_proj", "k_proj", "v_proj"):
+        want = torch.einsum("ihd,ti->thd", b["attn"][proj]["w"], x)
+        got = (x @ folder[p + f"self_attn.{proj}.weight"].T).reshape(5, 2, 4)       # as plain.attention_layer does
+        torch.testing.assert_close(got, want)
+    heads = torch.randn(5, 2, 4, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
+    torch.testing.assert_close(heads.reshape(5, 8) @ folder[p + "self_attn.o_proj.weight"].T,
+                               torch.einsum("ihd,thd->ti", b["attn"]["o_proj"]["w"], heads))
+    import plain_gemma2 as plain
+    gate = torch.einsum("io,ti->to", b["ffn"]["ffn_0_gate"]["w"], x * 1e-3)
+    up = torch.einsum("io,ti->to", b["ffn"]["ffn_0"]["w"], x * 1e-3)
+    want = torch.einsum("io,ti->to", b["ffn"]["ffn_1"]["w"], plain.gelu_tanh(gate) * up)   # simply/model_lib.py:714-730
+    torch.testing.assert_close(plain.feed_forward(x * 1e-3, folder, p + "mlp."), want)
+    # the roles of the norms: the block of the plain implementation with the folder's names equals the block written
+    # with the reference's names in the reference's order (simply/model_lib.py:2669-2703)
+    cfg = dict(d, rms_norm_eps=1e-6, query_pre_attn_scalar=4, attn_logit_softcapping=None, sliding_window=None)
+    small = {k: v * 1e-3 for k, v in folder.items()}
+    pos = torch.arange(5)
+    h = x
+    y = plain.rms_norm(x, small[p + "input_layernorm.weight"], 1e-6)
+    y = plain.attention_layer(y, pos, small, p + "self_attn.", cfg, None)
+    y = plain.rms_norm(y, b["post_ln_0"]["scale"] * 1e-3, 1e-6)
+    x1 = y + h
+    y = plain.rms_norm(x1, b["pre_ln_1"]["scale"] * 1e-3, 1e-6)
+    y = plain.feed_forward(y, small, p + "mlp.")
+    y = plain.rms_norm(y, b["post_ln_1"]["scale"] * 1e-3, 1e-6)
+    torch.testing.assert_close(plain.block(x, pos, small, 1, cfg, None), y + x1)
