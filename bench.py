@@ -72,18 +72,63 @@ def sync():
     torch.cuda.synchronize()
 
 
-def run_decode(model, cfg, batch, context, steps, warmup, page_size, dtype):
-    """Returns (seconds per step, mean kv length over the timed steps)."""
+def fill_cache_random(lm, std: float = 0.5, seed: int = 0) -> None:
+    """Fills every page of keys and values with N(0, std), so that decode steps over a long context can be timed
+    without running the prompts that would have written them."""
     import torch
-    from simply_amd.engine.llm import LMInterface, fill_cache_random, preload
+    gen = torch.Generator(device=lm.executor.device)
+    gen.manual_seed(seed)
+    for v in lm.executor.cache.views:
+        if v.k_pages is not None and v.write:
+            for t in (v.k_pages, v.v_pages):
+                flat = t.view(-1)     # in slices, so that no float32 copy of a whole pool is made
+                step = 1 << 26
+                for i in range(0, flat.numel(), step):
+                    n = min(step, flat.numel() - i)
+                    flat[i:i + n] = (torch.randn(n, generator=gen, device=t.device, dtype=torch.float32) * std).to(t.dtype)
+
+
+def preload(lm, request_id, prompt_token_ids, params):
+    """Admits a request as if all of its prompt but the last token had been run, in portions of the engine's token
+    budget: its pages are reserved and given back as that run would have done (a windowed layer ends up holding its
+    window only) and hold what `fill_cache_random` put there, so the next steps are decode steps at the prompt's
+    length."""
+    from simply_amd.engine.scheduler import Status
+    r = lm.add_request(request_id, prompt_token_ids, params)
+    sched, cache = lm.scheduler, lm.executor.cache
+    sched.waiting.remove(r)
+    cache.admit(r.request_id)
+    n = r.num_tokens - 1
+    for at in range(0, n, sched.budget):
+        q = min(sched.budget, n - at)
+        cache.reserve(r.request_id, at, q)
+        cache.mark_issued([(r.request_id, at, q)])
+    lm.executor.num_computed[r.request_id] = (cache.admission[r.request_id], n)
+    r.num_computed = n
+    r.status = Status.RUNNING
+    sched.running.append(r)
+    return r
+
+
+def percentile(values, p):
+    v = sorted(values)
+    return v[min(len(v) - 1, int(round(p / 100.0 * (len(v) - 1))))]
+
+
+def run_decode(model, cfg, batch, context, steps, warmup, page_size, dtype, latency_steps=0):
+    """Returns (seconds per step, mean kv length over the timed steps, latencies): `steps` decode steps as the engine
+    runs them when nobody waits (several in a row on the device), then `latency_steps` more one at a time, the host
+    reading each step's tokens before the next: their seconds are the latencies."""
+    import torch
+    from simply_amd.engine.llm import LMInterface
     from simply_amd.sampling import SamplingParams
 
-    max_len = context + steps + warmup + 8
+    max_len = context + steps + warmup + latency_steps + 8
     lm = LMInterface(config=cfg, random_weights=0, activation_dtype=dtype, batch_size=batch, max_seq_len=max_len,
-                     page_size=page_size, max_num_issue_tokens=max(batch, 16), _model=model)
+                     page_size=page_size, max_num_issue_tokens=2048, _model=model)
     fill_cache_random(lm)
     g = torch.Generator().manual_seed(1)
-    params = SamplingParams(temperature=0.0, max_decode_steps=steps + warmup + 4, ignore_eos=True)
+    params = SamplingParams(temperature=0.0, max_decode_steps=steps + warmup + latency_steps + 4, ignore_eos=True)
     for i in range(batch):
         prompt = torch.randint(0, cfg.vocab_size, (context,), generator=g).tolist()
         preload(lm, f"b{i}", prompt, params)
@@ -102,18 +147,27 @@ def run_decode(model, cfg, batch, context, steps, warmup, page_size, dtype):
     first = context + warmup          # kv length seen by the first timed step
     mean_kv = first + (steps - 1) / 2
     assert all(len(r.output_token_ids) == warmup + steps for r in lm.scheduler.running)
+    latencies = []
+    if latency_steps:
+        lm.step(max_decode_steps=1)   # the single-step graph is recorded outside the timed steps
+        lm.step_log = []
+        for _ in range(latency_steps - 1):
+            lm.step(max_decode_steps=1)
+        latencies = [sec for _, _, sec in lm.step_log]
     del lm
     torch.cuda.empty_cache()
-    return dt, mean_kv
+    return dt, mean_kv, latencies
 
 
-def run_prefill(model, cfg, tokens, reps, page_size, dtype):
+def run_prefill(model, cfg, tokens, reps, page_size, dtype, portion=None):
+    """Seconds for a prompt of `tokens` tokens and its first sampled token: in one step, or in portions of `portion`
+    tokens (the scheduler cuts it under that token budget)."""
     import torch
     from simply_amd.engine.llm import LMInterface
     from simply_amd.sampling import SamplingParams
 
     lm = LMInterface(config=cfg, random_weights=0, activation_dtype=dtype, batch_size=1, max_seq_len=tokens + 8,
-                     page_size=page_size, max_num_issue_tokens=tokens, _model=model)
+                     page_size=page_size, max_num_issue_tokens=portion or tokens, _model=model)
     g = torch.Generator().manual_seed(2)
     params = SamplingParams(temperature=0.0, max_decode_steps=1, ignore_eos=True)
     times = []
@@ -121,9 +175,11 @@ def run_prefill(model, cfg, tokens, reps, page_size, dtype):
         prompt = torch.randint(0, cfg.vocab_size, (tokens,), generator=g).tolist()
         sync()
         t0 = time.perf_counter()
-        lm.generate(prompt, sampling_params=params)   # one step: the whole prompt, then one sampled token
+        steps_before = lm.stats["steps"]
+        lm.generate(prompt, sampling_params=params)   # the whole prompt, then one sampled token
         sync()
         times.append(time.perf_counter() - t0)
+        assert lm.stats["steps"] - steps_before == -(-tokens // (portion or tokens))
     del lm
     torch.cuda.empty_cache()
     return min(times[1:])
@@ -145,12 +201,26 @@ def run_requests(model, cfg, requests, prompt_min, prompt_max, new_tokens, page_
     lm.generate(prompts[:2], sampling_params=SamplingParams(temperature=0.0, max_decode_steps=4, ignore_eos=True))
     sync()
     before = dict(lm.stats)
+    lm.step_log = []
     t0 = time.perf_counter()
     outs = lm.generate(prompts, sampling_params=params)
     sync()
     dt = time.perf_counter() - t0
     assert all(len(o.output_token_ids) == new_tokens for o in outs)
     stats = {k: lm.stats[k] - before.get(k, 0) for k in lm.stats if isinstance(lm.stats[k], (int, float))}
+    # steps that ran a portion of some prompt (beside decoded tokens of others) against steps that only decoded
+    log = lm.step_log
+    stats["prompt_step_seconds"] = sum(sec for n, _, sec in log if n == 0)
+    stats["decode_step_seconds"] = sum(sec for n, _, sec in log if n > 0)
+    stats["prompt_steps"] = sum(1 for n, _, _ in log if n == 0)
+    stats["decode_steps"] = sum(n for n, _, _ in log if n > 0)
+    stats["prompt_step_tokens"] = sum(t for n, t, _ in log if n == 0)
+    per_decode_step = [sec / n for n, _, sec in log if n > 0]
+    stats["decode_step_ms_p50"] = 1e3 * percentile(per_decode_step, 50) if per_decode_step else None
+    stats["decode_step_ms_p99"] = 1e3 * percentile(per_decode_step, 99) if per_decode_step else None
+    prompt_steps = [sec for n, _, sec in log if n == 0]
+    stats["prompt_step_ms_p50"] = 1e3 * percentile(prompt_steps, 50) if prompt_steps else None
+    stats["prompt_step_ms_p99"] = 1e3 * percentile(prompt_steps, 99) if prompt_steps else None
     del lm
     torch.cuda.empty_cache()
     return dt, sum(lengths), requests * new_tokens, stats
@@ -168,6 +238,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--latency-steps", type=int, default=100,
+                    help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
     ap.add_argument("--requests", type=int, default=0,
                     help="instead of timed decode steps: a workload of this many requests through the scheduler")
@@ -202,6 +274,12 @@ def main():
             "value": round((prompt_tokens + new_tokens) / dt, 1), "unit": "tokens/s", "n_gpus": 1,
             "generated_per_s": round(new_tokens / dt, 1), "seconds": round(dt, 3), "prompt_tokens": prompt_tokens,
             "generated_tokens": new_tokens, "engine_steps": stats.get("steps"), "higher_is_better": True,
+            "phases": {"prompt_steps": stats["prompt_steps"], "prompt_step_seconds": round(stats["prompt_step_seconds"], 3),
+                       "prompt_step_tokens": stats["prompt_step_tokens"], "decode_steps": stats["decode_steps"],
+                       "decode_step_seconds": round(stats["decode_step_seconds"], 3)},
+            "latency_ms": {f"{k}_{q}": (round(stats[f"{k}_ms_{q}"], 3) if stats[f"{k}_ms_{q}"] else None)
+                           for k in ("decode_step", "prompt_step") for q in ("p50", "p99")},
+            "preemptions": stats.get("preemptions"),
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
             "config": {"model": f"gemma2-{args.shape}-shape", "layers": cfg.num_hidden_layers,
                        "layers_of_full_model": full_layers, "requests": args.requests, "prompt_min": args.prompt_min,
@@ -209,7 +287,8 @@ def main():
               flush=True)
         return
 
-    dt, mean_kv = run_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, args.page_size, args.dtype)
+    dt, mean_kv, latencies = run_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, args.page_size,
+                                        args.dtype, latency_steps=args.latency_steps)
     step_bytes = weight_bytes(cfg, esize) + args.batch * kv_bytes_per_request(cfg, mean_kv, esize)
     achieved = step_bytes / dt / 1e9
 
@@ -218,12 +297,16 @@ def main():
     peak = PEAK_TFLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
     prefill = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
                "frac": round(prefill_flops(cfg, T) / pt / 1e12 / peak, 4)}
+    # the same prompt in four portions, as it runs beside other requests under a token budget of a quarter of it
+    pc = run_prefill(model, cfg, T, 3, args.page_size, args.dtype, portion=-(-T // 4))
+    prefill_chunked = {"value": round(T / pc, 1), "tokens": T, "portions": 4, "ms": round(pc * 1e3, 3),
+                       "frac": round(prefill_flops(cfg, T) / pc / 1e12 / peak, 4)}
 
     points = {}
     if not args.no_points:
         for b in (1, 64):
             steps_b = max(10, min(args.steps, 30))
-            dtb, _ = run_decode(model, cfg, b, args.context, steps_b, 8, args.page_size, args.dtype)
+            dtb, _, _ = run_decode(model, cfg, b, args.context, steps_b, 8, args.page_size, args.dtype)
             points[f"decode_b{b}"] = round(b / dtb, 1)
 
     out = {
@@ -239,6 +322,10 @@ def main():
                    "page_size": args.page_size, "prefill_tokens": T, "weights": "random N(0,0.02)",
                    "parallelism": "single-gpu"},
         "prefill": prefill,
+        "prefill_chunked": prefill_chunked,
+        "step_latency_ms": {"p50": round(1e3 * percentile(latencies, 50), 4), "p99": round(1e3 * percentile(latencies, 99), 4),
+                            "steps": len(latencies), "what": "one decode step at a time, tokens read by the host"}
+        if latencies else None,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,

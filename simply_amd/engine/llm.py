@@ -89,6 +89,9 @@ class LMInterface:
         self._num_requests = 0
         self._num_scored = 0
         self.stats = {"steps": 0, "tokens": 0, "preemptions": 0, "seconds": 0.0}
+        #: set to a list to have every call of `step` add (decode steps it ran or 0 for a step with a portion of a
+        #: prompt, tokens, seconds): the host has the step's tokens when the call returns, so these are latencies
+        self.step_log: list[tuple[int, int, float]] | None = None
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request_id, prompt_token_ids: Sequence[int], params: SamplingParams | None = None) -> Request:
@@ -107,6 +110,7 @@ class LMInterface:
         """One scheduling decision and one run of the step function; when every scheduled request is decoding and
         nothing waits for admission, up to `intermediate_steps` (and `max_decode_steps`) decode steps in a row
         without the host in between.  Returns the requests that finished."""
+        t0 = time.perf_counter()
         out = self.scheduler.schedule()
         self.stats["preemptions"] += len(out.preempted)
         finished = list(out.finished)
@@ -133,6 +137,8 @@ class LMInterface:
                 self.stats["tokens"] += len(now)
                 if not live:
                     break
+            if self.step_log is not None:
+                self.step_log.append((n, n * len(entries), time.perf_counter() - t0))
             return finished
         logits = self.executor.step(entries)
         tokens: list = [None] * len(entries)
@@ -147,6 +153,10 @@ class LMInterface:
         finished += self.scheduler.update(out.scheduled, tokens, logprobs)
         self.stats["steps"] += 1
         self.stats["tokens"] += out.num_tokens
+        if self.step_log is not None:
+            # a decode step: every token that went in is one that the model had generated
+            decode_only = all(s.start >= len(s.request.prompt_token_ids) for s in out.scheduled)
+            self.step_log.append((1 if decode_only else 0, out.num_tokens, time.perf_counter() - t0))
         return finished
 
     def _decode_steps_ahead(self, scheduled, max_decode_steps: int | None) -> int:
@@ -229,41 +239,3 @@ class LMInterface:
 
 
 LLM = LMInterface
-
-
-def preload(lm: LMInterface, request_id, prompt_token_ids: Sequence[int], params: SamplingParams, *,
-            seed: int = 0) -> Request:
-    """For measurements: admits a request as if all of its prompt but the last token had been run.  Its
-    pages are reserved as a run would have reserved them and hold what `fill_cache_random` put there, so
-    the next steps are decode steps at the prompt's length without the cost of a real prefill."""
-    from .scheduler import Status
-
-    r = lm.add_request(request_id, prompt_token_ids, params)
-    sched, cache = lm.scheduler, lm.executor.cache
-    sched.waiting.remove(r)
-    cache.admit(r.request_id)
-    n = r.num_tokens - 1
-    if n > 0:
-        cache.reserve(r.request_id, 0, n)
-        # what a windowed group would have given back on the way
-        cache.reserve(r.request_id, n, 0)
-        lm.executor.num_computed[r.request_id] = (cache.admission[r.request_id], n)
-    r.num_computed = n
-    r.status = Status.RUNNING
-    sched.running.append(r)
-    return r
-
-
-def fill_cache_random(lm: LMInterface, std: float = 0.5, seed: int = 0) -> None:
-    """For measurements: fills every page of keys and values with N(0, std)."""
-    gen = torch.Generator(device=lm.executor.device)
-    gen.manual_seed(seed)
-    for v in lm.executor.cache.views:
-        if v.k_pages is not None and v.write:
-            for t in (v.k_pages, v.v_pages):
-                # in slices, so that no float32 copy of a whole pool is made
-                flat = t.view(-1)
-                step = 1 << 26
-                for i in range(0, flat.numel(), step):
-                    n = min(step, flat.numel() - i)
-                    flat[i:i + n] = (torch.randn(n, generator=gen, device=t.device, dtype=torch.float32) * std).to(t.dtype)

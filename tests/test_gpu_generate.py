@@ -40,7 +40,7 @@ def test_greedy_matches_plain(tmp_path, gpu_lib, dtype):
 
 
 def test_sampling_is_per_request(tmp_path, gpu_lib):
-    """BASELINE workload of the second tiny configuration: prompts of 1, 9, 23 and 40 tokens, pages of 4,
+    """The workload of the second tiny configuration: prompts of 1, 9, 23 and 40 tokens, pages of 4,
     mixed portions and decoding, temperature 0.7."""
     d = tiny.write_model("B", str(tmp_path / "B"), dtype=torch.float32, std=0.1)
     _, cfg = plain.load(d)
