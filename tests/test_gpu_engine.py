@@ -41,7 +41,7 @@ def run_cut(ex, rid, tokens, cuts):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "U"])
 def test_cuts_match_plain(tmp_path, name, dtype):
     d = tiny.write_model(name, str(tmp_path / name), std=0.3)
     vocab = plain.load(d)[1]["vocab_size"]

@@ -38,7 +38,10 @@ TINY_D = dict(
     final_logit_softcapping=30.0, tie_word_embeddings=True, max_position_embeddings=1024,
     hidden_activation="gelu_pytorch_tanh", initializer_range=0.05,
 )
-CONFIGS = {"A": (TINY_A, 0, 0.1), "B": (TINY_B, 1, 0.2), "C": (TINY_C, 2, 0.3), "D": (TINY_D, 3, 0.1)}
+# the first one with a head of its own (a random head gives continuations that do not repeat one token)
+TINY_U = dict(TINY_A, tie_word_embeddings=False)
+CONFIGS = {"A": (TINY_A, 0, 0.1), "B": (TINY_B, 1, 0.2), "C": (TINY_C, 2, 0.3), "D": (TINY_D, 3, 0.1),
+           "U": (TINY_U, 4, 0.1)}
 
 
 def write_model(name: str, out_dir: str, dtype=torch.float32, std: float | None = None) -> str:
