@@ -28,6 +28,9 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace sa {
 
+// Sub-tiles of 16 keys whose page a workgroup looks up once, into LDS, before its loop: 32768 keys.
+constexpr int kMaxRangeSubTiles = 2048;
+
 __device__ inline float fast_tanh(float x) {
   // tanh(x) = 1 - 2 / (exp(2x) + 1); exact at both ends, relative error ~1e-6 in between
   const float e = __expf(2.f * x);
@@ -45,6 +48,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   constexpr int NDB = HD / 16;  // output blocks of 16 dimensions
   __shared__ float o_s[2][16][HD + 1];   // a wave's output [row][d], while two waves are merged
   __shared__ float m_s[2][16], l_s[2][16];
+  __shared__ int2 where_s[kMaxRangeSubTiles];  // per sub-tile of this workgroup's range: its page, its block within it
 
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // the same for the whole wave: kept in a scalar register
@@ -67,6 +71,22 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   const int ntiles = tile1 - tile0;
   const int tb = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * split / num_splits);
   const int te = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * (split + 1) / num_splits);
+
+  // Where every sub-tile of 16 keys of the range lies: looked up here once, so that the loop below has no load
+  // whose address depends on another load.  (A sub-tile lies within one page: page_size is a multiple of 16.)
+  const int sub0 = 2 * tb;
+  const int nsub = 2 * (te - tb) < kMaxRangeSubTiles ? 2 * (te - tb) : kMaxRangeSubTiles;  // (the host has seen to it)
+  for (int i = tid; i < nsub; i += 256) {
+    const int key = (sub0 + i) * 16;
+    int2 w = {0, 0};
+    if (key < hi && key + 16 > lo) {
+      const int block = key / page_size;
+      w.x = table[block];
+      w.y = (key - block * page_size) / 16;
+    }
+    where_s[i] = w;
+  }
+  __syncthreads();
 
   // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
   bf16x8 qf[NDC];
@@ -96,20 +116,18 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     SubTile st;
     const int sk0 = tile * kTile + t * 16;
     st.ok = tile < te && sk0 < hi && sk0 + 16 > lo;  // wave-uniform
-    st.k = nullptr;
-    st.v = nullptr;
-    if (st.ok) {
-      const int page = table[sk0 / page_size];
-      const int off = sk0 % page_size;  // a multiple of 16
-      const size_t head = static_cast<size_t>(page) * Kh + kh;
-      // keys are stored in 16-key x 32-dimension blocks of operand order: block (off / 16, dc) is a contiguous KiB
-      st.k = k_pages + head * page_size * HD + static_cast<size_t>(off / 16) * (NDC * 512) + lane * 8;
-      st.v = v_pages + (head * HD + r) * page_size + off + grp * 4;
-    }
+    // A sub-tile outside the range is loaded all the same, from the pool's first page: every load of the loop is
+    // unconditional, the loop straight-line code, and the compiler counts the loads in flight (with a branch
+    // around a load it waits for all of them, and loads and products do not overlap).  What is loaded there is
+    // never used: its scores are masked and its values replaced by zeros.
+    const int2 w = where_s[st.ok ? 2 * tile + t - sub0 : 0];
+    const size_t head = st.ok ? static_cast<size_t>(w.x) * Kh + kh : 0;
+    const int blk = st.ok ? w.y : 0;
+    // keys are stored in 16-key x 32-dimension blocks of operand order: block (blk, dc) is a contiguous KiB
+    st.k = k_pages + head * page_size * HD + static_cast<size_t>(blk) * (NDC * 512) + lane * 8;
+    st.v = v_pages + (head * HD + r) * page_size + blk * 16 + grp * 4;
     return st;
   };
-  const bf16x8 zero8 = {};
-  const bf16x4 zero4 = {};
   struct TileRegs {
     SubTile st[2];
     bf16x8 kf[2][NDC];
@@ -122,15 +140,14 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int dc = 0; dc < NDC; ++dc)
-        b.kf[t][dc] = b.st[t].ok ? *reinterpret_cast<const bf16x8*>(b.st[t].k + dc * 512) : zero8;
+        b.kf[t][dc] = *reinterpret_cast<const bf16x8*>(b.st[t].k + dc * 512);
   };
   auto request_values = [&](TileRegs& b) {  // of the tile whose keys were requested last
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
-        b.vf[t][db] = b.st[t].ok ? *reinterpret_cast<const bf16x4*>(b.st[t].v + static_cast<size_t>(db) * 16 * page_size)
-                                 : zero4;
+        b.vf[t][db] = *reinterpret_cast<const bf16x4*>(b.st[t].v + static_cast<size_t>(db) * 16 * page_size);
   };
   // One tile from the registers of `b`; its keys, then its values, are requested anew for tile `next`.
   auto process = [&](TileRegs& b, int tile, int next) {
@@ -193,11 +210,11 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int v = 0; v < 4; ++v) a[t * 4 + v] = vcur[t][db][v];
-      if (tail) {
+      if (tail || !sub_ok[0] || !sub_ok[1]) {  // (wave-uniform, and rare: the range's first and last tile)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int key = key0 + (e / 4) * 16 + grp * 4 + (e % 4);
-          if (key >= hi) a[e] = to_bf16_raw(0.f);
+          if (key >= hi || !sub_ok[e / 4]) a[e] = to_bf16_raw(0.f);
         }
       }
 #pragma unroll
@@ -349,18 +366,26 @@ bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_
          (reinterpret_cast<uintptr_t>(q) & 15u) == 0;
 }
 
+// Tiles of kTile keys that a request reads at most.
+static int decode_max_tiles(int window, int max_kv_len) {
+  int span = window > 0 && window < max_kv_len ? window + 16 : max_kv_len;
+  if (span < 1) span = 1;
+  return (span + kTile - 1) / kTile + 1;
+}
+
 // Into how many ranges the keys of each request are cut (num_splits > 0 asks for that many).
 int paged_attention_decode_ranges(int seq_count, int Kh, int window, int max_kv_len, int num_splits) {
   const int units = seq_count * Kh;
-  int span = window > 0 && window < max_kv_len ? window + 16 : max_kv_len;  // keys a request reads at most
-  if (span < 1) span = 1;
-  const int max_tiles = (span + kTile - 1) / kTile + 1;
+  const int max_tiles = decode_max_tiles(window, max_kv_len);
   int KS = num_splits;
   if (KS <= 0) {
     KS = (256 + units / 2) / units;               // about one workgroup per CU: longer ranges amortise the set-up
     const int cap_by_work = (max_tiles + 3) / 4;  // at least 4 tiles (128 keys) per workgroup
     if (KS > cap_by_work) KS = cap_by_work;
   }
+  // (a workgroup looks up the pages of at most kMaxRangeSubTiles sub-tiles: two more than its share of the tiles has)
+  const int least = (2 * max_tiles + kMaxRangeSubTiles - 3) / (kMaxRangeSubTiles - 2);
+  if (KS < least) KS = least;
   if (KS > max_tiles) KS = max_tiles;
   if (KS > kMaxSplits) KS = kMaxSplits;
   if (KS < 1) KS = 1;
@@ -378,6 +403,11 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   int KS = paged_attention_decode_ranges(seq_count, Kh, window, max_kv_len, num_splits);
   const size_t per_split = static_cast<size_t>(units) * 16 * (hd + kRowExtra) * sizeof(float);
   while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
+  if (2 * ((decode_max_tiles(window, max_kv_len) + KS - 1) / KS + 1) > kMaxRangeSubTiles) {
+    set_error("paged_attention_decode: %d keys in %d ranges are more than %d keys per range; the workspace of %zu bytes "
+              "holds no more ranges", max_kv_len, KS, kMaxRangeSubTiles * 16, workspace_bytes);
+    return 1;
+  }
   const dim3 grid(KS, Kh, seq_count);
   const bf16* qp = static_cast<const bf16*>(q);
   const bf16* kp = static_cast<const bf16*>(k_pages);

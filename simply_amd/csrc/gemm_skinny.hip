@@ -23,11 +23,12 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
-constexpr int kUnroll = 4;
+// kUnroll: chunks of 32 columns of K whose loads a wave issues together (one register set).  4 everywhere: sets of 8
+// were slower where they could matter (the 2B down projection, 36 chunks a wave: 18.8 us against 15.7).
 constexpr int kMaxWaves = 16;
 
 // blockDim.x = 64 * NW (NW waves share the K range); a workgroup owns `tile_rows` (16, 8 or 4) rows of W.
-template <int MB, int EPI, bool PACKED>
+template <int MB, int EPI, bool PACKED, int kUnroll>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restrict__ A, int64_t lda,
                                                            const bf16* __restrict__ W, const bf16* __restrict__ W2,
                                                            void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N,
@@ -90,12 +91,59 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
           acc[1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[set][u], b[set][u][mb], acc[1][mb], 0, 0, 0);
       }
   };
-  load_set(0, c0);
-  for (int c = c0; c < c1; c += 2 * kUnroll) {
-    load_set(1, c + kUnroll);
-    mul_set(0);
-    load_set(0, c + 2 * kUnroll);
-    mul_set(1);
+  if (PACKED && K % 32 == 0) {
+    // Tiled weights and whole chunks (every real model's sizes): the loop's loads are unconditional, so that it is
+    // straight-line code and the compiler counts the loads in flight; with a branch around a load it waits for
+    // all of them before the first product, and the two register sets never overlap.  Activation rows beyond M are
+    // read from row M - 1: their products land in output rows that are not stored.
+    const bf16* arow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) arow[mb] = A + static_cast<size_t>(mb * 16 + r < M ? mb * 16 + r : M - 1) * lda + kq * 8;
+    auto load_full = [&](int set, int c) {   // chunks c .. c + kUnroll - 1, all within the wave's range
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        a[set][u] = load_frag(wrow + static_cast<size_t>(c + u) * 512);
+        if (EPI == 1) a2[set][u] = load_frag(w2row + static_cast<size_t>(c + u) * 512);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) b[set][u][mb] = load_frag(arow[mb] + (c + u) * 32);
+      }
+    };
+    const int sets = (c1 - c0) / kUnroll;   // full sets; what is left goes through the loads with tests below
+    int s = 0;
+    if (sets > 0) {
+      load_full(0, c0);
+      for (; s + 2 < sets; s += 2) {   // set 0 holds full set s
+        // (the scheduling barriers keep the compiler from moving the loads of a set behind the products of the
+        // other: it would then wait for them where it has put them, with nothing in flight across iterations)
+        load_full(1, c0 + (s + 1) * kUnroll);
+        __builtin_amdgcn_sched_barrier(0);
+        mul_set(0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_full(0, c0 + (s + 2) * kUnroll);
+        __builtin_amdgcn_sched_barrier(0);
+        mul_set(1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (sets - s == 2) {
+        load_full(1, c0 + (s + 1) * kUnroll);
+        mul_set(0);
+        mul_set(1);
+      } else {
+        mul_set(0);
+      }
+    }
+    if (c0 + sets * kUnroll < c1) {
+      load_set(0, c0 + sets * kUnroll);
+      mul_set(0);
+    }
+  } else {
+    load_set(0, c0);
+    for (int c = c0; c < c1; c += 2 * kUnroll) {
+      load_set(1, c + kUnroll);
+      mul_set(0);
+      load_set(0, c + 2 * kUnroll);
+      mul_set(1);
+    }
   }
 
   // lane holds D[n = 4 * (lane / 16) + v][m = lane % 16]; the waves' tiles are added up through LDS, in wave order
@@ -149,7 +197,7 @@ static void choose_shape(int N, int chunks, int planes, int MB, int* tile_rows, 
   *waves = nw;
 }
 
-template <int MB, bool PACKED>
+template <int MB, bool PACKED, int U>
 static void launch_skinny(const bf16* A, int64_t lda, const bf16* W, const bf16* W2, void* C, int c_dtype, int64_t ldc,
                           int M, int N, int K, int epi, int act, float cap, int tile_rows, int waves,
                           hipStream_t stream) {
@@ -158,13 +206,13 @@ static void launch_skinny(const bf16* A, int64_t lda, const bf16* W, const bf16*
   const int threads = waves * kWave;
   const size_t lds = static_cast<size_t>(waves) * (epi == 1 ? 2 : 1) * MB * 16 * 17 * sizeof(float);
   if (epi == 0)
-    gemm_skinny_kernel<MB, 0, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+    gemm_skinny_kernel<MB, 0, PACKED, U><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
                                                                       tile_rows, cap, act);
   else if (epi == 1)
-    gemm_skinny_kernel<MB, 1, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+    gemm_skinny_kernel<MB, 1, PACKED, U><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
                                                                       tile_rows, cap, act);
   else
-    gemm_skinny_kernel<MB, 2, PACKED><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+    gemm_skinny_kernel<MB, 2, PACKED, U><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
                                                                       tile_rows, cap, act);
 }
 
@@ -196,9 +244,9 @@ int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void*
 #define SA_SKINNY(MBV)                                                                                              \
   do {                                                                                                              \
     if (packed)                                                                                                     \
-      launch_skinny<MBV, true>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream);    \
+      launch_skinny<MBV, true, 4>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream); \
     else                                                                                                            \
-      launch_skinny<MBV, false>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream);   \
+      launch_skinny<MBV, false, 4>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream); \
   } while (0)
   if (MB == 1) SA_SKINNY(1);
   else if (MB == 2) SA_SKINNY(2);
