@@ -301,6 +301,10 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
     const int target = K >= 8192 ? 440 : 256;
     ks = (target + tiles / 2) / tiles;
     if (ks > stages / 4) ks = stages / 4;
+    // ... and no more cuts than keep the partial tiles (written and read again as 32-bit) at half the weights' bytes:
+    // at 256 rows of the 2B down projection 9 cuts (38 us) instead of 36 (54 us); at 64 rows nothing changes
+    const int by_traffic = static_cast<int>((static_cast<int64_t>(NW) * K * 2) / (2 * static_cast<int64_t>(M) * NW * 4));
+    if (ks > by_traffic) ks = by_traffic < 2 ? 2 : by_traffic;
   }
   if (ks > stages) ks = stages;
   if (ks < 1) ks = 1;

@@ -297,6 +297,16 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
         shape = sh[0];
       }
     }
+    // Few rows (portions of a few hundred tokens): the tiles above are too few for 256 CUs, and every workgroup
+    // walks all of K at the pace of its own slabs.  Small tiles with deeper pipelines put a workgroup on every CU
+    // (measured at the 2B shape, q/k/v and output projections: 13 and 11 us up to 256 rows with 64 x 64 tiles, 18 and
+    // 15 at 512 rows with 128 x 64, against 24 to 27 and 21 to 22 with 192 x 128).
+    if (epi == 0) {
+      auto tiles_of = [&](int rows, int wrows) { return static_cast<int64_t>((M + rows - 1) / rows) * ((NW + wrows - 1) / wrows); };
+      // (only while one round of them covers the product: two rounds of small tiles lose to one of large ones)
+      if (tiles_of(64, 64) <= wide::kCUs) shape = 6064064;
+      else if (tiles_of(128, 64) <= wide::kCUs) shape = 5128064;
+    }
   }
   switch (shape) {
     case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
@@ -304,6 +314,16 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
     case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
     case 2128192: wide::launch<4, 6, 2, 2, 4>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;  // two workgroups per CU
+    // small tiles, for products of a few hundred rows whose large tiles would leave most CUs idle (two or more
+    // workgroups per CU fit: 36 to 72 KiB of LDS each)
+    case 3128128: wide::launch<2, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3128064: wide::launch<2, 2, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3064128: wide::launch<1, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3064064: wide::launch<1, 2, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 6064064: wide::launch<1, 2, 4, 6>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 5128064: wide::launch<2, 2, 4, 5>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 4128128: wide::launch<2, 4, 4, 4>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 6064128: wide::launch<1, 4, 4, 6>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
     default:
       set_error("gemm: unknown wide tile %d", shape);
       return 1;

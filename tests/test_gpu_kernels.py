@@ -395,7 +395,7 @@ def test_gemm_tiled(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(257, 1000, 192), (300, 200, 128), (1, 16, 64), (700, 100, 64), (2048, 2304, 2048),
-                                   (513, 4096, 2304), (1000, 388, 1088)])
+                                   (513, 4096, 2304), (1000, 388, 1088), (64, 2304, 2048), (200, 4096, 2304)])
 def test_gemm_wide(M, N, K):
     """The wide-tile MFMA kernel for very many rows: its three tile shapes and its own choice, plain and gated,
     edges in M and N, odd numbers of slabs, strided rows in and out; and what it refuses."""
@@ -406,7 +406,9 @@ def test_gemm_wide(M, N, K):
     tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
     t = dict(rtol=2e-2, atol=2e-2)
     want, want_gated = ref.gemm(a, w).float(), ref.gemm(a, w, w2=w2).float()
-    for shape in (0, 2256192, 3256128, 3128256, 3192128, 2128192):
+    # large tiles, and the small ones with deeper pipelines that products of a few hundred rows get
+    for shape in (0, 2256192, 3256128, 3128256, 3192128, 2128192, 3128128, 3128064, 3064128, 3064064, 6064064, 5128064,
+                  4128128, 6064128):
         kw = dict(algo=ops.ALGO_WIDE, shape=shape)
         torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), want, **t)
         torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), want_gated, **t)
@@ -560,6 +562,26 @@ def test_score(V):
         assert (got[masked] == ops.SCORE_MASKED).all()
     got = ops.score(logits, temperature, top_k, top_p, worst)
     assert got[4] == ops.SCORE_MASKED and got[8] == ops.SCORE_MASKED and got[5] > -1e3   # greedy rows; a plain draw
+
+
+@pytest.mark.parametrize("M", [64, 100, 256, 400, 512, 768, 1100])
+@pytest.mark.parametrize("N,K", [(4096, 2304), (2304, 2048), (2304, 4608), (1000, 9216)])
+def test_gemm_dispatch_at_a_few_hundred_rows(M, N, K):
+    """What the dispatcher chooses by itself for portions of a few hundred tokens (small wide tiles for a short K,
+    the tiled kernel with K cut for a long one, large tiles beyond) against the reference, plain and gated."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles
+    a = rand((M, K), torch.bfloat16, 140)
+    w, w2 = rand((N, K), torch.bfloat16, 141, 0.03), rand((N, K), torch.bfloat16, 142, 0.03)
+    t = dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(ops.gemm(a, pack_tiles(w)).float(), ref.gemm(a, w).float(), **t)
+    if N <= 2304:
+        torch.testing.assert_close(ops.gemm(a, pack_gate_up(w, w2)).float(), ref.gemm(a, w, w2=w2).float(), **t)
+    # rows of wider rows in and out, as the attention output and the fused projection are
+    big, out = rand((M, K + 64), torch.bfloat16, 143), torch.zeros((M, N + 8), dtype=torch.bfloat16, device="cuda")
+    ops.gemm(big[:, 32:32 + K], pack_tiles(w), out=out[:, :N])
+    torch.testing.assert_close(out[:, :N].float(), ref.gemm(big[:, 32:32 + K], w).float(), **t)
+    assert not out[:, N:].any()
 
 
 @pytest.mark.parametrize("activation", [0, 1, 2])
