@@ -124,98 +124,97 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
   }
 }
 
-// The same for many rows (portions of prompts): a workgroup is one wave, which takes `rows_per_wave` rows in
-// turn, each row whole in registers as 4-element pieces (wave reductions only), and (rows of up to 2560 elements)
-// asks for the next row before it works on the one it has, so that stores and loads overlap a little.  NCH: 256-element pieces of a row at most; D % 4 == 0, 16-byte aligned.
-template <typename YT, typename OT, int NCH>
-__global__ __launch_bounds__(64) void add_rmsnorm_rows_kernel(
+// The same for many rows (portions of prompts), a row to a workgroup of four waves: every lane holds NP pieces of
+// four elements, all loads of a row are asked for before the first use, the two sums go through LDS.  A row is a
+// chain of load, sum, store, sum, store; with a row spread over four waves there are four times the waves to
+// overlap these chains than with a wave to a row: 2,048 rows of 2,304 elements (56 MB read and written) take 14 us
+// where a wave to a row took 20, 512 rows 6.6 against 9.0, 8,192 rows 52 against 77.  D % 4 == 0, D <= 1024 NP,
+// 16-byte aligned.
+template <typename YT, typename OT, int NP>
+__global__ __launch_bounds__(256) void add_rmsnorm_split_kernel(
     const YT* __restrict__ y, const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_one_post,
     float* __restrict__ residual, const void* __restrict__ w_next, int w_next_dtype, float eps_next, float plus_one_next,
-    OT* __restrict__ out, int T, int D, int rows_per_wave) {
-  const int lane = threadIdx.x;
-  const int row0 = blockIdx.x * rows_per_wave;
-  const int nrows = T - row0 < rows_per_wave ? T - row0 : rows_per_wave;
+    OT* __restrict__ out, int T, int D, int rows_per_group) {
+  __shared__ float scratch[32];
+  const int tid = threadIdx.x;
   using RawY = typename std::conditional<sizeof(YT) == 4, float4, uint2>::type;
+  auto scales = [&](const void* w, int dtype, float plus, int d) __attribute__((always_inline)) {
+    if (dtype == kBF16) {
+      const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const bf16*>(w) + d);
+      return float4{__uint_as_float(raw.x << 16) + plus, __uint_as_float(raw.x & 0xffff0000u) + plus,
+                    __uint_as_float(raw.y << 16) + plus, __uint_as_float(raw.y & 0xffff0000u) + plus};
+    }
+    const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(w) + d);
+    return float4{raw.x + plus, raw.y + plus, raw.z + plus, raw.w + plus};
+  };
+  float4 wp[NP], wn[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int d = (p * 256 + tid) * 4;
+    wp[p] = wn[p] = float4{1.f, 1.f, 1.f, 1.f};
+    if (d < D && w_post != nullptr) wp[p] = scales(w_post, w_post_dtype, plus_one_post, d);
+    if (d < D && w_next != nullptr) wn[p] = scales(w_next, w_next_dtype, plus_one_next, d);
+  }
   struct Row {
-    float4 h[NCH];
-    RawY y[NCH];
+    float4 h[NP];
+    RawY y[NP];
   };
   auto load = [&](int row, Row& b) __attribute__((always_inline)) {
     const size_t rb = static_cast<size_t>(row) * D;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int d = c * 256 + lane * 4;
+    for (int p = 0; p < NP; ++p) {
+      const int d = (p * 256 + tid) * 4;
+      b.h[p] = float4{0.f, 0.f, 0.f, 0.f};
+      b.y[p] = RawY{};
       if (d < D) {
-        b.h[c] = *reinterpret_cast<const float4*>(residual + rb + d);
-        b.y[c] = *reinterpret_cast<const RawY*>(y + rb + d);
+        b.h[p] = *reinterpret_cast<const float4*>(residual + rb + d);
+        b.y[p] = *reinterpret_cast<const RawY*>(y + rb + d);
       }
     }
   };
-  // four scale factors at a time (one 8-byte load when they are bfloat16)
-  auto scales = [&](const void* w, int dtype, float plus, int d, float* out4) __attribute__((always_inline)) {
-    if (dtype == kBF16) {
-      const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const bf16*>(w) + d);
-      out4[0] = __uint_as_float(raw.x << 16) + plus;
-      out4[1] = __uint_as_float(raw.x & 0xffff0000u) + plus;
-      out4[2] = __uint_as_float(raw.y << 16) + plus;
-      out4[3] = __uint_as_float(raw.y & 0xffff0000u) + plus;
-    } else {
-      const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(w) + d);
-      out4[0] = raw.x + plus;
-      out4[1] = raw.y + plus;
-      out4[2] = raw.z + plus;
-      out4[3] = raw.w + plus;
-    }
-  };
-  auto process = [&](int row, Row& b) __attribute__((always_inline)) {
+  auto process = [&](int row, Row& b, float* red) __attribute__((always_inline)) {
     const size_t rb = static_cast<size_t>(row) * D;
-    float4 yv[NCH];
+    float4 yv[NP];
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      if (c * 256 + lane * 4 >= D) {
-        yv[c] = float4{0.f, 0.f, 0.f, 0.f};
-        b.h[c] = float4{0.f, 0.f, 0.f, 0.f};
-      } else if constexpr (sizeof(YT) == 4) {
-        yv[c] = b.y[c];
-      } else {
-        yv[c] = float4{__uint_as_float(b.y[c].x << 16), __uint_as_float(b.y[c].x & 0xffff0000u),
-                       __uint_as_float(b.y[c].y << 16), __uint_as_float(b.y[c].y & 0xffff0000u)};
-      }
+    for (int p = 0; p < NP; ++p) {
+      if constexpr (sizeof(YT) == 4) yv[p] = b.y[p];
+      else yv[p] = float4{__uint_as_float(b.y[p].x << 16), __uint_as_float(b.y[p].x & 0xffff0000u),
+                          __uint_as_float(b.y[p].y << 16), __uint_as_float(b.y[p].y & 0xffff0000u)};
     }
     float r = 1.f;
     if (w_post != nullptr) {
       float ss = 0.f;
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) ss += yv[c].x * yv[c].x + yv[c].y * yv[c].y + yv[c].z * yv[c].z + yv[c].w * yv[c].w;
-      r = rsqrtf(wave_sum(ss) / static_cast<float>(D) + eps_post);
+      for (int p = 0; p < NP; ++p) ss += yv[p].x * yv[p].x + yv[p].y * yv[p].y + yv[p].z * yv[p].z + yv[p].w * yv[p].w;
+      r = rsqrtf(block_sum(ss, red) / static_cast<float>(D) + eps_post);
     }
     float ss2 = 0.f;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int d = c * 256 + lane * 4;
-      if (d >= D) continue;
-      float* h = reinterpret_cast<float*>(&b.h[c]);
-      const float* v = reinterpret_cast<const float*>(&yv[c]);
-      float w4[4] = {1.f, 1.f, 1.f, 1.f};
-      if (w_post != nullptr) scales(w_post, w_post_dtype, plus_one_post, d, w4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        h[e] += w_post != nullptr ? v[e] * r * w4[e] : v[e];
-        ss2 += h[e] * h[e];
+    for (int p = 0; p < NP; ++p) {
+      const int d = (p * 256 + tid) * 4;
+      float4& h = b.h[p];
+      if (w_post != nullptr) {
+        h.x += yv[p].x * r * wp[p].x;
+        h.y += yv[p].y * r * wp[p].y;
+        h.z += yv[p].z * r * wp[p].z;
+        h.w += yv[p].w * r * wp[p].w;
+      } else {
+        h.x += yv[p].x;
+        h.y += yv[p].y;
+        h.z += yv[p].z;
+        h.w += yv[p].w;
       }
-      *reinterpret_cast<float4*>(residual + rb + d) = b.h[c];
+      ss2 += h.x * h.x + h.y * h.y + h.z * h.z + h.w * h.w;
+      if (d < D) *reinterpret_cast<float4*>(residual + rb + d) = h;
     }
     if (w_next == nullptr) return;
-    const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(D) + eps_next);
+    const float r2 = rsqrtf(block_sum(ss2, red + 8) / static_cast<float>(D) + eps_next);
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int d = c * 256 + lane * 4;
+    for (int p = 0; p < NP; ++p) {
+      const int d = (p * 256 + tid) * 4;
       if (d >= D) continue;
-      const float* h = reinterpret_cast<const float*>(&b.h[c]);
-      float w4[4], o[4];
-      scales(w_next, w_next_dtype, plus_one_next, d, w4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = h[e] * r2 * w4[e];
+      const float4 h = b.h[p];
+      const float o[4] = {h.x * r2 * wn[p].x, h.y * r2 * wn[p].y, h.z * r2 * wn[p].z, h.w * r2 * wn[p].w};
       if constexpr (sizeof(OT) == 4) {
         *reinterpret_cast<float4*>(out + rb + d) = float4{o[0], o[1], o[2], o[3]};
       } else {
@@ -226,20 +225,17 @@ __global__ __launch_bounds__(64) void add_rmsnorm_rows_kernel(
       }
     }
   };
-  Row b0;
-  load(row0, b0);
-  if constexpr (NCH <= 10) {
-    Row b1;
-    for (int i = 0; i < nrows; i += 2) {
-      if (i + 1 < nrows) load(row0 + i + 1, b1);
-      process(row0 + i, b0);
-      if (i + 2 < nrows) load(row0 + i + 2, b0);
-      if (i + 1 < nrows) process(row0 + i + 1, b1);
-    }
-  } else {
-    for (int i = 0; i < nrows; ++i) {
-      if (i > 0) load(row0 + i, b0);
-      process(row0 + i, b0);
+  // the group's rows in turn; the next row is asked for before the one at hand is worked on
+  const int row0 = blockIdx.x * rows_per_group;
+  const int nrows = T - row0 < rows_per_group ? T - row0 : rows_per_group;
+  Row a, b;
+  load(row0, a);
+  for (int i = 0; i < nrows; i += 2) {
+    if (i + 1 < nrows) load(row0 + i + 1, b);
+    process(row0 + i, a, scratch);
+    if (i + 1 < nrows) {
+      if (i + 2 < nrows) load(row0 + i + 2, a);
+      process(row0 + i + 1, b, scratch + 16);
     }
   }
 }
@@ -575,33 +571,32 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
   if (T == 0) return 0;
   SA_REQUIRE(T > 0 && D > 0, "add_rmsnorm: bad sizes T=%d D=%d", T, D);
   SA_REQUIRE(w_next == nullptr || out != nullptr, "add_rmsnorm: a next norm needs an output");
-  // many rows (enough for two workgroups of four rows per compute unit): a wave per row
+  // many rows: a workgroup of four waves per row (or two rows)
   const auto aligned16 = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
   const int o_dtype = out != nullptr ? out_dtype : y_dtype;
-  if (T >= 512 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out) &&
+  if (T >= 64 && D % 4 == 0 && D <= 5120 && aligned16(y) && aligned16(residual) && aligned16(out) &&
       aligned16(w_post) && aligned16(w_next)) {
     const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
-    // rows of a wave: enough waves for two per compute unit first, then up to four rows each
-    // two rows to a wave once that still leaves two waves for every SIMD (measured: more rows to a wave are slower,
-    // a wave takes about 5 us for a row); rows of more than 2560 elements do not fit twice into the registers
-    const int rows_per_wave = T >= 1024 && D <= 2560 ? 2 : 1;
-    const int blocks = (T + rows_per_wave - 1) / rows_per_wave;
-#define SA_ROWS(YT, OT, NCH)                                                                                     \
-  add_rmsnorm_rows_kernel<YT, OT, NCH><<<blocks, 64, 0, stream>>>(static_cast<const YT*>(y), w_post, w_post_dtype, \
-                                                                  eps_post, pp, residual, w_next, w_next_dtype,    \
-                                                                  eps_next, pn, static_cast<OT*>(out), T, D,       \
-                                                                  rows_per_wave)
-#define SA_ROWS_N(YT, OT)     \
-  do {                        \
-    if (D <= 2560) SA_ROWS(YT, OT, 10); \
-    else SA_ROWS(YT, OT, 20); \
+    // two rows to a workgroup, the second asked for before the first is worked on, once there are rows enough
+    // (2,048 rows: 14.3 us against 16.8 with one; 512 rows: 8.2 against 6.6)
+    const int rpg = T >= 2048 ? 2 : 1;
+#define SA_SPLIT(YT, OT, NP)                                                                                       \
+  add_rmsnorm_split_kernel<YT, OT, NP><<<(T + rpg - 1) / rpg, 256, 0, stream>>>(                                   \
+      static_cast<const YT*>(y), w_post, w_post_dtype, eps_post, pp, residual, w_next, w_next_dtype, eps_next, pn, \
+      static_cast<OT*>(out), T, D, rpg)
+#define SA_SPLIT_N(YT, OT)            \
+  do {                                \
+    if (D <= 2048) SA_SPLIT(YT, OT, 2); \
+    else if (D <= 3072) SA_SPLIT(YT, OT, 3); \
+    else if (D <= 4096) SA_SPLIT(YT, OT, 4); \
+    else SA_SPLIT(YT, OT, 5);         \
   } while (0)
-    if (y_dtype == kBF16 && o_dtype == kBF16) SA_ROWS_N(bf16, bf16);
-    else if (y_dtype == kBF16) SA_ROWS_N(bf16, float);
-    else if (o_dtype == kBF16) SA_ROWS_N(float, bf16);
-    else SA_ROWS_N(float, float);
-#undef SA_ROWS_N
-#undef SA_ROWS
+    if (y_dtype == kBF16 && o_dtype == kBF16) SA_SPLIT_N(bf16, bf16);
+    else if (y_dtype == kBF16) SA_SPLIT_N(bf16, float);
+    else if (o_dtype == kBF16) SA_SPLIT_N(float, bf16);
+    else SA_SPLIT_N(float, float);
+#undef SA_SPLIT_N
+#undef SA_SPLIT
     return check_launch("add_rmsnorm");
   }
   add_rmsnorm_kernel<<<T, row_threads(D), 0, stream>>>(y, y_dtype, w_post, w_post_dtype, eps_post,

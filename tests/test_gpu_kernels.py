@@ -50,7 +50,8 @@ def test_rmsnorm(dtype, T, D):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304), (600, 2304), (513, 100), (515, 5000), (512, 6000), (517, 50)])
+@pytest.mark.parametrize("T,D", [(1, 48), (6, 100), (3, 2304), (600, 2304), (513, 100), (515, 5000), (512, 6000), (517, 50),
+                                 (64, 2304), (100, 3584), (2049, 2304), (2050, 4608), (2051, 1028), (2048, 5120)])
 def test_add_rmsnorm(dtype, T, D):
     from simply_amd.kernels import ops
     y = rand((T, D), dtype, 3, 2.0)
