@@ -238,6 +238,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prefill-chunked"],
+                    help="measure one part alone (for profiles); the line then holds that part only")
     ap.add_argument("--latency-steps", type=int, default=100,
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
@@ -287,10 +289,28 @@ def main():
               flush=True)
         return
 
+    if args.only in ("prefill", "prefill-chunked"):
+        T = args.prefill_tokens
+        portion = -(-T // 4) if args.only == "prefill-chunked" else None
+        pt = run_prefill(model, cfg, T, max(3, args.steps), args.page_size, args.dtype, portion=portion)
+        peak = PEAK_TFLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        print(json.dumps({"metric": f"prefill tokens/s ({T} tokens" + (", 4 portions)" if portion else ")"),
+                          "value": round(T / pt, 1), "unit": "tokens/s", "ms": round(pt * 1e3, 3),
+                          "frac": round(prefill_flops(cfg, T) / pt / 1e12 / peak, 4), "n_gpus": 1,
+                          "config": {"model": f"gemma2-{args.shape}-shape", "layers": cfg.num_hidden_layers}}), flush=True)
+        return
+
     dt, mean_kv, latencies = run_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, args.page_size,
                                         args.dtype, latency_steps=args.latency_steps)
     step_bytes = weight_bytes(cfg, esize) + args.batch * kv_bytes_per_request(cfg, mean_kv, esize)
     achieved = step_bytes / dt / 1e9
+
+    if args.only == "decode":
+        print(json.dumps({"metric": "decode tokens/s (batch %d, context %d)" % (args.batch, args.context),
+                          "value": round(args.batch / dt, 1), "unit": "tokens/s", "ms_per_step": round(dt * 1e3, 4),
+                          "roofline_frac": round(achieved / HBM_GBPS, 4), "n_gpus": 1, "steps": args.steps,
+                          "config": {"model": f"gemma2-{args.shape}-shape", "layers": cfg.num_hidden_layers}}), flush=True)
+        return
 
     T = args.prefill_tokens
     pt = run_prefill(model, cfg, T, 3, args.page_size, args.dtype)

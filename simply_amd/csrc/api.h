@@ -188,7 +188,10 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
 bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
                      const void* C, int c_dtype, int epi, int packed);
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
-              int shape, hipStream_t stream);
+              int shape, int ks, void* workspace, size_t workspace_bytes, hipStream_t stream);
+// C = epilogue(sum over z of partials[z][M][NW]): the second kernel of every product that cuts K over workgroups
+int gemm_sum_partials(const float* partials, int ks, void* C, int c_dtype, int64_t ldc, int M, int N, int NW, int epi,
+                      int act, float cap, hipStream_t stream);
 bool gemm_streams_weights(int M, int NW, int K);
 bool gemm_tiled_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2, int packed);
 int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, int64_t ldc, int M, int N, int K,

@@ -264,6 +264,16 @@ static void launch(const bf16* A, int64_t lda, const bf16* W, void* C, int c_dty
 
 }  // namespace tiled
 
+int gemm_sum_partials(const float* partials, int ks, void* C, int c_dtype, int64_t ldc, int M, int N, int NW, int epi,
+                      int act, float cap, hipStream_t stream) {
+  const size_t total = static_cast<size_t>(M) * N;
+  const int blocks = static_cast<int>((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+  if (epi == 1) tiled::gemm_reduce_kernel<1><<<blocks, 256, 0, stream>>>(partials, ks, C, c_dtype, ldc, M, N, NW, cap, act);
+  else if (epi == 2) tiled::gemm_reduce_kernel<2><<<blocks, 256, 0, stream>>>(partials, ks, C, c_dtype, ldc, M, N, NW, cap, act);
+  else tiled::gemm_reduce_kernel<0><<<blocks, 256, 0, stream>>>(partials, ks, C, c_dtype, ldc, M, N, NW, cap, act);
+  return check_launch("gemm_sum_partials");
+}
+
 // Whether a product of M rows against NW weight rows of length K is better off with 64 rows x 256 weight rows per
 // workgroup and K cut over workgroups than with the wide-tile kernel.  Measured at the 2B, 9B and 27B sizes: up to
 // 64 rows always; beyond that while M * NW stays below about a million (192 rows of a q/k/v projection, 256 to 384

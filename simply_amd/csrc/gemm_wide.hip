@@ -19,8 +19,12 @@
 //   * The products are taken transposed (W fragment as the first operand), so that a lane holds four neighbouring
 //     columns of one row of C and stores them as one 8-byte piece.
 //
-// Epilogues: none; gated (C = gelu_tanh(A.Wg^T) * (A.Wu^T), both rounded to bfloat16 first, from one weight whose
+// Epilogues: none; gated (C = act(A.Wg^T) * (A.Wu^T), both rounded to bfloat16 first, from one weight whose
 // 16-row tiles alternate between Wg and Wu).  K must be a multiple of 64, N and ldc of 4.
+//
+// K may be cut over gridDim.z workgroups (a few hundred rows against a long K and few weight rows: too few tiles for
+// 256 CUs otherwise): each writes its 32-bit partial tile to `partials` [z][M][N], and the tiled kernel's sum kernel
+// adds them up.
 #include "api.h"
 #include "common.h"
 
@@ -61,7 +65,8 @@ __device__ __forceinline__ void load_to_lds(const bf16* base, uint32_t offset, u
 template <int WM, int WN, int WAVES_M, int EPI, int NSTAGE, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __restrict__ A, int64_t lda,
                                                         const bf16* __restrict__ W, bf16* __restrict__ C, int64_t ldc,
-                                                        int M, int N, int K, int chunks, int act) {
+                                                        int M, int N, int K, int chunks, int act,
+                                                        float* __restrict__ partials) {
   constexpr int WAVES_N = WAVES / WAVES_M;
   constexpr int MT = WAVES_M * WM, NT = WAVES_N * WN;  // 16-row tiles of A and of W per workgroup
   constexpr int BM = MT * 16;
@@ -96,6 +101,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
       bx = full * GX + rem % width;
     }
   }
+  // this workgroup's share of K: slabs slab0 .. slab0 + slabs
+  const int slabs_all = K / BK;
+  const int slab0 = static_cast<int>(static_cast<int64_t>(blockIdx.z) * slabs_all / gridDim.z);
+  const int slabs = static_cast<int>(static_cast<int64_t>(blockIdx.z + 1) * slabs_all / gridDim.z) - slab0;
+  A += static_cast<size_t>(slab0) * BK;
   const int m_base = by * BM;
   const int NW = EPI == 1 ? 2 * ((N + 15) / 16) * 16 : N;
   const int ntiles = (NW + 15) / 16;
@@ -120,7 +130,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
   for (int i = 0; i < WPW; ++i) {
     const int nt = nt_base + tile_mine + (WAVES / 2) * i;
     const int clamped = __builtin_amdgcn_readfirstlane(nt < ntiles ? nt : ntiles - 1);
-    w_from[i] = W + (static_cast<size_t>(clamped) * chunks + half_mine) * 512;
+    w_from[i] = W + (static_cast<size_t>(clamped) * chunks + half_mine) * 512 + static_cast<size_t>(slab0) * 1024;
   }
   // load n (of LOADS) of slab `slab` into buffer `buf`
   constexpr int LOADS = APW + WPW;
@@ -146,7 +156,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
     const int r = lane % 16;
     a_frag[kc] = r * 64 + ((kc * 4 + lane / 16) ^ (r / 2)) * 8;
   }
-  const int slabs = K / BK;
   // Fragments of the two halves of a slab (columns 0 .. 31 and 32 .. 63) in registers of their own.  The products
   // of the second half are held back until after the next barrier, where they cover the time that the fragment
   // reads of the next slab's first half take; the reads of the second half are covered by the products of the
@@ -223,6 +232,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
   for (int i = 0; i < WM; ++i) {
     const int m = m_base + (wm * WM + i) * 16 + row;
     if (m >= M) continue;
+    if (EPI == 3) {  // this workgroup's share of the sum, as it is
+      float* p_row = partials + (static_cast<size_t>(blockIdx.z) * M + m) * N;
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        const int n = (nt_base + wn * WN + j) * 16 + quad * 4;
+        if (n < N) *reinterpret_cast<floatx4*>(p_row + n) = acc[i][j];
+      }
+      continue;
+    }
     bf16* c_row = C + static_cast<size_t>(m) * ldc;
     constexpr int OUT = EPI == 1 ? WN / 2 : WN;
 #pragma unroll
@@ -249,16 +267,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
 
 template <int WM, int WN, int WAVES_M, int NSTAGE, int WAVES = 8>
 static void launch(const bf16* A, int64_t lda, const bf16* W, bf16* C, int64_t ldc, int M, int N, int K, int epi,
-                   int act, hipStream_t stream) {
+                   int act, int ks, float* partials, hipStream_t stream) {
   constexpr int BM = WAVES_M * WM * 16, BNW = (WAVES / WAVES_M) * WN * 16;
   const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-  const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM);
+  const dim3 grid((NW + BNW - 1) / BNW, (M + BM - 1) / BM, ks);
   if (epi == 1)
     gemm_wide_kernel<WM, WN, WAVES_M, 1, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32,
-                                                                                         act);
+                                                                                         act, nullptr);
+  else if (ks > 1)
+    gemm_wide_kernel<WM, WN, WAVES_M, 3, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32,
+                                                                                         act, partials);
   else
     gemm_wide_kernel<WM, WN, WAVES_M, 0, NSTAGE, WAVES><<<grid, WAVES * 64, 0, stream>>>(A, lda, W, C, ldc, M, N, K, K / 32,
-                                                                                         act);
+                                                                                         act, nullptr);
 }
 
 }  // namespace wide
@@ -273,8 +294,17 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
 
 // shape: 0: chosen here; else stages * 1000000 + rows * 1000 + weight rows of a workgroup's tile (2256192, 3256128,
 // 3128256, 3192128; 2128192: workgroups of four waves, two to a CU).
+// ks > 1 cuts K over that many workgroups per tile (no epilogue only; the partial tiles go through `workspace`,
+// which must hold ks * M * N floats).
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
-              int shape, hipStream_t stream) {
+              int shape, int ks, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (ks < 1) ks = 1;
+  if (ks > K / wide::BK) ks = K / wide::BK;
+  if (ks > 1 && (epi != 0 || workspace == nullptr || static_cast<size_t>(ks) * M * N * sizeof(float) > workspace_bytes)) {
+    set_error("gemm: the wide kernel cuts K only without an epilogue and with a workspace of ks * M * N floats");
+    return 1;
+  }
+  float* ws = static_cast<float*>(workspace);
   const bf16* a = static_cast<const bf16*>(A);
   const bf16* w = static_cast<const bf16*>(W);
   bf16* c = static_cast<bf16*>(C);
@@ -297,38 +327,67 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
         shape = sh[0];
       }
     }
-    // Few rows (portions of a few hundred tokens): the tiles above are too few for 256 CUs, and every workgroup
-    // walks all of K at the pace of its own slabs.  Small tiles with deeper pipelines put a workgroup on every CU
-    // (measured at the 2B shape, q/k/v and output projections: 13 and 11 us up to 256 rows with 64 x 64 tiles, 18 and
-    // 15 at 512 rows with 128 x 64, against 24 to 27 and 21 to 22 with 192 x 128).
-    if (epi == 0) {
-      auto tiles_of = [&](int rows, int wrows) { return static_cast<int64_t>((M + rows - 1) / rows) * ((NW + wrows - 1) / wrows); };
-      // (only while one round of them covers the product: two rounds of small tiles lose to one of large ones)
-      if (tiles_of(64, 64) <= wide::kCUs) shape = 6064064;
-      else if (tiles_of(128, 64) <= wide::kCUs) shape = 5128064;
+    // Up to 1,536 rows without an epilogue (portions of prompts, many decoding requests): the tiles above are too few
+    // for 256 CUs, and every workgroup walks all of K at the pace of its own slabs.  Smaller tiles with deeper
+    // pipelines, and K cut over workgroups so that about one round of them covers the GPU, chosen by a model of the
+    // time fitted to measurements at the 2B, 9B and 27B sizes (64 to 2,048 rows, seven tiles, one to fourteen cuts;
+    // it is within 6 % of the best measured choice nearly everywhere, and a fifth faster in sum than either the
+    // uncut tiles above or the tiled kernel with its cut: the 2B down projection at 512 rows takes 36 us against 55).
+    if (epi == 0 && M >= 64 && M <= 1536) {
+      struct Tile { int code, rows, wrows; double eff, start; };  // share of the MFMA rate in the loop; us to start
+      static const Tile tiles[7] = {{3128128, 128, 128, 0.425, 1.44}, {3128256, 128, 256, 0.535, 2.03},
+                                    {3192128, 192, 128, 0.535, 1.25}, {3256128, 256, 128, 0.615, 1.58},
+                                    {5128064, 128, 64, 0.326, 0.85},  {6064064, 64, 64, 0.234, 0.80},
+                                    {6064128, 64, 128, 0.277, 1.08}};
+      const int slabs = K / wide::BK;
+      double best_us = -1.0;
+      int best_ks = 1;
+      for (const Tile& t : tiles) {
+        const int64_t count = static_cast<int64_t>((M + t.rows - 1) / t.rows) * ((N + t.wrows - 1) / t.wrows);
+        const int cuts[3] = {1, static_cast<int>(wide::kCUs / count), static_cast<int>(2 * wide::kCUs / count)};
+        for (int c = 0; c < 3; ++c) {
+          const int cut = cuts[c];
+          if (cut < 1 || (c > 0 && (cut < 2 || cut == cuts[c - 1])) || cut > slabs / 4) continue;
+          const double partial_bytes = static_cast<double>(cut) * M * N * 4;
+          if (cut > 1 && (ws == nullptr || partial_bytes > static_cast<double>(workspace_bytes))) continue;
+          const int64_t rounds = (count * cut + wide::kCUs - 1) / wide::kCUs;
+          const int per = (slabs + cut - 1) / cut;
+          // a CU's MFMA rate: 4.9 M multiply-adds of bfloat16 a microsecond
+          double us = rounds * (static_cast<double>(per) * t.rows * t.wrows * wide::BK / (4.9e6 * t.eff) + t.start) + 3.2;
+          if (cut > 1) us += partial_bytes / 5.5e6 + partial_bytes / 4.9e6 + 3.7;  // written, read again, the sum kernel
+          if (best_us < 0 || us < best_us) {
+            best_us = us;
+            shape = t.code;
+            best_ks = cut;
+          }
+        }
+      }
+      if (ks == 1) ks = best_ks;
     }
   }
   switch (shape) {
-    case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 2128192: wide::launch<4, 6, 2, 2, 4>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;  // two workgroups per CU
+    case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 3128256: wide::launch<4, 4, 2, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 3192128: wide::launch<3, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 2128192: wide::launch<4, 6, 2, 2, 4>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;  // two workgroups per CU
     // small tiles, for products of a few hundred rows whose large tiles would leave most CUs idle (two or more
     // workgroups per CU fit: 36 to 72 KiB of LDS each)
-    case 3128128: wide::launch<2, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 3128064: wide::launch<2, 2, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 3064128: wide::launch<1, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 3064064: wide::launch<1, 2, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 6064064: wide::launch<1, 2, 4, 6>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 5128064: wide::launch<2, 2, 4, 5>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 4128128: wide::launch<2, 4, 4, 4>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
-    case 6064128: wide::launch<1, 4, 4, 6>(a, lda, w, c, ldc, M, N, K, epi, act, stream); break;
+    case 3128128: wide::launch<2, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 3128064: wide::launch<2, 2, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 3064128: wide::launch<1, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 3064064: wide::launch<1, 2, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 6064064: wide::launch<1, 2, 4, 6>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 5128064: wide::launch<2, 2, 4, 5>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 4128128: wide::launch<2, 4, 4, 4>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
+    case 6064128: wide::launch<1, 4, 4, 6>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
     default:
       set_error("gemm: unknown wide tile %d", shape);
       return 1;
   }
-  return check_launch("gemm_wide");
+  if (check_launch("gemm_wide")) return 1;
+  if (ks > 1) return gemm_sum_partials(ws, ks, C, kBF16, ldc, M, N, N, 0, 0, 0.f, stream);
+  return 0;
 }
 
 }  // namespace sa

@@ -72,23 +72,10 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   // without a cut of K (measured at 32 and 64 rows: 10-20 % faster than the tiled kernel with its sum kernel at the
   // 2B, 9B and 27B sizes)
   const int NW = epilogue == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-  // A few hundred rows against a long K and few weight rows (portions of prompts through the down projections): the
-  // wide kernel's tiles, too few for 256 CUs, would each walk all of K (86 us at 512 rows of the 2B shape); the tiled
-  // kernel's 128 x 128 tiles with K cut so that there is a workgroup per CU take 56 us, sum kernel included.
-  const int tiles128 = ((M + 127) / 128) * ((NW + 127) / 128);
-  if (algo == 0 && bf16_in && packed && epilogue != 1 && !gemm_streams_weights(M, NW, K) && K >= 4096 && tiles128 <= 96 &&
-      gemm_tiled_takes(M, N, K, lda, A, W, W2, packed)) {
-    int ks = (288 + tiles128 / 2) / tiles128;
-    if (ks > K / 64 / 4) ks = K / 64 / 4;
-    if (ks >= 2)
-      return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, act, cap, ks, workspace,
-                        static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
-  }
-  // 64 rows and more against a short K without the gated epilogue (q/k/v and output projections of portions of a
-  // few hundred tokens): the wide kernel's small tiles, a workgroup per CU (13 and 11 us at the 2B shape against 19 to
-  // 27 for the tiled kernel with K cut and its sum kernel)
-  const bool small_wide = epilogue == 0 && M >= 64 && K < 4096 &&
-                          static_cast<int64_t>((M + 63) / 64) * ((N + 63) / 64) <= 256;
+  // 64 to 1,536 rows without an epilogue (q/k/v, output and down projections of portions of prompts and of many
+  // decoding requests): the wide kernel with a tile and a cut of K that it chooses for the sizes (at 64 rows of the 2B
+  // down projection 15 us against 23 for the tiled kernel with its cut; at 512 rows 36 against 55)
+  const bool small_wide = epilogue == 0 && M >= 64 && M <= 1536 && N <= 16384;
   const bool wide_first = !gemm_streams_weights(M, NW, K) || (epilogue == 1 && M > 16) || small_wide;
   if (algo == 4 || (algo == 0 && bf16_in && packed && wide_first)) {
     const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
@@ -96,7 +83,11 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                "gemm: the wide MFMA kernel takes bfloat16 in and out with tiled weights, no soft-cap, K a multiple of "
                "64, N and ldc of 4, lda of 8; got N=%d K=%d lda=%lld ldc=%lld tiled=%d", N, K, (long long)lda,
                (long long)ldc, packed);
-    if (takes) return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape : 0, stream);
+    // (a shape given by the caller may carry a cut of K in front: cuts * 10000000 + shape)
+    if (takes)
+      return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape % 10000000 : 0,
+                       algo == 4 ? shape / 10000000 : 1, workspace,
+                       static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
   }
   if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || tiled_first))) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);

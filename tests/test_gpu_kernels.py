@@ -413,10 +413,18 @@ def test_gemm_wide(M, N, K):
         kw = dict(algo=ops.ALGO_WIDE, shape=shape)
         torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), want, **t)
         torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), want_gated, **t)
-    # the same rows whatever the tile and whoever else is in the batch, to the bit: every sum runs along K in order
+    # K cut over two, three and seven workgroups per tile (their partial tiles summed by a second kernel); a cut
+    # that K is too short for shrinks to what it allows
+    for shape in (20000000 + 3128128, 30000000 + 6064064, 70000000 + 3256128, 20000000 + 5128064, 30000000 + 3192128):
+        torch.testing.assert_close(ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=shape).float(), want, **t)
+    if K >= 128:
+        with pytest.raises(KernelError, match="cuts K only without"):
+            ops.gemm(a, tw2, algo=ops.ALGO_WIDE, shape=20000000 + 3128128)
+    # the same rows whatever the tile and whoever else is in the batch, to the bit, while K is not cut: every sum
+    # runs along K in order
     one = ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=2256192)
     assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=3128256))
-    assert torch.equal(one[: M // 2 + 1], ops.gemm(a[: M // 2 + 1], tw, algo=ops.ALGO_WIDE))
+    assert torch.equal(one[: M // 2 + 1], ops.gemm(a[: M // 2 + 1], tw, algo=ops.ALGO_WIDE, shape=3192128))
     assert torch.equal(one, ops.gemm(a, tw, algo=ops.ALGO_TILED, shape=1))   # (K in one piece: the same order)
     # rows inside wider rows, in and out
     kw = dict(algo=ops.ALGO_WIDE)
@@ -565,11 +573,12 @@ def test_score(V):
     assert got[4] == ops.SCORE_MASKED and got[8] == ops.SCORE_MASKED and got[5] > -1e3   # greedy rows; a plain draw
 
 
-@pytest.mark.parametrize("M", [64, 100, 256, 400, 512, 768, 1100])
-@pytest.mark.parametrize("N,K", [(4096, 2304), (2304, 2048), (2304, 4608), (1000, 9216)])
+@pytest.mark.parametrize("M", [64, 100, 256, 400, 512, 768, 1100, 1536, 1537])
+@pytest.mark.parametrize("N,K", [(4096, 2304), (2304, 2048), (2304, 4608), (1000, 9216), (2304, 9216)])
 def test_gemm_dispatch_at_a_few_hundred_rows(M, N, K):
-    """What the dispatcher chooses by itself for portions of a few hundred tokens (small wide tiles for a short K,
-    the tiled kernel with K cut for a long one, large tiles beyond) against the reference, plain and gated."""
+    """What the dispatcher chooses by itself for portions of a few hundred tokens and for many decoding requests
+    (the wide kernel with a tile and a cut of K that it fits to the sizes; large tiles beyond) against the reference,
+    plain and gated."""
     from simply_amd.kernels import ops
     from simply_amd.kernels.packing import pack_gate_up, pack_tiles
     a = rand((M, K), torch.bfloat16, 140)
