@@ -318,6 +318,20 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
   }
   const float my = tid < KS ? base[tid * stride + HD] : -INFINITY;
   const float ly = tid < KS ? base[tid * stride + HD + 1] : 0.f;
+  // The threads are `parts` groups of HD / 4: group p adds up ranges p, p + parts, ... for four dimensions per
+  // thread, then group 0 adds the groups up in order.  The first kAhead ranges of a thread are asked for here,
+  // before the weights are known: their loads are under way together with those of the maxima and sums above, so
+  // the kernel waits for memory once, not twice.
+  constexpr int kAhead = 8;
+  const int quarter = HD / 4, parts = 256 / quarter;
+  const int c = tid % quarter, part = tid / quarter;
+  float4 ahead[kAhead];
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) {
+    const int y = part + i * parts;
+    ahead[i] = (part < parts && y < KS) ? *reinterpret_cast<const float4*>(base + y * stride + 4 * c)
+                                        : float4{0.f, 0.f, 0.f, 0.f};
+  }
   // maximum over the ranges
   float mx = wave_max(my);
   if (tid % kWave == 0) scratch[tid / kWave] = mx;
@@ -326,13 +340,18 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
   const float wy = my == -INFINITY ? 0.f : __expf(my - Mg);
   if (tid < KS) w_s[tid] = wy;
   const float Lg = block_sum(ly * wy, scratch + 4);  // has its own barriers; w_s is complete after them
-  // The threads are `parts` groups of HD / 4: group p adds up ranges p, p + parts, ... for four dimensions per
-  // thread (the loads of a thread do not depend on each other), then group 0 adds the groups up in order.
-  const int quarter = HD / 4, parts = 256 / quarter;
-  const int c = tid % quarter, part = tid / quarter;
   float4 o = {0.f, 0.f, 0.f, 0.f};
   if (part < parts) {
-    for (int y = part; y < KS; y += parts) {
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+      const int y = part + i * parts;
+      const float w = y < KS ? w_s[y] : 0.f;
+      o.x += ahead[i].x * w;
+      o.y += ahead[i].y * w;
+      o.z += ahead[i].z * w;
+      o.w += ahead[i].w * w;
+    }
+    for (int y = part + kAhead * parts; y < KS; y += parts) {
       const float4 v = *reinterpret_cast<const float4*>(base + y * stride + 4 * c);
       const float w = w_s[y];
       o.x += v.x * w;
