@@ -56,8 +56,8 @@ def cmd_generate(argv) -> int:
     _flag(ap, "top_k", type=int, default=-1)
     _flag(ap, "top_p", type=float, default=1.0)
     _flag(ap, "max_num_issue_tokens", type=int, default=2048)
-    _flag(ap, "intermediate_steps", type=int, default=8,
-          help="decode steps that may run in a row on the device before the host looks at the tokens")
+    _flag(ap, "intermediate_steps", type=int, default=64,
+          help="decode steps that may run in a row without a new scheduling decision (a run ends when a request ends)")
     _flag(ap, "seed", type=int, default=0)
     _flag(ap, "ignore_eos", action="store_true")
     args = ap.parse_args(argv)

@@ -35,6 +35,9 @@ class StepContext:
     q_lens: list[int]             # tokens of the request in this step
     cu_q_lens: list[int]          # [S + 1] offsets of the requests in the flat batch
     _units: dict = dataclasses.field(default_factory=dict)
+    #: set for a step whose launches are recorded and replayed for later steps: the most keys that any step that
+    #: replays them may have (kernels size their plans by `max_kv_len`, which is then this bound)
+    kv_bound: int = 0
 
     @property
     def num_seqs(self) -> int:
@@ -46,8 +49,9 @@ class StepContext:
 
     @property
     def max_kv_len(self) -> int:
-        """The most keys that any request of the step may attend to."""
-        return max(s + q for s, q in zip(self.seq_starts, self.q_lens))
+        """The most keys that any request of the step may attend to (of any step that replays this one's launches,
+        if it is recorded)."""
+        return max(self.kv_bound, max(s + q for s, q in zip(self.seq_starts, self.q_lens)))
 
     def short_requests(self, max_tokens: int) -> tuple[int, int]:
         """(number of leading requests with at most max_tokens tokens, number of their tokens)."""

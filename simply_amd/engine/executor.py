@@ -62,7 +62,8 @@ class Executor:
         # where every recorded step writes its logits, [batch_size, vocab] float32: made at the first such step
         self._graph_logits: torch.Tensor | None = None
         # several decode steps in a row without the host (decode_many): what was drawn in each, and the step count
-        self._records: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None
+        self._records: tuple[torch.Tensor, ...] | None = None
+        self._side_stream = None    # on which results of steps in a row travel to the host while later steps run
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid: Hashable) -> int:
@@ -95,6 +96,7 @@ class Executor:
         this call's result; the recording that follows executes nothing (a mixer that keeps a state of its own would
         otherwise advance it twice)."""
         key = (T, self._context_bucket(ctx))
+        ctx.kv_bound = 1 << key[1]
         out = self._shared_logits()[:T]
         graph = self._graphs.get(key)
         if graph is not None:
@@ -122,8 +124,11 @@ class Executor:
         return graph
 
     @staticmethod
-    def _context_bucket(ctx: StepContext) -> int:
-        return max(ctx.max_kv_len - 1, 0).bit_length()
+    def _context_bucket(ctx: StepContext, ahead: int = 0) -> int:
+        """Recorded steps are kept per power of two of the longest context: a recording serves every step (and, with
+        `ahead` further steps in a row, every run of steps) whose longest context stays within 2 ** bucket keys, and
+        its kernels are planned for that many (`StepContext.kv_bound`)."""
+        return max(ctx.max_kv_len + ahead - 1, 0).bit_length()
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
@@ -144,13 +149,21 @@ class Executor:
         self.cache.mark_issued(wants)
         return logits
 
-    def decode_many(self, entries: Sequence[StepEntry], num_steps: int, sampler) -> tuple[list[list[int]], list[list[float]]]:
-        """`num_steps` decode steps in a row for requests that bring one token each (after
-        `SamplingState.continue_decode`, simply/utils/ragged_paged_attention.py, which loops on the device for up
-        to `intermediate_steps`): every step's drawn tokens are the next step's input, on the device; the host
-        comes back in once, at the end.  `sampler` has been staged (`Sampler.stage`) with one row per entry, in
-        the entries' order.  Pages for all the steps are reserved first (`OutOfPages` if they do not fit).
-        Returns (tokens, log-probabilities), each [num_steps][entry]."""
+    def decode_many(self, entries: Sequence[StepEntry], num_steps: int, sampler, on_step=None, lookahead: int = 8,
+                    chunk: int = 4) -> tuple[list[list[int]], list[list[float]]]:
+        """Up to `num_steps` decode steps in a row for requests that bring one token each (after
+        `SamplingState.continue_decode`, simply/utils/ragged_paged_attention.py:2065-2103, which loops on the device
+        until `until_fn` holds or `intermediate_steps` have run): every step's drawn tokens are the next step's
+        input, on the device.  `sampler` has been staged (`Sampler.stage`) with one row per entry, in the entries'
+        order.  Pages for all the steps are reserved first (`OutOfPages` if they do not fit).
+
+        `on_step(k, tokens, logprobs) -> bool`, if given, is called for every step, in order, as its results reach
+        the host, while up to `lookahead` later steps are already launched (results come out in chunks of `chunk`
+        steps, copied on a stream of their own); once it returns False no further step is launched, and the steps
+        already launched still finish and are delivered.  That is the device loop's `until_fn` with the host's
+        view of the requests: a request that ends runs at most `lookahead + chunk` steps too many, all other rows of
+        those steps are ordinary tokens.  Without `on_step` all steps run and the host comes back in once.
+        Returns (tokens, logprobs) of the steps that ran, each [step][entry]."""
         entries = list(entries)
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
             raise ValueError("decode_many: every request brings one token whose logits are wanted")
@@ -164,6 +177,8 @@ class Executor:
                 tokens.append(toks[:B].tolist())
                 logprobs.append(lps[:B].tolist())
                 sampler.draw_counters[:B] += 1
+                if on_step is not None and not on_step(k, tokens[-1], logprobs[-1]):
+                    break
                 entries = [StepEntry(e.request_id, [t], [0]) for e, t in zip(entries, tokens[-1])]
             return tokens, logprobs
         prepared = self._prepare(entries, reserve_ahead=num_steps)
@@ -174,9 +189,11 @@ class Executor:
             room = max(num_steps, 64)   # recorded graphs hold these addresses: made once for any usual run
             self._records = (torch.empty(room * cap, dtype=torch.int32, device=self.device),
                              torch.empty(room * cap, dtype=torch.float32, device=self.device),
-                             torch.zeros(1, dtype=torch.int32, device=self.device))
+                             torch.zeros(1, dtype=torch.int32, device=self.device),
+                             torch.empty(room * cap, dtype=torch.int32, pin_memory=True),
+                             torch.empty(room * cap, dtype=torch.float32, pin_memory=True))
             self._graphs = {k: v for k, v in self._graphs.items() if k[0] != "many"}  # they hold the old addresses
-        rec_tok, rec_lp, counter = self._records
+        rec_tok, rec_lp, counter, host_tok, host_lp = self._records
         max_steps = rec_tok.numel() // cap
         out_tok, out_lp = rec_tok[:max_steps * B].view(max_steps, B), rec_lp[:max_steps * B].view(max_steps, B)
         from ..kernels import ops
@@ -193,20 +210,59 @@ class Executor:
                                  self.cache.page_size, ctx.groups[g.group_id].slot_mapping)
 
         ops.fill_(counter, 0)
-        key = ("many", B, self._context_bucket(ctx), max_steps, id(sampler), sampler.modes)
+        key = ("many", B, self._context_bucket(ctx, num_steps - 1), max_steps, id(sampler), sampler.modes)
+        ctx.kv_bound = 1 << key[2]
         graph = self._graphs.get(key)
-        done = 0
+        launched = 0
         if graph is None:
             one_step()   # once eagerly (it counts as the first step), then recorded
-            done = 1
+            launched = 1
             graph = self._graphs[key] = self._record(one_step)
-        for _ in range(done, num_steps):
-            graph.replay()
-        tokens = out_tok[:num_steps].tolist()      # waits for the steps
-        logprobs = out_lp[:num_steps].tolist()
+        if on_step is None:
+            lookahead = chunk = num_steps
+        if self._side_stream is None:
+            self._side_stream = torch.cuda.Stream(device=self.device)
+        side = self._side_stream
+        pending: list[tuple[int, int, torch.cuda.Event]] = []   # steps [a, b) on their way to the host
+        copied = read = 0
+        go = True
+        tokens, logprobs = [], []
+
+        def copy_out(upto: int) -> int:
+            reached = torch.cuda.Event()
+            reached.record()
+            side.wait_event(reached)
+            with torch.cuda.stream(side):
+                host_tok[copied * B:upto * B].copy_(rec_tok[copied * B:upto * B], non_blocking=True)
+                host_lp[copied * B:upto * B].copy_(rec_lp[copied * B:upto * B], non_blocking=True)
+                arrived = torch.cuda.Event()
+                arrived.record(side)
+            pending.append((copied, upto, arrived))
+            return upto
+
+        while True:
+            while go and launched < num_steps and launched - read < max(lookahead, 1):
+                if launched - copied >= chunk:
+                    copied = copy_out(launched)
+                graph.replay()
+                launched += 1
+            if copied < launched and (launched - copied >= chunk or not go or launched == num_steps):
+                copied = copy_out(launched)
+            if not pending:
+                break
+            a, b, arrived = pending.pop(0)
+            arrived.synchronize()
+            toks, lps = host_tok[a * B:b * B].view(b - a, B).tolist(), host_lp[a * B:b * B].view(b - a, B).tolist()
+            for k in range(a, b):
+                tokens.append(toks[k - a])
+                logprobs.append(lps[k - a])
+                if on_step is not None and not on_step(k, tokens[-1], logprobs[-1]):
+                    go = False
+            read = b
         for rid, start, _ in wants:
-            self.num_computed[rid] = (self.cache.admission[rid], start + num_steps)
-        self.cache.mark_issued([(rid, start, num_steps) for rid, start, _ in wants])
+            if rid in self.cache.requests:   # (not one that `on_step` has finished and freed meanwhile)
+                self.num_computed[rid] = (self.cache.admission[rid], start + launched)
+        self.cache.mark_issued([(rid, start, launched) for rid, start, _ in wants if rid in self.cache.requests])
         return tokens, logprobs
 
     def _prepare(self, entries: Sequence[StepEntry], reserve_ahead: int = 1):

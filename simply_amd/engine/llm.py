@@ -54,7 +54,7 @@ class LMInterface:
                  activation_dtype: str = "bfloat16", batch_size: int = 8, max_seq_len: int | None = None,
                  page_size: int = 16, max_num_issue_tokens: int = 2048, total_num_pages: int | None = None,
                  seed: int = 0, device: str = "cuda:0", poison_freed_pages: bool = False, use_graphs: bool = True,
-                 library_gemm_min_rows: int | None = None, intermediate_steps: int = 8, _model=None):
+                 library_gemm_min_rows: int | None = None, intermediate_steps: int = 64, _model=None):
         from ..kernels import lib
 
         lib.load()  # fails here, loudly, if the kernel library is missing and cannot be built
@@ -82,8 +82,9 @@ class LMInterface:
         self.scheduler = Scheduler(self.executor.cache, max_num_issue_tokens=self.engine_config.issue_budget,
                                    max_seq_len=max_seq_len)
         self.sampler = Sampler(device, max(batch_size, 1))
-        # decode steps that may run in a row on the device before the host looks at the tokens
-        # (simply/serving/common_flags.py:84 --intermediate_steps)
+        # decode steps that may run in a row without a new scheduling decision (simply/serving/common_flags.py:84
+        # --intermediate_steps, 1024 there, in a loop on the device that ends when a request has ended); here the
+        # host reads every step's tokens a few steps behind the device and ends the run when a request has ended
         self.intermediate_steps = max(1, int(intermediate_steps))
         self.seed = int(seed)
         self._num_requests = 0
@@ -124,21 +125,29 @@ class LMInterface:
         if n > 1:
             reqs = [s.request for s in out.scheduled]
             self.sampler.stage([r.params for r in reqs], [r.seed for r in reqs], [len(r.output_token_ids) for r in reqs])
-            step_tokens, step_logprobs = self.executor.decode_many(entries, n, self.sampler)
+            index = {id(s): i for i, s in enumerate(out.scheduled)}
             live = list(out.scheduled)
-            for k in range(n):
-                index = {id(s): i for i, s in enumerate(out.scheduled)}
+            ran = [0]
+
+            def on_step(k, step_tokens, step_logprobs) -> bool:
+                """A step's results have reached the host (later steps may be running already): the scheduler takes
+                them; the steps in a row go on while nobody has finished."""
+                nonlocal live
+                if not live:
+                    return False
                 now = [Scheduled(s.request, s.start + k, 1, True) for s in live]
-                done = self.scheduler.update(now, [step_tokens[k][index[id(s)]] for s in live],
-                                             [step_logprobs[k][index[id(s)]] for s in live])
-                finished += done
+                done = self.scheduler.update(now, [step_tokens[index[id(s)]] for s in live],
+                                             [step_logprobs[index[id(s)]] for s in live])
+                finished.extend(done)
                 live = [s for s in live if s.request.status is Status.RUNNING]
                 self.stats["steps"] += 1
                 self.stats["tokens"] += len(now)
-                if not live:
-                    break
+                ran[0] += 1
+                return bool(live) and not done
+
+            self.executor.decode_many(entries, n, self.sampler, on_step=on_step)
             if self.step_log is not None:
-                self.step_log.append((n, n * len(entries), time.perf_counter() - t0))
+                self.step_log.append((ran[0], ran[0] * len(entries), time.perf_counter() - t0))
             return finished
         logits = self.executor.step(entries)
         tokens: list = [None] * len(entries)

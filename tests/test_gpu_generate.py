@@ -101,6 +101,22 @@ def test_steps_in_a_row_on_the_device(tmp_path, gpu_lib, dtype):
     out = lm_eos.generate([prompts[0]], sampling_params=[SamplingParams(temperature=0.0, max_decode_steps=37)])[0]
     assert out.output_token_ids == one[0].output_token_ids[:one[0].output_token_ids.index(eos) + 1]
     assert out.finish_reason == "eos"
+    # ... and the others go on as if nothing had happened, although the host learns of the end a few steps late, when
+    # further steps are already launched: a token that two of the four requests draw, at different times, as the end
+    # of sequence for all of them; freed pages are overwritten at once
+    common = [t for t in one[1].output_token_ids[3:] if t in one[2].output_token_ids[3:]]
+    eos = common[0] if common else one[2].output_token_ids[7]
+
+    def with_eos(steps):
+        m = LMInterface(d, intermediate_steps=steps, poison_freed_pages=True, **kw)
+        m.model.spec = dataclasses.replace(m.model.spec, eos_token_ids=(eos,))
+        outs = m.generate(prompts, sampling_params=plist)
+        m.executor.cache.check()
+        return [(o.output_token_ids, o.finish_reason) for o in outs]
+
+    want = with_eos(1)
+    assert sum(reason == "eos" for _, reason in want) >= 1
+    assert with_eos(64) == want and with_eos(3) == want
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
