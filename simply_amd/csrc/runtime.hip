@@ -48,8 +48,8 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
   SA_REQUIRE(algo >= 0 && algo <= 4, "gemm: unknown algorithm %d", algo);
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
-  // up to 16 rows, and up to 32 for products without the gated epilogue and with K below 4608 (measured at the
-  // 2B, 9B and 27B sizes: the few-rows kernel, whose waves read the activations from L2, beats the tiled one with
+  // up to 16 rows, and up to 32 for products without the gated epilogue and with K below 4096 (measured at the
+  // 2B, 9B and 27B sizes: the few-rows kernel, whose waves read the activations from L2, beats the kernels with
   // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower).  Not from 8 rows on
   // against so many weight rows that the tiled kernel fills the GPU without a cut of K (the head over a large
   // vocabulary: 7 % faster at 8 rows, 30 % at 16, 80 % at 32; up to 6 rows the few-rows kernel wins).
@@ -59,7 +59,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   const bool long_k = packed && epilogue != 1 && K >= 24576;
   const bool tiled_first = many_weight_rows || long_k;
   if (algo == 2 ||
-      (algo == 0 && bf16_in && !tiled_first && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4608)))) {
+      (algo == 0 && bf16_in && !tiled_first && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4096)))) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
@@ -72,10 +72,10 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
   // without a cut of K (measured at 32 and 64 rows: 10-20 % faster than the tiled kernel with its sum kernel at the
   // 2B, 9B and 27B sizes)
   const int NW = epilogue == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-  // 64 to 1,536 rows without an epilogue (q/k/v, output and down projections of portions of prompts and of many
-  // decoding requests): the wide kernel with a tile and a cut of K that it chooses for the sizes (at 64 rows of the 2B
-  // down projection 15 us against 23 for the tiled kernel with its cut; at 512 rows 36 against 55)
-  const bool small_wide = epilogue == 0 && M >= 64 && M <= 1536 && N <= 16384;
+  // 17 to 1,536 rows without an epilogue (q/k/v, output and down projections of portions of prompts and of many
+  // decoding requests): the wide kernel with a tile and a cut of K that it chooses for the sizes (2B down projection:
+  // 13 us at 17 rows, 15 at 64, 36 at 512, against 19, 23 and 55 for the tiled kernel with its cut)
+  const bool small_wide = epilogue == 0 && M >= 17 && M <= 1536 && N <= 16384;
   const bool wide_first = !gemm_streams_weights(M, NW, K) || (epilogue == 1 && M > 16) || small_wide;
   if (algo == 4 || (algo == 0 && bf16_in && packed && wide_first)) {
     const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);

@@ -573,7 +573,7 @@ def test_score(V):
     assert got[4] == ops.SCORE_MASKED and got[8] == ops.SCORE_MASKED and got[5] > -1e3   # greedy rows; a plain draw
 
 
-@pytest.mark.parametrize("M", [64, 100, 256, 400, 512, 768, 1100, 1536, 1537])
+@pytest.mark.parametrize("M", [17, 33, 48, 64, 100, 256, 400, 512, 768, 1100, 1536, 1537])
 @pytest.mark.parametrize("N,K", [(4096, 2304), (2304, 2048), (2304, 4608), (1000, 9216), (2304, 9216)])
 def test_gemm_dispatch_at_a_few_hundred_rows(M, N, K):
     """What the dispatcher chooses by itself for portions of a few hundred tokens and for many decoding requests
