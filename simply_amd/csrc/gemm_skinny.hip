@@ -28,7 +28,13 @@ __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<con
 constexpr int kMaxWaves = 16;
 
 // blockDim.x = 64 * NW (NW waves share the K range); a workgroup owns `tile_rows` (16, 8 or 4) rows of W.
-template <int MB, int EPI, bool PACKED, int kUnroll>
+// G (1, 2 or 4; more than 1 only with MB == 1, tiled weights and up to 16 / G rows): a load of activations brings
+// G consecutive chunks of K at once, rows 0 .. 16 / G - 1 of chunk g in the operand's columns g * (16 / G) ..: with
+// few rows the 16 columns of the operand would otherwise hold copies, and the loads of the activations, which come
+// from L2 and are as many as those of the weights, cost a quarter of the kernel (12 against 9 us at the 2B down
+// projection without them).  The product of chunk g is right in its own columns only and has an accumulator of its
+// own; the G accumulators are added up, column group by column group, after the loop.
+template <int MB, int EPI, bool PACKED, int kUnroll, int G>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restrict__ A, int64_t lda,
                                                            const bf16* __restrict__ W, const bf16* __restrict__ W2,
                                                            void* __restrict__ C, int c_dtype, int64_t ldc, int M, int N,
@@ -43,11 +49,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
   const int c0 = static_cast<int>(static_cast<int64_t>(chunks) * wave / NW);
   const int c1 = static_cast<int>(static_cast<int64_t>(chunks) * (wave + 1) / NW);
 
-  floatx4 acc[NP][MB];
+  static_assert(G == 1 || (MB == 1 && PACKED && kUnroll % G == 0), "chunks share a load only for up to 16 rows");
+  floatx4 acc[NP][MB * G];  // [p][mb], or [p][g]
 #pragma unroll
   for (int p = 0; p < NP; ++p)
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[p][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mb = 0; mb < MB * G; ++mb) acc[p][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const bool row_ok = r < tile_rows && n0 + r < N;
   // row-major W: this lane's row, 8 elements at k.  Tiled W (see pack_tiles): tile (n0 / 16), chunk c is one
@@ -97,16 +104,33 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
     // all of them before the first product, and the two register sets never overlap.  Activation rows beyond M are
     // read from row M - 1: their products land in output rows that are not stored.
     const bf16* arow[MB];
+    constexpr int kCols = 16 / G;  // columns of the operand per chunk: lane column r holds row r % kCols of chunk r / kCols
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) arow[mb] = A + static_cast<size_t>(mb * 16 + r < M ? mb * 16 + r : M - 1) * lda + kq * 8;
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = mb * 16 + r % kCols;
+      arow[mb] = A + static_cast<size_t>(m < M ? m : M - 1) * lda + (r / kCols) * 32 + kq * 8;
+    }
     auto load_full = [&](int set, int c) {   // chunks c .. c + kUnroll - 1, all within the wave's range
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         a[set][u] = load_frag(wrow + static_cast<size_t>(c + u) * 512);
         if (EPI == 1) a2[set][u] = load_frag(w2row + static_cast<size_t>(c + u) * 512);
+        if (u % G == 0) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) b[set][u][mb] = load_frag(arow[mb] + (c + u) * 32);
+          for (int mb = 0; mb < MB; ++mb) b[set][u / G][mb] = load_frag(arow[mb] + (c + u) * 32);
+        }
       }
+    };
+    auto mul_full = [&](int set) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const int to = G == 1 ? mb : u % G;
+          acc[0][to] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[set][u], b[set][u / G][mb], acc[0][to], 0, 0, 0);
+          if (EPI == 1)
+            acc[1][to] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[set][u], b[set][u / G][mb], acc[1][to], 0, 0, 0);
+        }
     };
     const int sets = (c1 - c0) / kUnroll;   // full sets; what is left goes through the loads with tests below
     int s = 0;
@@ -117,24 +141,32 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
         // other: it would then wait for them where it has put them, with nothing in flight across iterations)
         load_full(1, c0 + (s + 1) * kUnroll);
         __builtin_amdgcn_sched_barrier(0);
-        mul_set(0);
+        mul_full(0);
         __builtin_amdgcn_sched_barrier(0);
         load_full(0, c0 + (s + 2) * kUnroll);
         __builtin_amdgcn_sched_barrier(0);
-        mul_set(1);
+        mul_full(1);
         __builtin_amdgcn_sched_barrier(0);
       }
       if (sets - s == 2) {
         load_full(1, c0 + (s + 1) * kUnroll);
-        mul_set(0);
-        mul_set(1);
+        mul_full(0);
+        mul_full(1);
       } else {
-        mul_set(0);
+        mul_full(0);
       }
     }
-    if (c0 + sets * kUnroll < c1) {
+    if (c0 + sets * kUnroll < c1) {  // (row m in column m: into the first accumulator, whose columns these are)
       load_set(0, c0 + sets * kUnroll);
       mul_set(0);
+    }
+    if (G > 1) {  // column r of the sum: accumulator g's column g * kCols + r
+#pragma unroll
+      for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int g = 1; g < G; ++g)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[p][0][v] += __shfl(acc[p][g][v], kq * 16 + (r + g * kCols) % 16, kWave);
     }
   } else {
     load_set(0, c0);
@@ -197,7 +229,7 @@ static void choose_shape(int N, int chunks, int planes, int MB, int* tile_rows, 
   *waves = nw;
 }
 
-template <int MB, bool PACKED, int U>
+template <int MB, bool PACKED, int U, int G = 1>
 static void launch_skinny(const bf16* A, int64_t lda, const bf16* W, const bf16* W2, void* C, int c_dtype, int64_t ldc,
                           int M, int N, int K, int epi, int act, float cap, int tile_rows, int waves,
                           hipStream_t stream) {
@@ -206,13 +238,13 @@ static void launch_skinny(const bf16* A, int64_t lda, const bf16* W, const bf16*
   const int threads = waves * kWave;
   const size_t lds = static_cast<size_t>(waves) * (epi == 1 ? 2 : 1) * MB * 16 * 17 * sizeof(float);
   if (epi == 0)
-    gemm_skinny_kernel<MB, 0, PACKED, U><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+    gemm_skinny_kernel<MB, 0, PACKED, U, G><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
                                                                       tile_rows, cap, act);
   else if (epi == 1)
-    gemm_skinny_kernel<MB, 1, PACKED, U><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+    gemm_skinny_kernel<MB, 1, PACKED, U, G><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
                                                                       tile_rows, cap, act);
   else
-    gemm_skinny_kernel<MB, 2, PACKED, U><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
+    gemm_skinny_kernel<MB, 2, PACKED, U, G><<<grid, threads, lds, stream>>>(A, lda, W, W2, C, c_dtype, ldc, M, N, K, chunks,
                                                                       tile_rows, cap, act);
 }
 
@@ -248,7 +280,12 @@ int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void*
     else                                                                                                            \
       launch_skinny<MBV, false, 4>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream); \
   } while (0)
-  if (MB == 1) SA_SKINNY(1);
+  // up to 8 rows against tiled weights: two or four chunks of K to a load of activations
+  if (packed && K % 32 == 0 && tile_rows == 16 && M <= 4)
+    launch_skinny<1, true, 4, 4>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream);
+  else if (packed && K % 32 == 0 && tile_rows == 16 && M <= 8)
+    launch_skinny<1, true, 4, 2>(a, lda, w, w2, C, c_dtype, ldc, M, N, K, epi, act, cap, tile_rows, waves, stream);
+  else if (MB == 1) SA_SKINNY(1);
   else if (MB == 2) SA_SKINNY(2);
   else SA_SKINNY(4);
 #undef SA_SKINNY
