@@ -266,6 +266,37 @@ def test_gemm_skinny(M, N, K):
                                rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 7, 8, 9])
+@pytest.mark.parametrize("N,K", [(48, 64), (100, 96), (2304, 2048), (333, 1120), (1000, 2304), (200, 9216)])
+def test_gemm_skinny_with_tiled_weights_and_few_rows(M, N, K):
+    """Up to 8 rows against tiled weights: one load of activations brings two or four chunks of K, each chunk's product
+    has an accumulator of its own (right in its own columns only) and they are added up after the loop.  Numbers of
+    chunks per wave that are and are not multiples of the four chunks of a register set, rows that do not fill their
+    share of the columns (3 of 4, 5 and 7 of 8), plain, gated and soft-capped; a hot row and a hot column of K show
+    a chunk that lands in the wrong accumulator or a wrong column."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles
+    a, w, w2 = rand((M, K), torch.bfloat16, 58), rand((N, K), torch.bfloat16, 59, 0.05), rand((N, K), torch.bfloat16, 60, 0.05)
+    a[M - 1, K // 3] = 40.0      # one activation that stands out: its chunk must meet its own weights
+    a[0, K - 1] = -30.0
+    t = dict(rtol=2e-2, atol=2e-2)
+    for waves in (0, 1, 3, 8):
+        kw = dict(algo=ops.ALGO_SKINNY, shape=1600 + waves if waves else 0)
+        if waves and waves > K // 64:
+            continue
+        torch.testing.assert_close(ops.gemm(a, pack_tiles(w), **kw).float(), ref.gemm(a, w).float(), **t)
+        torch.testing.assert_close(ops.gemm(a, pack_gate_up(w, w2), **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
+        torch.testing.assert_close(ops.gemm(a, pack_tiles(w), soft_cap=3.0, out_dtype=torch.float32, **kw),
+                                   ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+    # rows of wider rows, as the attention output is
+    big = rand((M, K + 32), torch.bfloat16, 61)
+    torch.testing.assert_close(ops.gemm(big[:, 16:16 + K], pack_tiles(w), algo=ops.ALGO_SKINNY).float(),
+                               ref.gemm(big[:, 16:16 + K], w).float(), **t)
+    # the same rows to the bit whoever else is in the batch, within the kernel's variants of up to 4, up to 8 and more rows
+    if M in (2, 3, 4):
+        assert torch.equal(ops.gemm(a, pack_tiles(w), algo=ops.ALGO_SKINNY)[:1], ops.gemm(a[:1], pack_tiles(w), algo=ops.ALGO_SKINNY))
+
+
 def test_gemm_skinny_refuses_what_it_does_not_take():
     from simply_amd.kernels import ops
     from simply_amd.kernels.lib import KernelError
