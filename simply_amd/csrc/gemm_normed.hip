@@ -43,7 +43,7 @@ struct RotaryArgs {
 };
 
 // NCH: 256-element pieces of a row (K <= 256 * NCH): 10, 14 or 18
-template <int EPI, int NCH>
+template <int EPI, int NCH, bool EXACT>
 __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     const bf16* __restrict__ y, const float* __restrict__ h_in, float* __restrict__ h_out,
     const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_post,
@@ -101,25 +101,37 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
       if (NP == 2) acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[set][u], b, acc[1], 0, 0, 0);
     }
   };
-  // both sets of fragments are asked for before the norms: a wave's share of a tile is two or three sets, so most
-  // of the first tile is on its way while the norms are computed
   const int nseg = (c1 - c0 + kUnroll - 1) / kUnroll;  // sets of fragments per tile for this wave
   // (rows of more than 3584 elements leave no registers for the second set during the norms)
   constexpr bool kBothSetsFirst = NCH <= 14;
-  load_set(0, c0);
-  if (kBothSetsFirst && nseg >= 2) load_set(1, c0 + kUnroll);
-
-  // ---- the two norms, one wave per row.  A lane holds 4 consecutive elements of each 256-element piece of the
-  // row; all loads of a row are issued before the first use, so a row costs one trip to L2.
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
   const bool add = y != nullptr, post = add && w_post != nullptr;
-  for (int m = wave; m < act_rows; m += kWaves) {
-    bf16* dst = act + static_cast<size_t>(m) * pitch;
-    if (m >= M) {
-      for (int d = lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
-      continue;
-    }
-    const size_t rb = static_cast<size_t>(m) * K;
+  if constexpr (EXACT) {
+    // The first fragments of W are asked for before the norms are computed, so that their way from HBM overlaps the
+    // norms; but after the loads of the wave's first row: loads come back in the order in which they were asked
+    // for, and the norms, whose operands lie in L2, must not wait for the weights.  Unconditional loads (a chunk
+    // beyond the wave's share reads the last chunk and is set to zero afterwards): with a branch around a load the
+    // compiler waits for all loads in flight where it next uses one.
+    // (`from`: the tile's first fragment of this lane, through a value that the compiler cannot see through and that
+    // is made after the row's loads: it would otherwise move the weights' loads up to the kernel's start)
+    auto load_first = [&](int set, int c, const bf16* from) __attribute__((always_inline)) {
+  #pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const size_t at = static_cast<size_t>(c + u < chunks ? c + u : chunks - 1) * 512;
+        a[set][u] = load_frag(from + at);
+        if (NP == 2) a2[set][u] = load_frag(from + pair_off + at);
+      }
+    };
+    auto zero_beyond = [&](int set, int c) __attribute__((always_inline)) {
+  #pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        a[set][u] = c + u < c1 ? a[set][u] : zero;
+        if (NP == 2) a2[set][u] = c + u < c1 ? a2[set][u] : zero;
+      }
+    };
+
+    // ---- the two norms, one wave per row.  A lane holds 4 consecutive elements of each 256-element piece of the
+    // row; all loads of a row are issued before the first use, so a row costs one trip to L2.
     // (rows of more than 2560 elements: the norms' scale factors are read where they are used, from L1 after the
     // first row, instead of ahead with the row: the registers do not hold both)
     constexpr bool kAhead = NCH <= 10;
@@ -127,63 +139,195 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     bf16x4 yv[NCH], wpv[kAhead ? NCH : 1], wnv[kAhead ? NCH : 1];
     const bf16* wp16 = static_cast<const bf16*>(w_post);
     const bf16* wn16 = static_cast<const bf16*>(w_next);
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int d = c * 256 + lane * 4;
-      hv[c] = d < K ? *reinterpret_cast<const float4*>(h_in + rb + d) : float4{0.f, 0.f, 0.f, 0.f};
-      yv[c] = (add && d < K) ? *reinterpret_cast<const bf16x4*>(y + rb + d) : bf16x4{};
-      if constexpr (kAhead) {
-        wpv[c] = (post && d < K) ? *reinterpret_cast<const bf16x4*>(wp16 + d) : bf16x4{};
-        wnv[c] = d < K ? *reinterpret_cast<const bf16x4*>(wn16 + d) : bf16x4{};
+    // what is not there (no y, no post-norm) is read from what is, and not used: every load is unconditional
+    const bf16* y_from = add ? y : reinterpret_cast<const bf16*>(h_in);
+    const bf16* wp_from = post ? wp16 : wn16;
+    auto ask_row = [&](int m) __attribute__((always_inline)) {
+      const size_t rb = static_cast<size_t>(m < M ? m : M - 1) * K;
+  #pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int d = c * 256 + lane * 4, at = (EXACT || d < K) ? d : 0;
+        hv[c] = *reinterpret_cast<const float4*>(h_in + rb + at);
+        yv[c] = *reinterpret_cast<const bf16x4*>(y_from + rb + at);
+        if constexpr (kAhead) {
+          wpv[c] = *reinterpret_cast<const bf16x4*>(wp_from + at);
+          wnv[c] = *reinterpret_cast<const bf16x4*>(wn16 + at);
+        }
+      }
+    };
+    // (No branch between a row's loads and their first use: the compiler would move the loads into the branch, behind
+    // the weights' loads.  What a branch would skip is computed and dropped by a select.)
+    auto norm_row = [&](int m) __attribute__((always_inline)) {
+      bf16* dst = act + static_cast<size_t>(m) * pitch;
+      const bool valid = m < M;
+      const size_t rb = static_cast<size_t>(valid ? m : M - 1) * K;
+      auto post_scale = [&](int c, int d) __attribute__((always_inline)) {
+        if constexpr (kAhead) return wpv[c];
+        else return *reinterpret_cast<const bf16x4*>(wp_from + d);
+      };
+      auto next_scale = [&](int c, int d) __attribute__((always_inline)) {
+        if constexpr (kAhead) return wnv[c];
+        else return *reinterpret_cast<const bf16x4*>(wn16 + d);
+      };
+      float ss = 0.f;
+  #pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const bool in_row = EXACT || c * 256 + lane * 4 < K;  // (pieces beyond the row were read from its start: zeros in the sums)
+  #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float v = in_row ? static_cast<float>(yv[c][e]) : 0.f;
+          ss += v * v;
+        }
+      }
+      const float rr = post ? rsqrtf(wave_sum(ss) / static_cast<float>(K) + eps_post) : 1.f;
+      float ss2 = 0.f;
+  #pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int d = c * 256 + lane * 4;
+        const bool in_row = EXACT || d < K;
+        float* h = reinterpret_cast<float*>(&hv[c]);
+        const bf16x4 ws = post_scale(c, in_row ? d : 0);
+  #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float v = static_cast<float>(yv[c][e]);
+          const float t = post ? v * rr * (static_cast<float>(ws[e]) + plus_post) : v;
+          h[e] = in_row ? h[e] + (add ? t : 0.f) : 0.f;
+          ss2 += h[e] * h[e];
+        }
+      }
+      if (add && blockIdx.x == 0 && valid) {
+  #pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          const int d = c * 256 + lane * 4;
+          if (EXACT || d < K) *reinterpret_cast<float4*>(h_out + rb + d) = hv[c];
+        }
+      }
+      const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(K) + eps_next);
+  #pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int d = c * 256 + lane * 4;
+        if (!EXACT && d >= K) continue;
+        const float* h = reinterpret_cast<const float*>(&hv[c]);
+        const bf16x4 ws = next_scale(c, d);
+  #pragma unroll
+        for (int e = 0; e < 4; ++e)
+          dst[d + e] = float_to_bf16(valid ? h[e] * r2 * (static_cast<float>(ws[e]) + plus_next) : 0.f);
+      }
+      for (int d = K + lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
+    };
+    auto zero_row = [&](int m) __attribute__((always_inline)) {
+      bf16* dst = act + static_cast<size_t>(m) * pitch;
+      for (int d = lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
+    };
+    // A wave without a row (fewer rows than waves) asks for no row: the loads of a workgroup's eight waves go through
+    // one path of 64 bytes a clock, and eight copies of a row (a single request decoding) would hold the weights up.
+    int lane_elems = lane * 8;
+    if (wave < M) {
+      ask_row(wave);
+      asm volatile("" : "+v"(lane_elems));
+      const bf16* first_from = wrow - lane * 8 + lane_elems;
+      __builtin_amdgcn_sched_barrier(0);
+      load_first(0, c0, first_from);
+      __builtin_amdgcn_sched_barrier(0);
+      norm_row(wave);
+    } else {
+      load_first(0, c0, wrow);
+      zero_row(wave);
+    }
+    asm volatile("" : "+v"(lane_elems));
+    const bf16* second_from = wrow - lane * 8 + lane_elems;
+    __builtin_amdgcn_sched_barrier(0);
+    if (kBothSetsFirst) load_first(1, c0 + kUnroll, second_from);   // on its way during the further rows, the barrier and the first set's products
+    for (int m = wave + kWaves; m < act_rows; m += kWaves) {
+      if (m < M) {
+        ask_row(m);
+        norm_row(m);
+      } else {
+        zero_row(m);
       }
     }
-    auto post_scale = [&](int c, int d) __attribute__((always_inline)) {
-      if constexpr (kAhead) return wpv[c];
-      else return *reinterpret_cast<const bf16x4*>(wp16 + d);
-    };
-    auto next_scale = [&](int c, int d) __attribute__((always_inline)) {
-      if constexpr (kAhead) return wnv[c];
-      else return *reinterpret_cast<const bf16x4*>(wn16 + d);
-    };
-    if (add) {
-      float rr = 1.f;
-      if (post) {
-        float ss = 0.f;
-#pragma unroll
-        for (int c = 0; c < NCH; ++c)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) ss += static_cast<float>(yv[c][e]) * static_cast<float>(yv[c][e]);
-        rr = rsqrtf(wave_sum(ss) / static_cast<float>(K) + eps_post);
+    zero_beyond(0, c0);
+    if (kBothSetsFirst) zero_beyond(1, c0 + kUnroll);
+  } else {
+    // both sets of fragments are asked for before the norms: a wave's share of a tile is two or three sets, so most
+    // of the first tile is on its way while the norms are computed
+    load_set(0, c0);
+    if (kBothSetsFirst && nseg >= 2) load_set(1, c0 + kUnroll);
+
+    // ---- the two norms, one wave per row.  A lane holds 4 consecutive elements of each 256-element piece of the
+    // row; all loads of a row are issued before the first use, so a row costs one trip to L2.
+    for (int m = wave; m < act_rows; m += kWaves) {
+      bf16* dst = act + static_cast<size_t>(m) * pitch;
+      if (m >= M) {
+        for (int d = lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
+        continue;
       }
-#pragma unroll
+      const size_t rb = static_cast<size_t>(m) * K;
+      // (rows of more than 2560 elements: the norms' scale factors are read where they are used, from L1 after the
+      // first row, instead of ahead with the row: the registers do not hold both)
+      constexpr bool kAhead = NCH <= 10;
+      float4 hv[NCH];
+      bf16x4 yv[NCH], wpv[kAhead ? NCH : 1], wnv[kAhead ? NCH : 1];
+      const bf16* wp16 = static_cast<const bf16*>(w_post);
+      const bf16* wn16 = static_cast<const bf16*>(w_next);
+  #pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int d = c * 256 + lane * 4;
+        hv[c] = d < K ? *reinterpret_cast<const float4*>(h_in + rb + d) : float4{0.f, 0.f, 0.f, 0.f};
+        yv[c] = (add && d < K) ? *reinterpret_cast<const bf16x4*>(y + rb + d) : bf16x4{};
+        if constexpr (kAhead) {
+          wpv[c] = (post && d < K) ? *reinterpret_cast<const bf16x4*>(wp16 + d) : bf16x4{};
+          wnv[c] = d < K ? *reinterpret_cast<const bf16x4*>(wn16 + d) : bf16x4{};
+        }
+      }
+      auto post_scale = [&](int c, int d) __attribute__((always_inline)) {
+        if constexpr (kAhead) return wpv[c];
+        else return *reinterpret_cast<const bf16x4*>(wp16 + d);
+      };
+      auto next_scale = [&](int c, int d) __attribute__((always_inline)) {
+        if constexpr (kAhead) return wnv[c];
+        else return *reinterpret_cast<const bf16x4*>(wn16 + d);
+      };
+      if (add) {
+        float rr = 1.f;
+        if (post) {
+          float ss = 0.f;
+  #pragma unroll
+          for (int c = 0; c < NCH; ++c)
+  #pragma unroll
+            for (int e = 0; e < 4; ++e) ss += static_cast<float>(yv[c][e]) * static_cast<float>(yv[c][e]);
+          rr = rsqrtf(wave_sum(ss) / static_cast<float>(K) + eps_post);
+        }
+  #pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          const int d = c * 256 + lane * 4;
+          if (d >= K) continue;
+          float* h = reinterpret_cast<float*>(&hv[c]);
+          const bf16x4 ws = post ? post_scale(c, d) : bf16x4{};
+  #pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float v = static_cast<float>(yv[c][e]);
+            h[e] += post ? v * rr * (static_cast<float>(ws[e]) + plus_post) : v;
+          }
+          if (blockIdx.x == 0) *reinterpret_cast<float4*>(h_out + rb + d) = hv[c];
+        }
+      }
+      float ss2 = 0.f;
+  #pragma unroll
+      for (int c = 0; c < NCH; ++c) ss2 += hv[c].x * hv[c].x + hv[c].y * hv[c].y + hv[c].z * hv[c].z + hv[c].w * hv[c].w;
+      const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(K) + eps_next);
+  #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         const int d = c * 256 + lane * 4;
         if (d >= K) continue;
-        float* h = reinterpret_cast<float*>(&hv[c]);
-        const bf16x4 ws = post ? post_scale(c, d) : bf16x4{};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float v = static_cast<float>(yv[c][e]);
-          h[e] += post ? v * rr * (static_cast<float>(ws[e]) + plus_post) : v;
-        }
-        if (blockIdx.x == 0) *reinterpret_cast<float4*>(h_out + rb + d) = hv[c];
+        const float* h = reinterpret_cast<const float*>(&hv[c]);
+        const bf16x4 ws = next_scale(c, d);
+  #pragma unroll
+        for (int e = 0; e < 4; ++e)
+          dst[d + e] = float_to_bf16(h[e] * r2 * (static_cast<float>(ws[e]) + plus_next));
       }
+      for (int d = K + lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
     }
-    float ss2 = 0.f;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) ss2 += hv[c].x * hv[c].x + hv[c].y * hv[c].y + hv[c].z * hv[c].z + hv[c].w * hv[c].w;
-    const float r2 = rsqrtf(wave_sum(ss2) / static_cast<float>(K) + eps_next);
-#pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-      const int d = c * 256 + lane * 4;
-      if (d >= K) continue;
-      const float* h = reinterpret_cast<const float*>(&hv[c]);
-      const bf16x4 ws = next_scale(c, d);
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        dst[d + e] = float_to_bf16(h[e] * r2 * (static_cast<float>(ws[e]) + plus_next));
-    }
-    for (int d = K + lane; d < pitch; d += kWave) dst[d] = float_to_bf16(0.f);
   }
   if (!kBothSetsFirst && nseg >= 2) load_set(1, c0 + kUnroll);
   __syncthreads();
@@ -282,7 +426,7 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
   }
 }
 
-template <int EPI, int NCH>
+template <int EPI, int NCH, bool EXACT = false>
 static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype, float eps_post,
                   float plus_post, const void* w_next, int w_next_dtype, float eps_next, float plus_next, const bf16* W,
                   void* C, int c_dtype, int64_t ldc, int M, int N, int K, float cap, int activation,
@@ -290,7 +434,7 @@ static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_
   const int act_rows = M <= 8 ? 8 : 16;
   const size_t lds = static_cast<size_t>(act_rows) * (K + 8) * sizeof(bf16) +
                      static_cast<size_t>(kWaves) * ((EPI == 1 || EPI == 3) ? 2 : 1) * 16 * 17 * sizeof(float);
-  auto kernel = gemm_normed_kernel<EPI, NCH>;
+  auto kernel = gemm_normed_kernel<EPI, NCH, EXACT>;
   if (lds > 64 * 1024) {
     static bool raised = false;  // per instantiation
     if (!raised) {
@@ -343,8 +487,16 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
 #define SA_NORMED(EPI, NCH)                                                                                      \
   return normed::launch<EPI, NCH>(yb, h_in, h_out, w_post, w_post_dtype, eps_post, pp, w_next, w_next_dtype, eps_next, \
                                   pn, w, C, c_dtype, ldc, M, N, K, cap, activation, normed::RotaryArgs{}, stream)
+#define SA_NORMED_EXACT(EPI, NCH)                                                                                  \
+  return normed::launch<EPI, NCH, true>(yb, h_in, h_out, w_post, w_post_dtype, eps_post, pp, w_next, w_next_dtype,   \
+                                        eps_next, pn, w, C, c_dtype, ldc, M, N, K, cap, activation, normed::RotaryArgs{}, \
+                                        stream)
 #define SA_NORMED_K(EPI)          \
   do {                            \
+    /* rows of a whole number of 256-element pieces, up to 2560 wide: the prologue without per-piece tests */     \
+    if (K == 2048) SA_NORMED_EXACT(EPI, 8);                                                                        \
+    if (K == 2304) SA_NORMED_EXACT(EPI, 9);                                                                        \
+    if (K == 2560) SA_NORMED_EXACT(EPI, 10);                                                                       \
     if (K <= 2560) SA_NORMED(EPI, 10); \
     if (K <= 3584) SA_NORMED(EPI, 14); \
     SA_NORMED(EPI, 18);           \
@@ -353,6 +505,7 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
   if (epilogue == 1) SA_NORMED_K(1);
   SA_NORMED_K(2);
 #undef SA_NORMED_K
+#undef SA_NORMED_EXACT
 #undef SA_NORMED
 }
 
@@ -387,6 +540,15 @@ extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_
   return normed::launch<3, NCH>(static_cast<const bf16*>(y), h_in, h_out, w_post, w_post_dtype, eps_post,             \
                                 plus_one_post ? 1.f : 0.f, w_next, w_next_dtype, eps_next, plus_one_next ? 1.f : 0.f, \
                                 static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, 0.f, 0, rot, stream)
+#define SA_ROTARY_EXACT(NCH)                                                                                        \
+  return normed::launch<3, NCH, true>(static_cast<const bf16*>(y), h_in, h_out, w_post, w_post_dtype, eps_post,        \
+                                      plus_one_post ? 1.f : 0.f, w_next, w_next_dtype, eps_next,                       \
+                                      plus_one_next ? 1.f : 0.f, static_cast<const bf16*>(W), C, c_dtype, ldc, M, N, K, \
+                                      0.f, 0, rot, stream)
+  if (K == 2048) SA_ROTARY_EXACT(8);
+  if (K == 2304) SA_ROTARY_EXACT(9);
+  if (K == 2560) SA_ROTARY_EXACT(10);
+#undef SA_ROTARY_EXACT
   if (K <= 2560) SA_ROTARY(10);
   if (K <= 3584) SA_ROTARY(14);
   SA_ROTARY(18);

@@ -664,9 +664,9 @@ def test_gated_activations_in_every_product_kernel(M, activation):
         ops.gemm(a, tg, activation=3)
 
 
-@pytest.mark.parametrize("M", [1, 8, 13, 16])
-@pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (3584, 512), (4608, 64), (4640, 64), (96, 40),
-                                 (72, 64)])
+@pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16])
+@pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (2048, 200), (3584, 512), (4608, 64), (4640, 64),
+                                 (96, 40), (72, 64)])
 def test_gemm_normed(M, K, N):
     """Residual sum, two norms and the product in one kernel against the separate references."""
     from simply_amd.kernels import ops
