@@ -322,7 +322,7 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
   // thread, then group 0 adds the groups up in order.  The first kAhead ranges of a thread are asked for here,
   // before the weights are known: their loads are under way together with those of the maxima and sums above, so
   // the kernel waits for memory once, not twice.
-  constexpr int kAhead = 8;
+  constexpr int kAhead = 16;
   const int quarter = HD / 4, parts = 256 / quarter;
   const int c = tid % quarter, part = tid / quarter;
   float4 ahead[kAhead];
@@ -399,11 +399,11 @@ int paged_attention_decode_ranges(int seq_count, int Kh, int window, int max_kv_
   int KS = num_splits;
   if (KS <= 0) {
     KS = (256 + units / 2) / units;               // about one workgroup per CU: longer ranges amortise the set-up
-    const int cap_by_work = (max_tiles + 3) / 4;  // at least 4 tiles (128 keys) per workgroup
+    const int cap_by_work = (max_tiles + 1) / 2;  // at least 2 tiles (64 keys) per workgroup
     if (KS > cap_by_work) KS = cap_by_work;
-    // ... and for one or two requests no more than 32 ranges, or ranges of 16 tiles: every range costs the second
-    // kernel a row to add up (one request of 8,192 keys at the 2B shape: 19.0 us with 32 ranges, 20.6 with 64)
-    const int cap_by_merge = max_tiles / 16 > 32 ? max_tiles / 16 : 32;
+    // ... and no more than 64 ranges, or ranges of 16 tiles: a thread of the second kernel has 16 ranges' partial
+    // results on their way at once (one request of 8,192 keys at the 2B shape: 18.5 us with 64 ranges, 19.4 with 32)
+    const int cap_by_merge = max_tiles / 16 > 64 ? max_tiles / 16 : 64;
     if (KS > cap_by_merge) KS = cap_by_merge;
   }
   // (a workgroup looks up the pages of at most kMaxRangeSubTiles sub-tiles: two more than its share of the tiles has)
