@@ -22,7 +22,6 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 namespace normed {
 
 constexpr int kWaves = 8;
-constexpr int kUnroll = 4;
 constexpr int kMaxGroups = 256;  // one workgroup per compute unit; each takes the same number of tiles, or one fewer
 
 __device__ inline bf16x8 load_frag(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -43,7 +42,9 @@ struct RotaryArgs {
 };
 
 // NCH: 256-element pieces of a row (K <= 256 * NCH): 10, 14 or 18
-template <int EPI, int NCH, bool EXACT>
+// kUnroll: fragments of a register set (chunks of 32 columns of K whose loads a wave issues together); 4: sets of 5,
+// two to a tile at the 2B width instead of three, were no faster (q/k/v 8.8 against 8.1 us at one row)
+template <int EPI, int NCH, bool EXACT, int kUnroll>
 __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
     const bf16* __restrict__ y, const float* __restrict__ h_in, float* __restrict__ h_out,
     const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_post,
@@ -426,7 +427,7 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
   }
 }
 
-template <int EPI, int NCH, bool EXACT = false>
+template <int EPI, int NCH, bool EXACT = false, int kUnroll = 4>
 static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype, float eps_post,
                   float plus_post, const void* w_next, int w_next_dtype, float eps_next, float plus_next, const bf16* W,
                   void* C, int c_dtype, int64_t ldc, int M, int N, int K, float cap, int activation,
@@ -434,7 +435,7 @@ static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_
   const int act_rows = M <= 8 ? 8 : 16;
   const size_t lds = static_cast<size_t>(act_rows) * (K + 8) * sizeof(bf16) +
                      static_cast<size_t>(kWaves) * ((EPI == 1 || EPI == 3) ? 2 : 1) * 16 * 17 * sizeof(float);
-  auto kernel = gemm_normed_kernel<EPI, NCH, EXACT>;
+  auto kernel = gemm_normed_kernel<EPI, NCH, EXACT, kUnroll>;
   if (lds > 64 * 1024) {
     static bool raised = false;  // per instantiation
     if (!raised) {
