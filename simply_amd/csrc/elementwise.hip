@@ -359,6 +359,12 @@ __global__ __launch_bounds__(256) void rope_cache_write_rows_kernel(
 // portion that starts at a page's edge), writes each dimension's 16 keys as two 16-byte pieces instead of 16
 // scattered 2-byte ones.
 constexpr int kRotTokens = 8, kValTokens = 16, kWideMaxHalf = 256;
+// two floats rounded to bfloat16 (to nearest even, one instruction for both), the first in the low half
+__device__ inline uint32_t pack_bf16(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  const bf16x2 p = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+  return __builtin_bit_cast(uint32_t, p);
+}
 __global__ __launch_bounds__(256) void rope_cache_write_wide_kernel(
     bf16* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ timescale,
     float inv_scale_factor, float q_div, const int64_t* __restrict__ slot_mapping, bf16* __restrict__ k_pages,
@@ -378,44 +384,70 @@ __global__ __launch_bounds__(256) void rope_cache_write_wide_kernel(
     __syncthreads();
     const int groups = half / 8, per_token = (H + K) * groups;
     const bool tiled = keys_tiled(page_size, hd);
-    for (int item = tid; item < nt * per_token; item += blockDim.x) {
-      const int j = item / per_token, head = (item % per_token) / groups, i = (item % groups) * 8;
-      bf16* src = qkv + static_cast<size_t>(t0 + j) * row_stride + static_cast<size_t>(head) * hd + i;
-      bf16* to1 = src;
-      bf16* to2 = src + half;
-      if (head >= H) {
-        const int64_t slot = k_pages != nullptr ? slot_mapping[t0 + j] : -1;
-        if (slot < 0) continue;
-        const int koff = static_cast<int>(slot % page_size);
-        bf16* page = k_pages + ((slot / page_size) * K + (head - H)) * page_size * hd;
-        to1 = page + key_index(tiled, page_size, hd, koff, i);
-        to2 = page + key_index(tiled, page_size, hd, koff, i + half);
-      }
-      const uint4 a = *reinterpret_cast<const uint4*>(src), b = *reinterpret_cast<const uint4*>(src + half);
-      const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
-      uint32_t o1[4], o2[4];
-      const float* sj = sn + j * half + i;
-      const float* cj = cs + j * half + i;
+    // Six items a thread at a time (all that a thread has at the usual sizes), their loads asked for together: one
+    // after the other they are six trips to memory in a row.  The query scale is a multiplication by the reciprocal:
+    // a division per rotated value was a third of the arithmetic, which is most of a block's time (timestamps: 8.9
+    // of 10.6 us before, 6 of 7.7 after).
+    constexpr int kBatch = 6;
+    const float q_mul = 1.f / q_div;
+    const int total = nt * per_token;
+    for (int first = tid; first < total; first += blockDim.x * kBatch) {
+      uint4 av[kBatch], bv[kBatch];
+      bf16* to1[kBatch];
+      bf16* to2[kBatch];
+      int jj[kBatch], ii[kBatch];
+      float scale[kBatch];
+      bool ok[kBatch];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        float r1[2], r2[2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const float x1 = __uint_as_float(e ? aw[w] & 0xffff0000u : aw[w] << 16);
-          const float x2 = __uint_as_float(e ? bw[w] & 0xffff0000u : bw[w] << 16);
-          const float s = sj[2 * w + e], c = cj[2 * w + e];
-          r1[e] = x1 * c - x2 * s;
-          r2[e] = x2 * c + x1 * s;
-          if (head < H) {
-            r1[e] = r1[e] / q_div;
-            r2[e] = r2[e] / q_div;
+      for (int u = 0; u < kBatch; ++u) {
+        const int item = first + u * static_cast<int>(blockDim.x);
+        ok[u] = item < total;
+        const int it = ok[u] ? item : 0;
+        const int j = it / per_token, head = (it % per_token) / groups, i = (it % groups) * 8;
+        bf16* src = qkv + static_cast<size_t>(t0 + j) * row_stride + static_cast<size_t>(head) * hd + i;
+        jj[u] = j;
+        ii[u] = i;
+        scale[u] = head < H ? q_mul : 1.f;
+        to1[u] = src;
+        to2[u] = src + half;
+        if (head >= H) {
+          const int64_t slot = k_pages != nullptr ? slot_mapping[t0 + j] : -1;
+          if (slot < 0) {
+            ok[u] = false;
+          } else {
+            const int koff = static_cast<int>(slot % page_size);
+            bf16* page = k_pages + ((slot / page_size) * K + (head - H)) * page_size * hd;
+            to1[u] = page + key_index(tiled, page_size, hd, koff, i);
+            to2[u] = page + key_index(tiled, page_size, hd, koff, i + half);
           }
         }
-        o1[w] = static_cast<uint32_t>(float_to_bf16(r1[0]).bits) | (static_cast<uint32_t>(float_to_bf16(r1[1]).bits) << 16);
-        o2[w] = static_cast<uint32_t>(float_to_bf16(r2[0]).bits) | (static_cast<uint32_t>(float_to_bf16(r2[1]).bits) << 16);
+        av[u] = *reinterpret_cast<const uint4*>(src);
+        bv[u] = *reinterpret_cast<const uint4*>(src + half);
       }
-      *reinterpret_cast<uint4*>(to1) = uint4{o1[0], o1[1], o1[2], o1[3]};
-      *reinterpret_cast<uint4*>(to2) = uint4{o2[0], o2[1], o2[2], o2[3]};
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        if (!ok[u]) continue;
+        const uint32_t aw[4] = {av[u].x, av[u].y, av[u].z, av[u].w}, bw[4] = {bv[u].x, bv[u].y, bv[u].z, bv[u].w};
+        uint32_t o1[4], o2[4];
+        const float* sj = sn + jj[u] * half + ii[u];
+        const float* cj = cs + jj[u] * half + ii[u];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float r1[2], r2[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const float x1 = __uint_as_float(e ? aw[w] & 0xffff0000u : aw[w] << 16);
+            const float x2 = __uint_as_float(e ? bw[w] & 0xffff0000u : bw[w] << 16);
+            const float s = sj[2 * w + e], c = cj[2 * w + e];
+            r1[e] = (x1 * c - x2 * s) * scale[u];
+            r2[e] = (x2 * c + x1 * s) * scale[u];
+          }
+          o1[w] = pack_bf16(r1[0], r1[1]);
+          o2[w] = pack_bf16(r2[0], r2[1]);
+        }
+        *reinterpret_cast<uint4*>(to1[u]) = uint4{o1[0], o1[1], o1[2], o1[3]};
+        *reinterpret_cast<uint4*>(to2[u]) = uint4{o2[0], o2[1], o2[2], o2[3]};
+      }
     }
     return;
   }
