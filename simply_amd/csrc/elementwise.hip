@@ -374,63 +374,60 @@ __global__ __launch_bounds__(256) void rope_cache_write_wide_kernel(
   if (static_cast<int>(blockIdx.x) < rot_blocks) {
     const int t0 = blockIdx.x * kRotTokens;
     const int nt = T - t0 < kRotTokens ? T - t0 : kRotTokens;
-    for (int idx = tid; idx < nt * half; idx += blockDim.x) {
-      float s = 0.f, c = 1.f;
-      if (timescale != nullptr)
-        sincosf(static_cast<float>(positions[t0 + idx / half]) / timescale[idx % half] * inv_scale_factor, &s, &c);
-      sn[idx] = s;
-      cs[idx] = c;
-    }
-    __syncthreads();
     const int groups = half / 8, per_token = (H + K) * groups;
     const bool tiled = keys_tiled(page_size, hd);
     // Six items a thread at a time (all that a thread has at the usual sizes), their loads asked for together: one
-    // after the other they are six trips to memory in a row.  The query scale is a multiplication by the reciprocal:
-    // a division per rotated value was a third of the arithmetic, which is most of a block's time (timestamps: 8.9
-    // of 10.6 us before, 6 of 7.7 after).
+    // after the other they are six trips to memory in a row; and the first six before the sines and cosines are
+    // computed, which takes as long as the loads are under way.  The query scale is a multiplication by the
+    // reciprocal: a division per rotated value was a third of the arithmetic, which is most of a block's time
+    // (timestamps: 8.9 of 10.6 us before, 6 of 7.7 after).
     constexpr int kBatch = 6;
     const float q_mul = 1.f / q_div;
     const int total = nt * per_token;
-    for (int first = tid; first < total; first += blockDim.x * kBatch) {
+    struct Batch {
       uint4 av[kBatch], bv[kBatch];
       bf16* to1[kBatch];
       bf16* to2[kBatch];
       int jj[kBatch], ii[kBatch];
       float scale[kBatch];
       bool ok[kBatch];
+    };
+    auto ask = [&](int first, Batch& b) __attribute__((always_inline)) {
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
         const int item = first + u * static_cast<int>(blockDim.x);
-        ok[u] = item < total;
-        const int it = ok[u] ? item : 0;
+        b.ok[u] = item < total;
+        const int it = b.ok[u] ? item : 0;
         const int j = it / per_token, head = (it % per_token) / groups, i = (it % groups) * 8;
         bf16* src = qkv + static_cast<size_t>(t0 + j) * row_stride + static_cast<size_t>(head) * hd + i;
-        jj[u] = j;
-        ii[u] = i;
-        scale[u] = head < H ? q_mul : 1.f;
-        to1[u] = src;
-        to2[u] = src + half;
+        b.jj[u] = j;
+        b.ii[u] = i;
+        b.scale[u] = head < H ? q_mul : 1.f;
+        b.to1[u] = src;
+        b.to2[u] = src + half;
         if (head >= H) {
           const int64_t slot = k_pages != nullptr ? slot_mapping[t0 + j] : -1;
           if (slot < 0) {
-            ok[u] = false;
+            b.ok[u] = false;
           } else {
             const int koff = static_cast<int>(slot % page_size);
             bf16* page = k_pages + ((slot / page_size) * K + (head - H)) * page_size * hd;
-            to1[u] = page + key_index(tiled, page_size, hd, koff, i);
-            to2[u] = page + key_index(tiled, page_size, hd, koff, i + half);
+            b.to1[u] = page + key_index(tiled, page_size, hd, koff, i);
+            b.to2[u] = page + key_index(tiled, page_size, hd, koff, i + half);
           }
         }
-        av[u] = *reinterpret_cast<const uint4*>(src);
-        bv[u] = *reinterpret_cast<const uint4*>(src + half);
+        b.av[u] = *reinterpret_cast<const uint4*>(src);
+        b.bv[u] = *reinterpret_cast<const uint4*>(src + half);
       }
+    };
+    auto rotate = [&](const Batch& b) __attribute__((always_inline)) {
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        if (!ok[u]) continue;
-        const uint32_t aw[4] = {av[u].x, av[u].y, av[u].z, av[u].w}, bw[4] = {bv[u].x, bv[u].y, bv[u].z, bv[u].w};
+        if (!b.ok[u]) continue;
+        const uint32_t aw[4] = {b.av[u].x, b.av[u].y, b.av[u].z, b.av[u].w}, bw[4] = {b.bv[u].x, b.bv[u].y, b.bv[u].z, b.bv[u].w};
         uint32_t o1[4], o2[4];
-        const float* sj = sn + jj[u] * half + ii[u];
-        const float* cj = cs + jj[u] * half + ii[u];
+        const float* sj = sn + b.jj[u] * half + b.ii[u];
+        const float* cj = cs + b.jj[u] * half + b.ii[u];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           float r1[2], r2[2];
@@ -439,15 +436,30 @@ __global__ __launch_bounds__(256) void rope_cache_write_wide_kernel(
             const float x1 = __uint_as_float(e ? aw[w] & 0xffff0000u : aw[w] << 16);
             const float x2 = __uint_as_float(e ? bw[w] & 0xffff0000u : bw[w] << 16);
             const float s = sj[2 * w + e], c = cj[2 * w + e];
-            r1[e] = (x1 * c - x2 * s) * scale[u];
-            r2[e] = (x2 * c + x1 * s) * scale[u];
+            r1[e] = (x1 * c - x2 * s) * b.scale[u];
+            r2[e] = (x2 * c + x1 * s) * b.scale[u];
           }
           o1[w] = pack_bf16(r1[0], r1[1]);
           o2[w] = pack_bf16(r2[0], r2[1]);
         }
-        *reinterpret_cast<uint4*>(to1[u]) = uint4{o1[0], o1[1], o1[2], o1[3]};
-        *reinterpret_cast<uint4*>(to2[u]) = uint4{o2[0], o2[1], o2[2], o2[3]};
+        *reinterpret_cast<uint4*>(b.to1[u]) = uint4{o1[0], o1[1], o1[2], o1[3]};
+        *reinterpret_cast<uint4*>(b.to2[u]) = uint4{o2[0], o2[1], o2[2], o2[3]};
       }
+    };
+    Batch batch;
+    ask(tid, batch);
+    for (int idx = tid; idx < nt * half; idx += blockDim.x) {
+      float s = 0.f, c = 1.f;
+      if (timescale != nullptr)
+        sincosf(static_cast<float>(positions[t0 + idx / half]) / timescale[idx % half] * inv_scale_factor, &s, &c);
+      sn[idx] = s;
+      cs[idx] = c;
+    }
+    __syncthreads();
+    rotate(batch);
+    for (int first = tid + static_cast<int>(blockDim.x) * kBatch; first < total; first += blockDim.x * kBatch) {
+      ask(first, batch);
+      rotate(batch);
     }
     return;
   }
