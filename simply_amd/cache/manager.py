@@ -259,6 +259,7 @@ class CacheManager:
         self.views: list[CacheView] = []
         self._group_entries: dict[int, list[int]] = {}
         self._device_tables: dict[int, torch.Tensor] = {}
+        self._stage_host = self._stage_dev = self._stage_done = None  # what `sync_tables` sends its rows through
         by_need: dict[PagedKVNeed, CacheGroup] = {}
         max_blocks = ceil_div(self.max_seq_len, self.page_size)
         for i, (need, cache_from) in enumerate(needs):
@@ -455,13 +456,38 @@ class CacheManager:
             raise CacheError(f"request {rid!r}: keys [{lo}, {start + q_len}) are not all held in group {group_id}")
 
     def sync_tables(self) -> dict[int, torch.Tensor]:
-        """Brings the device copies of the block tables up to date."""
-        for g in self.groups:
-            if self.device is not None and g.dirty_slots:
-                dev = self._device_tables[g.group_id]
+        """Brings the device copies of the block tables up to date.  The rows that have changed go through a pinned
+        block in one copy that does not wait for the device, and are put into place there: a step's launches can
+        then follow the last step's without the stream running empty in between."""
+        dirty = [g for g in self.groups if g.dirty_slots] if self.device is not None else []
+        if dirty and torch.device(self.device).type != "cuda":
+            for g in dirty:
                 rows = sorted(g.dirty_slots)
-                idx = torch.as_tensor(rows, dtype=torch.long)
-                dev.index_copy_(0, idx.to(self.device), torch.from_numpy(g.table[rows]).to(self.device))
+                self._device_tables[g.group_id].index_copy_(0, torch.as_tensor(rows, dtype=torch.long),
+                                                            torch.from_numpy(g.table[rows]))
+        elif dirty:
+            if self._stage_host is None:
+                ints = sum(self.num_slots * (g.max_blocks + 3) for g in self.groups)
+                self._stage_host = torch.empty(ints, dtype=torch.int32, pin_memory=True)
+                self._stage_dev = torch.empty(ints, dtype=torch.int32, device=self.device)
+                self._stage_done = torch.cuda.Event()
+            self._stage_done.synchronize()  # the last copy out of the pinned block has finished
+            host, dev = self._stage_host.numpy(), self._stage_dev
+            at, parts = 0, []
+            for g in dirty:
+                rows = sorted(g.dirty_slots)
+                n, body = len(rows), at + 2 * len(rows)  # the rows' numbers as 64-bit integers, then the rows
+                host[at:body].view(np.int64)[:] = rows
+                host[body:body + n * g.max_blocks].reshape(n, g.max_blocks)[:] = g.table[rows]
+                parts.append((g, at, n, body))
+                at = body + n * g.max_blocks
+                at += at & 1
+            dev[:at].copy_(self._stage_host[:at], non_blocking=True)
+            self._stage_done.record()
+            for g, first, n, body in parts:
+                self._device_tables[g.group_id].index_copy_(0, dev[first:body].view(torch.int64),
+                                                            dev[body:body + n * g.max_blocks].view(n, g.max_blocks))
+        for g in self.groups:
             g.dirty_slots.clear()
         return self._device_tables
 

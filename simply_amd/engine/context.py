@@ -7,8 +7,9 @@ segment ids and absolute segment positions).  The description is independent of 
 from __future__ import annotations
 
 import dataclasses
-from typing import Hashable
+from typing import Callable, Hashable
 
+import numpy as np
 import torch
 
 
@@ -38,6 +39,9 @@ class StepContext:
     #: set for a step whose launches are recorded and replayed for later steps: the most keys that any step that
     #: replays them may have (kernels size their plans by `max_kv_len`, which is then this bound)
     kv_bound: int = 0
+    #: brings an integer array that a part makes for the step to the device without waiting for the device (the
+    #: executor's pinned block); None: a plain copy
+    to_device: Callable[[np.ndarray], torch.Tensor] | None = None
 
     @property
     def num_seqs(self) -> int:
@@ -78,11 +82,15 @@ class StepContext:
                 if q <= tokens_per_unit:
                     few.append((slot, first, q, start))
                     continue
-                for o in range(0, q, tokens_per_unit):
-                    many.append((slot, first + o, min(tokens_per_unit, q - o), start + o))
-                while len(many) % group:
-                    many.append((slot, first + q, 0, start + q))
-            units = torch.tensor(few + many, dtype=torch.int32).to(self.positions.device, non_blocking=True)
-            cached = (units, len(few), len(many), tokens_per_unit)
+                count = -(-q // tokens_per_unit)
+                at = np.minimum(np.arange(-(-count // group) * group) * tokens_per_unit, q)
+                block = np.empty((len(at), 4), dtype=np.int32)
+                block[:, 0], block[:, 1], block[:, 3] = slot, first + at, start + at
+                block[:, 2] = np.minimum(q - at, tokens_per_unit)
+                many.append(block)
+            rows = np.concatenate([np.asarray(few, dtype=np.int32).reshape(-1, 4)] + many)
+            units = self.to_device(rows) if self.to_device is not None else \
+                torch.from_numpy(rows).to(self.positions.device)
+            cached = (units, len(few), len(rows) - len(few), tokens_per_unit)
             self._units[key] = cached
         return cached

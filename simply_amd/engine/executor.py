@@ -55,6 +55,13 @@ class Executor:
         self._host = torch.empty(self._words, dtype=torch.int32, pin_memory=self._on_gpu)
         self._dev = torch.empty(self._words, dtype=torch.int32, device=self.device)
         self._copied = torch.cuda.Event() if self._on_gpu else None
+        # a second pinned block for integer arrays that parts make for a step (the units of an attention kernel):
+        # a step's arrays lie one behind the other in it
+        self._extra_words = 4 * (cap + 8 * config.batch_size)
+        self._extra_host = torch.empty(self._extra_words, dtype=torch.int32, pin_memory=True) if self._on_gpu else None
+        self._extra_dev = torch.empty(self._extra_words, dtype=torch.int32, device=self.device) if self._on_gpu else None
+        self._extra_copied = torch.cuda.Event() if self._on_gpu else None
+        self._extra_used = 0
         # decode-only steps (one token per request) are captured once per number of requests and order of magnitude
         # of the context (the attention kernels choose their cut of the keys when they are recorded) and replayed
         self._graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
@@ -265,6 +272,22 @@ class Executor:
         self.cache.mark_issued([(rid, start, launched) for rid, start, _ in wants if rid in self.cache.requests])
         return tokens, logprobs
 
+    def _to_device(self, array: np.ndarray) -> torch.Tensor:
+        """An int32 array of the step on the device, through the pinned block if it still fits: the copy does not
+        wait for the device, so the stream keeps its lead over the launches."""
+        words = array.size
+        if not self._on_gpu or array.dtype != np.int32 or self._extra_used + words > self._extra_words:
+            return torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
+        at = self._extra_used
+        if at == 0:
+            self._extra_copied.synchronize()  # the last step's copies out of the block have finished
+        self._extra_used = at + words
+        self._extra_host.numpy()[at:at + words] = array.reshape(-1)
+        dev = self._extra_dev[at:at + words]
+        dev.copy_(self._extra_host[at:at + words], non_blocking=True)
+        self._extra_copied.record()
+        return dev.view(array.shape)
+
     def _prepare(self, entries: Sequence[StepEntry], reserve_ahead: int = 1):
         """Checks the entries, reserves their pages (for `reserve_ahead` tokens where an entry brings one token
         and more steps follow without the host), lays the step out in the staging buffer and copies it to the
@@ -348,7 +371,8 @@ class Executor:
         ctx = StepContext(dtype=self.dtype, num_tokens=T, positions=dev[cap:cap + T], token_seq=dev[2 * cap:2 * cap + T],
                           seq_meta=dev[self._meta_at:self._meta_at + 4 * len(entries)].view(len(entries), 4),
                           groups=groups, request_ids=ctx_ids, seq_slots=ctx_slots, seq_starts=ctx_starts, q_lens=ctx_q,
-                          cu_q_lens=cu)
+                          cu_q_lens=cu, to_device=self._to_device)
+        self._extra_used = 0
         logit_rows = dev[3 * cap:3 * cap + R] if R else None
         return T, R, ctx, logit_rows, [(rid, start, len(e.tokens)) for (rid, start, _), e in zip(wants, entries)], \
             len(entries)
