@@ -21,6 +21,27 @@ struct SeqMeta {
 
 __device__ inline __bf16 to_bf16_raw(float f) { return static_cast<__bf16>(f); }
 
+// A value of the lanes l, l ^ 16, l ^ 32 and l ^ 48 combined (the four lanes that share a row of an MFMA result),
+// in every one of them, with gfx950's swaps of 16- and 32-lane rows between two registers: one instruction each
+// on the vector unit, where a shuffle goes through the LDS crossbar and waits behind the operand reads queued there.
+// v_permlane16_swap exchanges rows 1 and 3 of its first operand with rows 0 and 2 of its second, v_permlane32_swap
+// the upper half of the first with the lower half of the second: from two copies of x come [x0 x0 x2 x2] and
+// [x1 x1 x3 x3], then the halves.
+template <typename Op>
+__device__ __forceinline__ float over_row_lanes(float x, Op op) {
+  const unsigned u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned v = __float_as_uint(op(__uint_as_float(a[0]), __uint_as_float(a[1])));
+  const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return op(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float max_over_row_lanes(float x) {
+  return over_row_lanes(x, [](float a, float b) { return fmaxf(a, b); });
+}
+__device__ __forceinline__ float sum_over_row_lanes(float x) {
+  return over_row_lanes(x, [](float a, float b) { return a + b; });
+}
+
 // Partial results of key ranges lie in the workspace as [unit * Kh + kh][range][16 rows][hd + kRowExtra] floats:
 // the unnormalised output, then the maximum and the sum of the row (and two unused words: rows stay 16-byte
 // aligned).  Adds them up, range by range in order, into `out`.  max_q_len: the most tokens in a unit.

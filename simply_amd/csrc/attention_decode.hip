@@ -183,8 +183,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
         p[t][v] = x;
         mx = fmaxf(mx, x);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    mx = max_over_row_lanes(mx);
     const float m_new = fmaxf(m_run, mx);
     // a row that has seen no visible key yet keeps m = -inf; exp(-inf - -inf) must not appear
     const float alpha = m_new == -INFINITY ? 1.f : __expf(m_run - m_new);
@@ -237,8 +236,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 
   // ---- merge the four waves in two rounds through LDS (waves 2, 3 into 0, 1; then 1 into 0).
   // acc[db][v] is O^T[d = db * 16 + 4 * grp + v][row r].
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
+  l_run = sum_over_row_lanes(l_run);
   auto put = [&](int slot) {
 #pragma unroll
     for (int db = 0; db < NDB; ++db)

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int r = lane % 16, grp = lane / 16;
-  const int split = blockIdx.x, num_splits = gridDim.x, kh = blockIdx.y;
+  const int split = blockIdx.y, num_splits = gridDim.y, kh = blockIdx.x;
   // later units of a prompt see more keys: they are started first
   const int group = gridDim.z - 1 - blockIdx.z;
   const int u0 = unit_begin + group * GROUP;
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // one tile from LDS, for this wave's rows
+  Pages next;  // the pages of the tile after the one that is located
   // one tile from the buffer `stage`, for this wave's rows; meanwhile the located tile is asked for into the buffer
   // at byte address `to`
   auto compute = [&](int tile, const __bf16* stage, uint32_t to) __attribute__((always_inline)) {
@@ -212,6 +212,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
 #pragma unroll
     for (int j = 0; j < R; ++j) any = any || (rows[j] > 0 && key0 <= pos_last[j] && key0 + kTile > lo_first[j]);
     if (tile >= te || !any) {  // no row of the wave sees a key of it
+      next = look_up(tile + 2);
 #pragma unroll
       for (int i = 0; i < CPW; ++i) ask(i, to);
       return;
@@ -258,6 +259,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
         vf[batch % 2][b] = *reinterpret_cast<const bf16x8*>(v_s + ((batch * VB + b) * 64 + lane) * 8);
     };
     read_values(0);
+    // the pages of the tile after the next are looked up here: the table's entries arrive during the softmax
+    // arithmetic, with the value operands (a wait for operands from LDS is a wait for scalar loads as well)
+    next = look_up(tile + 2);
     __builtin_amdgcn_sched_barrier(0);
     bf16x8 pf[R];
     float alpha[R];
@@ -289,8 +293,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int v = 0; v < 4; ++v) mx = fmaxf(mx, y[t][v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = max_over_row_lanes(mx);
       const float m_new = fmaxf(m_run[j], mx);
       // a row that has seen no visible key yet keeps m = -inf; 2^(-inf - -inf) must not appear
       alpha[j] = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run[j] - m_new);
@@ -345,14 +348,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
     locate(look_up(tb));
 #pragma unroll
     for (int i = 0; i < CPW; ++i) ask(i, lds0);
-    Pages next = look_up(tb + 1);
+    next = look_up(tb + 1);
     // tile `tile` has been asked for into `cur`; `other` held tile - 1 and takes tile + 1
     auto step = [&](int tile, const __bf16* cur, uint32_t other) __attribute__((always_inline)) {
       __builtin_amdgcn_sched_barrier(0);
       __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's chunks of `tile` have arrived
       bare_barrier();  // and everyone's; and every wave has finished tile - 1
       locate(next);
-      next = look_up(tile + 2);
       compute(tile, cur, other);
     };
     const int te2 = tb + (te - tb + 1) / 2 * 2;
@@ -368,8 +370,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
 #pragma unroll
   for (int j = 0; j < R; ++j) {
     float l = l_run[j];
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
+    l = sum_over_row_lanes(l);
     if (!row_ok[j]) continue;
     if (num_chunks == 1) {
       bf16* op = out + static_cast<size_t>(q_row[j]) * out_stride + static_cast<size_t>(kh * G + g) * HD;
@@ -446,7 +447,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
     ++chunk;
     KS = (max_tiles + chunk - 1) / chunk;
   }
-  const dim3 grid(KS, Kh, groups);
+  const dim3 grid(Kh, KS, groups);
   const bf16* qp = static_cast<const bf16*>(q);
   const bf16* kp = static_cast<const bf16*>(k_pages);
   const bf16* vp = static_cast<const bf16*>(v_pages);
