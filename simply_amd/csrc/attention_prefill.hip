@@ -398,7 +398,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
 
 }  // namespace prefill
 
-constexpr int kPrefillRowTiles = 1;  // R: units per wave (2 was tried: three times slower, the registers of 32 rows spill)
+// R: units per wave.  2 halves the operand reads from LDS per row, but was 2.5 times slower: the compiler then keeps
+// the accumulators of 32 rows in the registers that the arithmetic needs, a few loop invariants are spilled, and every
+// reload of one waits for all outstanding memory loads, which are the next tile's keys and values.
+constexpr int kPrefillRowTiles = 1;
 
 int paged_attention_prefill_group() { return prefill::kWaves * kPrefillRowTiles; }
 
