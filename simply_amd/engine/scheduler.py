@@ -146,6 +146,17 @@ class Scheduler:
         # 1. decoding requests, oldest first; each needs room for one token
         decoding = sorted((r for r in self.running if r.num_computed == r.num_tokens - 1), key=lambda r: r.arrival)
         scheduled_ids = set()
+        if decoding and budget >= len(decoding):
+            # the usual case, all of them fit: one question to the cache instead of one per request (each costs
+            # a pass over all live requests).  The requests one by one below decide the same when this holds.
+            wants = [(r.request_id, r.num_computed, 1) for r in decoding]
+            if self.cache.can_reserve(wants):
+                self.cache.reserve_all(wants)
+                for r in decoding:
+                    out.scheduled.append(Scheduled(r, r.num_computed, 1, True))
+                    scheduled_ids.add(r.request_id)
+                budget -= len(decoding)
+                decoding = []
         for r in decoding:
             if r.status is not Status.RUNNING or budget < 1:
                 continue
