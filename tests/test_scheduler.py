@@ -167,3 +167,21 @@ def test_max_input_len_keeps_the_tail():
     r = Request("t", list(range(30)), SamplingParams(max_input_len=10))
     sched.add(r)
     assert r.prompt_token_ids == list(range(20, 30))
+
+
+def test_decoding_requests_ask_the_cache_once():
+    """A step of decoding requests that all fit costs a fixed number of passes over the live requests, not one
+    per request; the decisions are those of the one-by-one path (oldest first, one token each)."""
+    cache, sched = make(num_pages=256, slots=32, budget=64, max_len=128)
+    for i in range(32):
+        sched.add(req(f"r{i}", 2, steps=50))
+    run_step(sched, sched.schedule())
+    run_step(sched, sched.schedule())
+    calls = []
+    original = cache.can_reserve
+    cache.can_reserve = lambda wants: calls.append(len(wants)) or original(wants)
+    out = sched.schedule()
+    assert [(s.request.request_id, s.num_tokens, s.samples) for s in out.scheduled] == \
+        [(f"r{i}", 1, True) for i in range(32)]
+    assert len(calls) <= 3 and max(calls) == 32
+    cache.check()
