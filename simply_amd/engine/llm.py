@@ -119,7 +119,7 @@ class LMInterface:
             return finished
         entries = []
         for s in out.scheduled:
-            toks = s.request.all_token_ids[s.start:s.start + s.num_tokens]
+            toks = s.request.tokens(s.start, s.num_tokens)
             entries.append(StepEntry(s.request.request_id, toks, [s.num_tokens - 1] if s.samples else [], s.start))
         n = self._decode_steps_ahead(out.scheduled, max_decode_steps)
         if n > 1:

@@ -55,6 +55,15 @@ class Request:
     def all_token_ids(self) -> list[int]:
         return self.prompt_token_ids + self.output_token_ids
 
+    def tokens(self, start: int, count: int) -> list[int]:
+        """Tokens start .. start + count - 1 of prompt and output together, without laying the two end to end."""
+        p = len(self.prompt_token_ids)
+        if start >= p:
+            return self.output_token_ids[start - p:start - p + count]
+        if start + count <= p:
+            return self.prompt_token_ids[start:start + count]
+        return self.prompt_token_ids[start:] + self.output_token_ids[:start + count - p]
+
     @property
     def num_tokens(self) -> int:
         return len(self.prompt_token_ids) + len(self.output_token_ids)

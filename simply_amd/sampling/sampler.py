@@ -49,12 +49,12 @@ class Sampler:
             raise ValueError(f"sample: {R} rows, room for {self.max_rows}")
         n = self.max_rows
         self.modes = self.modes_of(params)
-        for r, (p, s, c) in enumerate(zip(params, seeds, counters)):
-            self._f_host[r] = p.temperature
-            self._f_host[n + r] = p.top_p
-            self._i_host[r] = p.top_k
-            self._i_host[n + r] = c
-            self._s_host[r] = s
+        f, i, sd = self._f_host.numpy(), self._i_host.numpy(), self._s_host.numpy()
+        f[:R] = [p.temperature for p in params]
+        f[n:n + R] = [p.top_p for p in params]
+        i[:R] = [p.top_k for p in params]
+        i[n:n + R] = counters
+        sd[:R] = seeds
         self._f_dev.copy_(self._f_host, non_blocking=True)
         self._i_dev.copy_(self._i_host, non_blocking=True)
         self._s_dev.copy_(self._s_host, non_blocking=True)
