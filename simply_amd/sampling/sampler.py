@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from typing import Sequence
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -34,8 +35,11 @@ class Sampler:
         self._f_dev = torch.empty(2 * max_rows, dtype=torch.float32, device=self.device)
         self._i_dev = torch.empty(2 * max_rows, dtype=torch.int32, device=self.device)
         self._s_dev = torch.empty(max_rows, dtype=torch.int64, device=self.device)
-        self._tokens = torch.empty(max_rows, dtype=torch.int32, device=self.device)
-        self._logprobs = torch.empty(max_rows, dtype=torch.float32, device=self.device)
+        # tokens and log-probabilities in one buffer, so that one copy brings both to the host
+        self._out = torch.empty(2 * max_rows, dtype=torch.int32, device=self.device)
+        self._out_host = torch.empty(2 * max_rows, dtype=torch.int32, pin_memory=pin)
+        self._tokens = self._out[:max_rows]
+        self._logprobs = self._out[max_rows:].view(torch.float32)
         #: what the staged rows ask for (ops.SAMPLE_*): `launch` leaves out the kernels that none of them needs, so
         #: a recorded launch serves only rows that ask for no more than these
         self.modes = 0
@@ -93,4 +97,9 @@ class Sampler:
         self.stage(params, seeds, counters)
         tokens, logprobs = self.launch(logits)
         # one synchronising copy back: the scheduler needs the tokens to go on
-        return tokens[:R].tolist(), logprobs[:R].tolist()
+        n = self.max_rows
+        self._out_host.copy_(self._out, non_blocking=True)
+        if self.device.type == "cuda":
+            torch.cuda.current_stream(self.device).synchronize()
+        host = self._out_host.numpy()
+        return host[:R].tolist(), host[n:n + R].view(np.float32).tolist()
