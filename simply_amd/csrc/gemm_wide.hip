@@ -327,6 +327,13 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
         shape = sh[0];
       }
     }
+    // A gated product of few rows whose tiles of 128 weight rows make one round at most (the 2B and 9B feed-forward
+    // for up to 128 decoding requests) streams its weights: rows of 64 (or 128) with the deepest pipeline that fits
+    // are 5 to 25 % faster there than the large tiles (2B at 64 rows: 23 against 28 us; 9B: 39 against 48).
+    if (epi == 1 && M <= 128) {
+      const int rows = M <= 64 ? 64 : 128;
+      if (static_cast<int64_t>((M + rows - 1) / rows) * ((NW + 127) / 128) <= wide::kCUs) shape = M <= 64 ? 6064128 : 3128128;
+    }
     // 17 to 1,536 rows without an epilogue (portions of prompts, many decoding requests): the tiles above are too few
     // for 256 CUs, and every workgroup walks all of K at the pace of its own slabs.  Smaller tiles with deeper
     // pipelines, and K cut over workgroups so that about one round of them covers the GPU, chosen by a model of the
