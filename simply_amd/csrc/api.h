@@ -27,6 +27,12 @@ int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, int w_post_dt
                    int plus_one_post, float* residual, const void* w_next, int w_next_dtype, float eps_next,
                    int plus_one_next, void* out, int out_dtype, int T, int D, hipStream_t stream);
 
+// The same with y given as `planes` partial results [planes][T][D] float32 (sa_gemm_planes): y is their sum in the
+// order of the planes, rounded to bfloat16, as the sum kernel of the product would have left it.  D % 4 == 0.
+int sa_add_rmsnorm_planes(const float* y_planes, int planes, const void* w_post, int w_post_dtype, float eps_post,
+                          int plus_one_post, float* residual, const void* w_next, int w_next_dtype, float eps_next,
+                          int plus_one_next, void* out, int out_dtype, int T, int D, hipStream_t stream);
+
 // Fused projection rows [T, (H + 2K) * hd]: rotate q and k (timescale null: no rotation), divide q by
 // q_div, write k and v into the pages at slot_mapping[t] = page * page_size + offset (k_pages null: no write).
 int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, const int* positions, const float* timescale,
@@ -70,6 +76,17 @@ int sa_decode_slots(int B, const int* positions, const int* token_seq, const int
 int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C, int c_dtype,
             int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, int packed, int shape,
             void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
+// The same product, but where it is computed in cuts of K its last kernel, the sum of the cuts, is left to the
+// caller: *planes receives their number, and the workspace then holds [planes][M][N] float32 partial results whose
+// sum in the order of the planes, rounded to C's type, is the product (sa_add_rmsnorm_planes takes them).  *planes
+// == 1: C holds the product as after sa_gemm.
+// C = the sum of `count` planes [M][N] float32 in their order, rounded to C's type: the kernel that sa_gemm_planes
+// leaves out.
+int sa_sum_planes(const float* planes, int count, void* C, int c_dtype, int64_t ldc, int M, int N, hipStream_t stream);
+int sa_gemm_planes(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
+                   int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, int packed,
+                   int shape, void* workspace, int64_t workspace_bytes, int* planes, hipStream_t stream);
 
 // For 1..16 rows of bfloat16: h_out = h_in + norm(y; w_post) (y null: h_out is h_in and is not written; w_post null:
 // h_out = h_in + y), a = norm(h_out; w_next), C = epilogue(a . W^T) with W tiled (paired tiles for the gated
@@ -188,7 +205,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
 bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
                      const void* C, int c_dtype, int epi, int packed);
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
-              int shape, int ks, void* workspace, size_t workspace_bytes, hipStream_t stream);
+              int shape, int ks, void* workspace, size_t workspace_bytes, hipStream_t stream, int* planes_left = nullptr);
 // C = epilogue(sum over z of partials[z][M][NW]): the second kernel of every product that cuts K over workgroups
 int gemm_sum_partials(const float* partials, int ks, void* C, int c_dtype, int64_t ldc, int M, int N, int NW, int epi,
                       int act, float cap, hipStream_t stream);

@@ -130,11 +130,14 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
 // overlap these chains than with a wave to a row: 2,048 rows of 2,304 elements (56 MB read and written) take 14 us
 // where a wave to a row took 20, 512 rows 6.6 against 9.0, 8,192 rows 52 against 77.  D % 4 == 0, D <= 1024 NP,
 // 16-byte aligned.
-template <typename YT, typename OT, int NP>
+// PLANES (with YT = bf16, one row to a workgroup): y is not read but made, as the sum of that many float planes
+// [T][D] at y_planes in their order, rounded to bfloat16: what the sum kernel of a product with K cut over
+// workgroups would have written, without that kernel and its round trip through memory.
+template <typename YT, typename OT, int NP, bool PLANES = false>
 __global__ __launch_bounds__(256) void add_rmsnorm_split_kernel(
     const YT* __restrict__ y, const void* __restrict__ w_post, int w_post_dtype, float eps_post, float plus_one_post,
     float* __restrict__ residual, const void* __restrict__ w_next, int w_next_dtype, float eps_next, float plus_one_next,
-    OT* __restrict__ out, int T, int D, int rows_per_group) {
+    OT* __restrict__ out, int T, int D, int rows_per_group, const float* __restrict__ y_planes, int planes) {
   __shared__ float scratch[32];
   const int tid = threadIdx.x;
   using RawY = typename std::conditional<sizeof(YT) == 4, float4, uint2>::type;
@@ -168,7 +171,38 @@ __global__ __launch_bounds__(256) void add_rmsnorm_split_kernel(
       b.y[p] = RawY{};
       if (d < D) {
         b.h[p] = *reinterpret_cast<const float4*>(residual + rb + d);
-        b.y[p] = *reinterpret_cast<const RawY*>(y + rb + d);
+        if constexpr (!PLANES) b.y[p] = *reinterpret_cast<const RawY*>(y + rb + d);
+      }
+    }
+    if constexpr (PLANES) {
+      {
+        const size_t plane = static_cast<size_t>(T) * D;
+        float4 sum[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) sum[p] = float4{0.f, 0.f, 0.f, 0.f};
+        for (int z0 = 0; z0 < planes; z0 += 4) {
+          float4 part[4][NP];
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+              const int d = (p * 256 + tid) * 4;
+              part[j][p] = (z0 + j < planes && d < D)
+                               ? *reinterpret_cast<const float4*>(y_planes + (z0 + j) * plane + rb + d)
+                               : float4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+              sum[p].x += part[j][p].x; sum[p].y += part[j][p].y; sum[p].z += part[j][p].z; sum[p].w += part[j][p].w;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+          b.y[p].x = static_cast<uint32_t>(float_to_bf16(sum[p].x).bits) | (static_cast<uint32_t>(float_to_bf16(sum[p].y).bits) << 16);
+          b.y[p].y = static_cast<uint32_t>(float_to_bf16(sum[p].z).bits) | (static_cast<uint32_t>(float_to_bf16(sum[p].w).bits) << 16);
+        }
       }
     }
   };
@@ -627,7 +661,7 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
 #define SA_SPLIT(YT, OT, NP)                                                                                       \
   add_rmsnorm_split_kernel<YT, OT, NP><<<(T + rpg - 1) / rpg, 256, 0, stream>>>(                                   \
       static_cast<const YT*>(y), w_post, w_post_dtype, eps_post, pp, residual, w_next, w_next_dtype, eps_next, pn, \
-      static_cast<OT*>(out), T, D, rpg)
+      static_cast<OT*>(out), T, D, rpg, nullptr, 0)
 #define SA_SPLIT_N(YT, OT)            \
   do {                                \
     if (D <= 2048) SA_SPLIT(YT, OT, 2); \
@@ -647,6 +681,38 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
                                                        plus_one_post ? 1.f : 0.f, residual, w_next, w_next_dtype,
                                                        eps_next, plus_one_next ? 1.f : 0.f, out, out_dtype, D);
   return check_launch("add_rmsnorm");
+}
+
+extern "C" int sa_add_rmsnorm_planes(const float* y_planes, int planes, const void* w_post, int w_post_dtype,
+                                     float eps_post, int plus_one_post, float* residual, const void* w_next,
+                                     int w_next_dtype, float eps_next, int plus_one_next, void* out, int out_dtype,
+                                     int T, int D, hipStream_t stream) {
+  if (T == 0) return 0;
+  const auto aligned16 = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+  SA_REQUIRE(T > 0 && D > 0 && planes >= 1 && y_planes != nullptr, "add_rmsnorm_planes: bad sizes T=%d D=%d planes=%d",
+             T, D, planes);
+  SA_REQUIRE(D % 4 == 0 && D <= 5120 && aligned16(y_planes) && aligned16(residual) && aligned16(out) &&
+                 aligned16(w_post) && aligned16(w_next),
+             "add_rmsnorm_planes: rows of a multiple of 4 and at most 5120 elements, 16-byte aligned; got D=%d", D);
+  SA_REQUIRE(w_next == nullptr || out != nullptr, "add_rmsnorm_planes: a next norm needs an output");
+  SA_REQUIRE(out == nullptr || out_dtype == kBF16 || out_dtype == kF32, "add_rmsnorm_planes: unknown output type");
+  const float pp = plus_one_post ? 1.f : 0.f, pn = plus_one_next ? 1.f : 0.f;
+#define SA_PLANES(OT, NP)                                                                                         \
+  add_rmsnorm_split_kernel<bf16, OT, NP, true><<<T, 256, 0, stream>>>(nullptr, w_post, w_post_dtype, eps_post, pp,       \
+                                                                residual, w_next, w_next_dtype, eps_next, pn,      \
+                                                                static_cast<OT*>(out), T, D, 1, y_planes, planes)
+#define SA_PLANES_N(OT)              \
+  do {                               \
+    if (D <= 2048) SA_PLANES(OT, 2); \
+    else if (D <= 3072) SA_PLANES(OT, 3); \
+    else if (D <= 4096) SA_PLANES(OT, 4); \
+    else SA_PLANES(OT, 5);           \
+  } while (0)
+  if (out != nullptr && out_dtype == kF32) SA_PLANES_N(float);
+  else SA_PLANES_N(bf16);
+#undef SA_PLANES_N
+#undef SA_PLANES
+  return check_launch("add_rmsnorm_planes");
 }
 
 extern "C" int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, const int* positions,

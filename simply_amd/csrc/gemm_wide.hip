@@ -297,7 +297,7 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
 // ks > 1 cuts K over that many workgroups per tile (no epilogue only; the partial tiles go through `workspace`,
 // which must hold ks * M * N floats).
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
-              int shape, int ks, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+              int shape, int ks, void* workspace, size_t workspace_bytes, hipStream_t stream, int* planes_left) {
   if (ks < 1) ks = 1;
   if (ks > K / wide::BK) ks = K / wide::BK;
   if (ks > 1 && (epi != 0 || workspace == nullptr || static_cast<size_t>(ks) * M * N * sizeof(float) > workspace_bytes)) {
@@ -393,6 +393,10 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
       return 1;
   }
   if (check_launch("gemm_wide")) return 1;
+  if (planes_left != nullptr) {  // the caller adds the cuts' partial results up itself (ks planes of [M, N] floats)
+    *planes_left = ks;
+    return 0;
+  }
   if (ks > 1) return gemm_sum_partials(ws, ks, C, kBF16, ldc, M, N, N, 0, 0, 0.f, stream);
   return 0;
 }

@@ -32,9 +32,11 @@ using namespace sa;
 extern "C" const char* sa_last_error() { return g_error; }
 extern "C" int sa_version() { return 1; }
 
-extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
+static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
                        int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo,
-                       int packed, int shape, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+                       int packed, int shape, void* workspace, int64_t workspace_bytes, int* planes_left,
+                       hipStream_t stream) {
+  if (planes_left != nullptr) *planes_left = 1;
   if (M == 0 || N == 0) return 0;
   SA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
   SA_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld are below K=%d, N=%d", (long long)lda,
@@ -87,7 +89,7 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
     if (takes)
       return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape % 10000000 : 0,
                        algo == 4 ? shape / 10000000 : 1, workspace,
-                       static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
+                       static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream, planes_left);
   }
   if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || tiled_first))) {
     const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
@@ -99,6 +101,30 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                         static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
   }
   return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, stream);
+}
+
+extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
+                       int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo,
+                       int packed, int shape, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  return gemm_routed(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, algo, packed, shape,
+                     workspace, workspace_bytes, nullptr, stream);
+}
+
+extern "C" int sa_sum_planes(const float* planes, int count, void* C, int c_dtype, int64_t ldc, int M, int N,
+                             hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  SA_REQUIRE(planes != nullptr && count >= 1 && M > 0 && N > 0 && ldc >= N, "sum_planes: bad sizes %d x [%d, %d]",
+             count, M, N);
+  return gemm_sum_partials(planes, count, C, c_dtype, ldc, M, N, N, 0, 0, 0.f, stream);
+}
+
+extern "C" int sa_gemm_planes(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype,
+                              void* C, int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap,
+                              int algo, int packed, int shape, void* workspace, int64_t workspace_bytes, int* planes,
+                              hipStream_t stream) {
+  SA_REQUIRE(planes != nullptr, "gemm_planes: nowhere to put the number of planes");
+  return gemm_routed(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, algo, packed, shape,
+                     workspace, workspace_bytes, planes, stream);
 }
 
 extern "C" int sa_paged_attention(const void* q, int dtype, int64_t q_stride, const void* k_pages,

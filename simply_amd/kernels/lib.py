@@ -33,6 +33,9 @@ _SIGNATURES = {
     "sa_decode_advance": [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P],
     "sa_decode_slots": [_I, _P, _P, _P, _I, _I, _P, _P],
     "sa_gemm": [_P, _I, _L, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P],
+    "sa_gemm_planes": [_P, _I, _L, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L, _P, _P],
+    "sa_sum_planes": [_P, _I, _P, _I, _L, _I, _I, _P],
+    "sa_add_rmsnorm_planes": [_P, _I, _P, _I, _F, _I, _P, _P, _I, _F, _I, _P, _I, _I, _I, _P],
     "sa_paged_attention": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "sa_paged_attention_decode": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _L,
                                   _P],

@@ -111,13 +111,41 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, plus_one: bool, o
     return out
 
 
-def add_rmsnorm(y: torch.Tensor, residual: torch.Tensor, *, post_weight: torch.Tensor | None = None,
+class PartialSums:
+    """A matrix product whose cuts of K have not been added up yet (`gemm(..., defer_sum=True)`): `planes`
+    [cuts, M, N] float32 in the kernels' workspace, valid until the next kernel that uses the workspace, and `out`,
+    the tensor that the sum belongs in.  `add_rmsnorm` takes it in place of y and adds the planes up itself, which
+    saves the sum kernel and its round trip; anyone else calls `materialize()`."""
+
+    def __init__(self, planes: torch.Tensor, out: torch.Tensor):
+        self.planes, self.out = planes, out
+        self.shape, self.dtype, self.device = out.shape, out.dtype, out.device
+
+    def materialize(self) -> torch.Tensor:
+        """The product itself: the sum kernel, now."""
+        if self.planes is not None:
+            count, M, N = self.planes.shape
+            _lib.call("sa_sum_planes", _ptr(self.planes), count, _ptr(self.out), _code(self.out), self.out.stride(0), M, N,
+                      _stream())
+            self.planes = None
+        return self.out
+
+
+def add_rmsnorm(y: "torch.Tensor | PartialSums", residual: torch.Tensor, *, post_weight: torch.Tensor | None = None,
                 post_eps: float = 0.0, post_plus_one: bool = True, next_weight: torch.Tensor | None = None,
                 next_eps: float = 0.0, next_plus_one: bool = True, out_dtype: torch.dtype | None = None,
                 out: torch.Tensor | None = None) -> torch.Tensor | None:
     """residual += norm(y; post_weight) (or += y); returns norm(residual; next_weight) if asked."""
-    _dev(y, residual, post_weight, next_weight, out)
     T, D = residual.shape
+    planes = None
+    if isinstance(y, PartialSums):
+        fits = (y.planes is not None and D % 4 == 0 and D <= 5120 and y.dtype == torch.bfloat16
+                and tuple(y.shape) == (T, D) and all(w is None or w.data_ptr() % 16 == 0 for w in (post_weight, next_weight)))
+        if fits:
+            planes, y = y.planes, y.out   # (y stands for shape and type below; it is not read)
+        else:
+            y = y.materialize()
+    _dev(y, residual, post_weight, next_weight, out)
     if residual.dtype != torch.float32 or not residual.is_contiguous():
         raise KernelError("add_rmsnorm: the residual stream must be contiguous float32")
     if tuple(y.shape) != (T, D) or not y.is_contiguous():
@@ -132,6 +160,12 @@ def add_rmsnorm(y: torch.Tensor, residual: torch.Tensor, *, post_weight: torch.T
             raise KernelError("add_rmsnorm: bad output")
     else:
         out = None
+    if planes is not None:
+        _lib.call("sa_add_rmsnorm_planes", _ptr(planes), planes.shape[0], _ptr(post_weight),
+                  _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one),
+                  _ptr(residual), _ptr(next_weight), _code(next_weight) if next_weight is not None else 0,
+                  float(next_eps), int(next_plus_one), _ptr(out), _code(out) if out is not None else 0, T, D, _stream())
+        return out
     _lib.call("sa_add_rmsnorm", _ptr(y), _code(y), _ptr(post_weight),
               _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one),
               _ptr(residual), _ptr(next_weight), _code(next_weight) if next_weight is not None else 0,
@@ -305,9 +339,12 @@ def library_gemm_min_rows() -> int:
 
 def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
          soft_cap: float | None = None, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
-         algo: int = ALGO_AUTO, shape: int = 0, activation: int = ACT_GELU_TANH) -> torch.Tensor:
+         algo: int = ALGO_AUTO, shape: int = 0, activation: int = ACT_GELU_TANH,
+         defer_sum: bool = False) -> "torch.Tensor | PartialSums":
     """a[M, K] . w[N, K]^T.  With w2 (row-major weights) or a paired `TiledWeight`: act(a.wg^T) * (a.wu^T) with
-    the activation of that code.  With soft_cap: cap * tanh(. / cap).  w is a row-major tensor or a `TiledWeight`."""
+    the activation of that code.  With soft_cap: cap * tanh(. / cap).  w is a row-major tensor or a `TiledWeight`.
+    defer_sum: where the product is computed in cuts of K, leave their sum to the caller: the result is then a
+    `PartialSums` (else the tensor as always)."""
     packed = isinstance(w, TiledWeight)
     wd = w.data if packed else w
     w2d = None
@@ -347,6 +384,14 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
         # (not while a graph is recorded: the library may allocate a workspace)
         return torch.matmul(a, w.row_major.t(), out=out)
     ws = _workspace(a.device)
+    if defer_sum and epi == EPILOGUE_NONE and out.dtype == torch.bfloat16 and out.is_contiguous():
+        count = ctypes.c_int(1)
+        _lib.call("sa_gemm_planes", _ptr(a), _code(a), lda, _ptr(wd), _ptr(w2d), _code(wd), _ptr(out), _code(out), ldc, M, N,
+                  K, epi, cap, algo, int(packed), int(shape), _ptr(ws), ws.numel(), ctypes.byref(count), _stream())
+        if count.value > 1:
+            words = count.value * M * N
+            return PartialSums(ws.view(torch.float32)[:words].view(count.value, M, N), out)
+        return out
     _lib.call("sa_gemm", _ptr(a), _code(a), lda, _ptr(wd), _ptr(w2d), _code(wd), _ptr(out), _code(out), ldc, M, N, K, epi,
               cap, algo, int(packed), int(shape), _ptr(ws), ws.numel(), _stream())
     return out

@@ -19,6 +19,7 @@ from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight, pending_fits
 @MIXERS.register("paged_attention")
 class PagedAttention(Mixer):
     accepts_pending = True
+    defers_sum = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, query_scale: float,
                  soft_cap: float | None = None, window: int | None = None,
@@ -53,7 +54,7 @@ class PagedAttention(Mixer):
     def cache_need(self):
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, x, ctx, cache):
+    def forward(self, x, ctx, cache, defer_sum=False):
         H, K, hd = self.num_heads, self.num_kv_heads, self.head_dim
         group = ctx.groups[cache.group_id]
         pe = self.position_encoding
@@ -94,4 +95,4 @@ class PagedAttention(Mixer):
         else:
             ops.paged_attention(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions, H,
                                 window=self.window, soft_cap=self.soft_cap, out=o)
-        return ops.gemm(o, self.o_proj)
+        return ops.gemm(o, self.o_proj, defer_sum=defer_sum)

@@ -17,6 +17,9 @@ Parts, per kind, and what each must provide:
 
 A mixer or feed-forward that sets `accepts_pending` may be handed a `PendingNorm` instead of x: the norm (and the
 residual sum before it) that has not been computed yet, which `project` folds into the part's first product.
+One that sets `defers_sum` takes `forward(..., defer_sum=True)` and may then return its last product with the
+cuts of K not yet added up (`ops.PartialSums`); a block asks for that only when the norm that receives the result
+says `adds_partial_sums`, and hands the result to that norm's `add_into` before anything else runs.
 """
 from __future__ import annotations
 
@@ -209,6 +212,8 @@ class PositionEncoding(Part):
 class Mixer(Part):
     #: True if forward() takes a `PendingNorm` in place of x (and consumes it with `project`)
     accepts_pending = False
+    #: True if forward() takes defer_sum=True and may then return an `ops.PartialSums`
+    defers_sum = False
 
     def cache_need(self) -> PagedKVNeed | StateNeed | None:
         return None
@@ -222,6 +227,8 @@ class Mixer(Part):
 class FeedForward(Part):
     #: True if forward() takes a `PendingNorm` in place of x (and consumes it with `project`)
     accepts_pending = False
+    #: True if forward() takes defer_sum=True and may then return an `ops.PartialSums`
+    defers_sum = False
 
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         raise NotImplementedError

@@ -34,9 +34,14 @@ class SandwichBlock(Block):
             normed, h = normed.materialize(), normed.residual
         if normed is None:
             normed = n["pre_mixer"].forward(h, ctx.dtype)
-        y = self.mixer.forward(normed, ctx, cache)
+        # (a part's last product may leave the sum of its cuts of K to the norm behind it, where both can)
+        def defer(part, norm):
+            both = part.defers_sum and getattr(norm, "adds_partial_sums", False) and ctx.dtype == torch.bfloat16
+            return {"defer_sum": True} if both else {}
+
+        y = self.mixer.forward(normed, ctx, cache, **defer(self.mixer, n["post_mixer"]))
         normed = n["post_mixer"].add_into(h, y, n["pre_ffn"], ctx.dtype)
-        y = self.feed_forward.forward(normed, ctx)
+        y = self.feed_forward.forward(normed, ctx, **defer(self.feed_forward, n["post_ffn"]))
         normed_next = n["post_ffn"].add_into(h, y, next_norm, ctx.dtype)
         return h, normed_next
 

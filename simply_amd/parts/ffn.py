@@ -18,6 +18,7 @@ ACTIVATIONS.register("squared_relu", ops.ACT_SQUARED_RELU)
 @FEED_FORWARDS.register("gated_dense")
 class GatedDense(FeedForward):
     accepts_pending = True
+    defers_sum = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu_tanh"):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
@@ -40,7 +41,7 @@ class GatedDense(FeedForward):
             self.gate_up, self.gate_proj, self.up_proj = None, gate, up
         self.down_proj = as_product_weight(tensors["down_proj"], many_rows=True)
 
-    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx=None, defer_sum=False) -> torch.Tensor:
         # gelu(x.Wg^T) * (x.Wu^T), one kernel
         if self.gate_up is not None:
             z = project(x, self.gate_up, activation=self.activation_code)
@@ -48,4 +49,4 @@ class GatedDense(FeedForward):
             if isinstance(x, PendingNorm):
                 x = x.materialize()
             z = ops.gemm(x, self.gate_proj, w2=self.up_proj, activation=self.activation_code)
-        return ops.gemm(z, self.down_proj)
+        return ops.gemm(z, self.down_proj, defer_sum=defer_sum)

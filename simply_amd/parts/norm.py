@@ -13,6 +13,8 @@ from .base import Norm, ParamSpec
 class RMSNorm(Norm):
     #: the fused norm-and-product kernel computes exactly this norm from (scale, eps, scale_plus_one)
     fusable_rms = True
+    #: add_into takes a product whose cuts of K are not added up yet (`ops.PartialSums`) in place of y
+    adds_partial_sums = True
 
     def __init__(self, dim: int, eps: float, scale_plus_one: bool = True):
         self.dim = int(dim)

@@ -885,3 +885,34 @@ def test_gemm_normed_rotary(M, H, Kh, hd, P, K, rotate):
     got = ops.gemm_normed_rotary(None, h, None, tw, **norm, positions=positions, timescale=ts, scale_factor=1.0,
                                  query_scale=12.0, num_heads=H, num_kv_heads=Kh, head_dim=hd)
     torch.testing.assert_close(got[:, :H * hd].float(), want[:, :H * hd].float(), rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 2304, 2048), (64, 2304, 9216), (64, 2304, 2048), (100, 3584, 4096), (512, 2304, 9216),
+                                   (40, 200, 512), (8, 2304, 2048), (2048, 2304, 2048)])
+def test_deferred_sum_of_a_product_is_added_up_by_the_norm(M, N, K):
+    """A product computed in cuts of K may leave their sum to the residual/norm kernel behind it: residual stream and
+    normed activations are the same to the bit as with the product's own sum kernel in between, and `materialize()`
+    is that product."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_tiles
+    a = rand((M, K), torch.bfloat16, 95)
+    w = pack_tiles(rand((N, K), torch.bfloat16, 96, 0.05))
+    h0 = rand((M, N), torch.float32, 97, 3.0)
+    w1, w2 = rand((N,), torch.bfloat16, 98, 0.3), rand((N,), torch.bfloat16, 99, 0.3)
+    whole = ops.gemm(a, w)
+    for with_next in (True, False):
+        kw = dict(post_weight=w1, post_eps=1e-6, next_weight=w2 if with_next else None, next_eps=1e-6,
+                  out_dtype=torch.bfloat16)
+        h_want, h_got = h0.clone(), h0.clone()
+        o_want = ops.add_rmsnorm(whole, h_want, **kw)
+        y = ops.gemm(a, w, defer_sum=True)
+        o_got = ops.add_rmsnorm(y, h_got, **kw)
+        assert torch.equal(h_got, h_want)
+        assert (o_got is None) == (o_want is None) and (o_got is None or torch.equal(o_got, o_want))
+    y = ops.gemm(a, w, defer_sum=True)
+    if isinstance(y, ops.PartialSums):
+        assert y.planes.shape[0] > 1 and torch.equal(y.materialize(), whole)
+    else:
+        assert torch.equal(y, whole)
+    if (M, N, K) in ((64, 2304, 9216), (512, 2304, 9216)):
+        assert isinstance(ops.gemm(a, w, defer_sum=True), ops.PartialSums)   # these sizes do cut K
