@@ -39,6 +39,15 @@ int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, const int* pos
                         float scale_factor, float q_div, const int64_t* slot_mapping, void* k_pages, void* v_pages,
                         int T, int H, int K, int hd, int page_size, hipStream_t stream);
 
+// The same for a projection whose cuts of K are not added up yet (sa_gemm_planes): its elements are the sums of
+// `count` planes [T][(H + 2K) hd] float32, rounded to bfloat16; the rotated and scaled queries go to qkv (bfloat16
+// rows of row_stride elements; its key and value columns are not written).  A block per (token, head): for up to a
+// few hundred tokens.
+int sa_rope_cache_write_planes(const float* planes, int count, void* qkv, int64_t row_stride, const int* positions,
+                               const float* timescale, float scale_factor, float q_div, const int64_t* slot_mapping,
+                               void* k_pages, void* v_pages, int T, int H, int K, int hd, int page_size,
+                               hipStream_t stream);
+
 // Rotation alone, in place, then division by div.
 int sa_rope(void* x, int dtype, int64_t row_stride, const int* positions, const float* timescale, float scale_factor,
             float div, int T, int n_heads, int hd, hipStream_t stream);

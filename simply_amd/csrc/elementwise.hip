@@ -286,10 +286,21 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
                                         const float* __restrict__ timescale /* [hd/2] or null = no rotation */,
                                         float inv_scale_factor, float q_div, const int64_t* __restrict__ slot_mapping,
                                         T* __restrict__ k_pages, T* __restrict__ v_pages, int H, int K, int hd,
-                                        int page_size) {
+                                        int page_size, const float* __restrict__ planes = nullptr, int count = 0,
+                                        size_t plane_words = 0) {
   const int t = blockIdx.x, head = blockIdx.y;
   const int half = hd / 2;
   T* src = qkv + static_cast<size_t>(t) * row_stride + static_cast<size_t>(head) * hd;
+  // planes: the projection has not been added up yet; its element is the sum of `count` planes [tokens][(H + 2K) hd]
+  // in their order, rounded to T as the product's sum kernel would have left it in qkv
+  const float* part = planes == nullptr ? nullptr
+                                        : planes + (static_cast<size_t>(t) * (H + 2 * K) + head) * hd;
+  auto at = [&](int i) __attribute__((always_inline)) {
+    if (part == nullptr) return to_float(src[i]);
+    float sum = 0.f;
+    for (int z = 0; z < count; ++z) sum += part[z * plane_words + i];
+    return to_float(from_float<T>(sum));
+  };
   const float pos = static_cast<float>(positions[t]);
   if (head < H + K) {
     const bool is_q = head < H;
@@ -307,7 +318,7 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
     }
     const bool tiled = to_pages && keys_tiled(page_size, hd);
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      const float x1 = to_float(src[i]), x2 = to_float(src[i + half]);
+      const float x1 = at(i), x2 = at(i + half);
       float o1 = x1, o2 = x2;
       if (timescale != nullptr) {
         const float angle = pos / timescale[i] * inv_scale_factor;
@@ -335,7 +346,7 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int64_t row_stride,
     const int64_t page = slot / page_size, off = slot % page_size;
     // value pages are [page, head, hd, page_size]: the keys of a page are contiguous for each dimension
     T* dst = v_pages + (page * K + (head - H - K)) * page_size * hd + off;
-    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[static_cast<size_t>(i) * page_size] = src[i];
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[static_cast<size_t>(i) * page_size] = from_float<T>(at(i));
   }
 }
 
@@ -767,6 +778,28 @@ extern "C" int sa_rope_cache_write(void* qkv, int dtype, int64_t row_stride, con
   else
     SA_REQUIRE(false, "rope_cache_write: unknown dtype %d", dtype);
   return check_launch("rope_cache_write");
+}
+
+extern "C" int sa_rope_cache_write_planes(const float* planes, int count, void* qkv, int64_t row_stride,
+                                          const int* positions, const float* timescale, float scale_factor,
+                                          float q_div, const int64_t* slot_mapping, void* k_pages, void* v_pages,
+                                          int T, int H, int K, int hd, int page_size, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(planes != nullptr && count >= 1, "rope_cache_write_planes: no planes");
+  SA_REQUIRE(hd > 0 && hd % 2 == 0, "rope_cache_write: head size %d must be even", hd);
+  SA_REQUIRE(H >= 0 && K >= 0 && H + 2 * K > 0, "rope_cache_write: bad head counts H=%d K=%d", H, K);
+  SA_REQUIRE(row_stride >= static_cast<int64_t>(H + 2 * K) * hd, "rope_cache_write: row stride %lld is too small",
+             (long long)row_stride);
+  SA_REQUIRE(page_size > 0 && scale_factor > 0.f && q_div > 0.f, "rope_cache_write: bad page size, scale factor or query scale");
+  SA_REQUIRE((k_pages == nullptr) == (v_pages == nullptr) && (k_pages == nullptr || slot_mapping != nullptr),
+             "rope_cache_write: key pages, value pages and slots come together");
+  const dim3 grid(T, H + 2 * K);
+  const int threads = hd / 2 >= 128 ? 128 : 64;
+  rope_cache_write_kernel<bf16><<<grid, threads, 0, stream>>>(
+      static_cast<bf16*>(qkv), row_stride, positions, timescale, 1.f / scale_factor, q_div, slot_mapping,
+      static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H, K, hd, page_size, planes, count,
+      static_cast<size_t>(T) * (H + 2 * K) * hd);
+  return check_launch("rope_cache_write_planes");
 }
 
 extern "C" int sa_rope(void* x, int dtype, int64_t row_stride, const int* positions, const float* timescale,

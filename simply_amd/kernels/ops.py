@@ -185,11 +185,19 @@ def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtyp
     return P
 
 
-def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, timescale: torch.Tensor | None, scale_factor: float,
-                     q_div: float, num_heads: int, num_kv_heads: int, head_dim: int,
+def rope_cache_write(qkv: "torch.Tensor | PartialSums", positions: torch.Tensor, timescale: torch.Tensor | None,
+                     scale_factor: float, q_div: float, num_heads: int, num_kv_heads: int, head_dim: int,
                      slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
-                     v_pages: torch.Tensor | None = None) -> None:
-    """In place on the fused projection rows; writes keys and values into their pages."""
+                     v_pages: torch.Tensor | None = None) -> torch.Tensor:
+    """In place on the fused projection rows; writes keys and values into their pages.  A projection whose cuts of K
+    are not added up yet is added up on the way (up to 256 tokens; its queries go to the tensor that it belongs in).
+    Returns the projection's tensor, of which the queries are then the rotated and scaled ones."""
+    planes = None
+    if isinstance(qkv, PartialSums):
+        if qkv.planes is not None and qkv.shape[0] <= 256 and qkv.dtype == torch.bfloat16:
+            planes, qkv = qkv.planes, qkv.out
+        else:
+            qkv = qkv.materialize()
     _dev(qkv, positions, timescale, slot_mapping, k_pages, v_pages)
     stride = _rows(qkv, "rope_cache_write: qkv")
     T = qkv.shape[0]
@@ -210,9 +218,15 @@ def rope_cache_write(qkv: torch.Tensor, positions: torch.Tensor, timescale: torc
                               f"size {head_dim}")
         if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
             raise KernelError("rope_cache_write: slot_mapping must be int64 [T]")
+    if planes is not None:
+        _lib.call("sa_rope_cache_write_planes", _ptr(planes), planes.shape[0], _ptr(qkv), stride, _ptr(positions),
+                  _ptr(timescale), float(scale_factor), float(q_div), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages),
+                  T, num_heads, num_kv_heads, head_dim, page_size, _stream())
+        return qkv
     _lib.call("sa_rope_cache_write", _ptr(qkv), _code(qkv), stride, _ptr(positions), _ptr(timescale),
               float(scale_factor), float(q_div), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), T, num_heads,
               num_kv_heads, head_dim, page_size, _stream())
+    return qkv
 
 
 def rope(x: torch.Tensor, positions: torch.Tensor, timescale: torch.Tensor, scale_factor: float, div: float,

@@ -71,11 +71,13 @@ class PagedAttention(Mixer):
                 ops.gemm_normed_rotary, w=self.qkv_proj, positions=ctx.positions, timescale=table, scale_factor=sf,
                 query_scale=self.query_scale, num_heads=H, num_kv_heads=K, head_dim=hd, **pages))
         else:
-            qkv = project(x, self.qkv_proj)
             if pe is None or rotary is not None:
+                # (the kernel behind the projection adds up its cuts of K, if it has any, on the way)
                 table, sf = rotary if rotary is not None else (None, 1.0)
-                ops.rope_cache_write(qkv, ctx.positions, table, sf, self.query_scale, H, K, hd, **pages)
+                qkv = ops.rope_cache_write(project(x, self.qkv_proj, defer_sum=True), ctx.positions, table, sf,
+                                           self.query_scale, H, K, hd, **pages)
             else:
+                qkv = project(x, self.qkv_proj)
                 # another position encoding: applied by the part itself, then the plain scale-and-write kernel
                 pe.apply(qkv, ctx.positions, H, hd, 1.0)
                 pe.apply(qkv[:, H * hd:], ctx.positions, K, hd, 1.0)

@@ -154,11 +154,11 @@ def pending_product(x: PendingNorm, run) -> torch.Tensor:
 
 
 def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | None = None,
-            out: torch.Tensor | None = None, activation: int = 0) -> torch.Tensor:
+            out: torch.Tensor | None = None, activation: int = 0, defer_sum: bool = False) -> torch.Tensor:
     """x . w^T (gated if w is a paired tiled weight) for activations x or a `PendingNorm`.  A pending norm is done
     inside the product's kernel when that kernel takes the sizes; otherwise it is materialized first.  `out`: where
     the result goes (a buffer of the caller's), else a new tensor.  `activation`: the gated product's (a code of
-    the ACTIVATIONS registry)."""
+    the ACTIVATIONS registry).  `defer_sum`: the result may be an `ops.PartialSums` (see `ops.gemm`)."""
     import functools
 
     from ..kernels import ops
@@ -169,7 +169,7 @@ def project(x, w, *, soft_cap: float | None = None, out_dtype: torch.dtype | Non
                                                         out_dtype=out_dtype or x.dtype, out=out,
                                                         activation=activation))
         x = x.materialize()
-    return ops.gemm(x, w, soft_cap=soft_cap, out_dtype=out_dtype, out=out, activation=activation)
+    return ops.gemm(x, w, soft_cap=soft_cap, out_dtype=out_dtype, out=out, activation=activation, defer_sum=defer_sum)
 
 
 class Part:

@@ -916,3 +916,30 @@ def test_deferred_sum_of_a_product_is_added_up_by_the_norm(M, N, K):
         assert torch.equal(y, whole)
     if (M, N, K) in ((64, 2304, 9216), (512, 2304, 9216)):
         assert isinstance(ops.gemm(a, w, defer_sum=True), ops.PartialSums)   # these sizes do cut K
+
+
+@pytest.mark.parametrize("T,H,K,hd,P", [(64, 8, 4, 256, 16), (17, 4, 2, 64, 16), (100, 16, 8, 128, 32), (33, 3, 1, 48, 4)])
+def test_deferred_sum_of_the_projection_is_added_up_by_the_rotary_kernel(T, H, K, hd, P):
+    """The fused q/k/v projection may leave the sum of its cuts of K to the rotate-and-write kernel: queries and
+    pages are the same to the bit as with the product's own sum kernel in between."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_tiles
+    D = 2304 if hd >= 128 else 512
+    N = (H + 2 * K) * hd
+    a = rand((T, D), torch.bfloat16, 101)
+    w = pack_tiles(rand((N, D), torch.bfloat16, 102, 0.05))
+    positions = (torch.arange(T, dtype=torch.int32) * 7 % 1000).cuda()
+    ts = (10000.0 ** (2 * torch.arange(hd // 2, dtype=torch.float64) / hd)).float().cuda()
+    pages = 2 * -(-T // P) + 3
+    slots = torch.randperm(pages * P, generator=torch.Generator().manual_seed(5))[:T].to(torch.int64).cuda()
+    results = []
+    for defer in (False, True):
+        kp = torch.zeros((pages, K, P, hd), dtype=torch.bfloat16, device="cuda")
+        vp = torch.zeros((pages, K, hd, P), dtype=torch.bfloat16, device="cuda")
+        y = ops.gemm(a, w, defer_sum=defer)
+        qkv = ops.rope_cache_write(y, positions, ts, 1.0, 16.0, H, K, hd, slot_mapping=slots, k_pages=kp, v_pages=vp)
+        results.append((qkv[:, :H * hd].clone(), kp, vp, isinstance(y, ops.PartialSums)))
+    (q0, k0, v0, _), (q1, k1, v1, cut) = results
+    assert torch.equal(q0, q1) and torch.equal(k0, k1) and torch.equal(v0, v1)
+    if (T, hd) == (64, 256):
+        assert cut   # this size does cut K
