@@ -55,15 +55,32 @@ __device__ inline void store_f(void* p, int dtype, size_t i, float v) {
   else static_cast<bf16*>(p)[i] = float_to_bf16(v);
 }
 
+// A value of all 64 lanes of a wave combined, in every lane (all lanes active): within rows of 16 lanes by data-parallel
+// primitives on the vector unit (quad exchanges, then the mirrored half row and the mirrored row: every lane of a quad,
+// then of a half row, holds the same partial result, so the mirror image brings the other half's), across rows by
+// gfx950's row swaps.  Eight instructions where six shuffles through the LDS crossbar took 500 to 700 clocks.
+template <int CTRL>
+__device__ __forceinline__ float lane_exchange(float v) {  // a DPP control: the value of another lane of the row
+  const int bits = __float_as_int(v);
+  return __int_as_float(__builtin_amdgcn_update_dpp(bits, bits, CTRL, 0xF, 0xF, false));
+}
+template <typename Op>
+__device__ __forceinline__ float wave_combine(float v, Op op) {
+  v = op(v, lane_exchange<0xB1>(v));   // quad_perm [1, 0, 3, 2]
+  v = op(v, lane_exchange<0x4E>(v));   // quad_perm [2, 3, 0, 1]
+  v = op(v, lane_exchange<0x141>(v));  // row_half_mirror
+  v = op(v, lane_exchange<0x140>(v));  // row_mirror
+  const unsigned u = __float_as_uint(v);
+  const auto rows = __builtin_amdgcn_permlane16_swap(u, u, false, false);   // [r0 r0 r2 r2], [r1 r1 r3 r3]
+  const unsigned w = __float_as_uint(op(__uint_as_float(rows[0]), __uint_as_float(rows[1])));
+  const auto halves = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return op(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+}
 __device__ inline float wave_sum(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
+  return wave_combine(v, [](float a, float b) { return a + b; });
 }
 __device__ inline float wave_max(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-  return v;
+  return wave_combine(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
 // Sum over a block of up to 1024 threads; every thread gets the result.  The
