@@ -160,13 +160,20 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
       load_set(0, c0 + sets * kUnroll);
       mul_set(0);
     }
-    if (G > 1) {  // column r of the sum: accumulator g's column g * kCols + r
+    if (G > 1) {  // column r of the sum: accumulator g's column g * kCols + r, that is its row of 16 lanes rotated
+                  // (a rotation on the vector unit, DPP row_ror, not a shuffle through LDS)
 #pragma unroll
       for (int p = 0; p < NP; ++p)
 #pragma unroll
-        for (int g = 1; g < G; ++g)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) acc[p][0][v] += __shfl(acc[p][g][v], kq * 16 + (r + g * kCols) % 16, kWave);
+        for (int v = 0; v < 4; ++v) {
+          if constexpr (G == 2) {
+            acc[p][0][v] += lane_exchange<0x120 + 8>(acc[p][1][v]);
+          } else if constexpr (G == 4) {
+            acc[p][0][v] += lane_exchange<0x120 + 12>(acc[p][1][v]);
+            acc[p][0][v] += lane_exchange<0x120 + 8>(acc[p][2][v]);
+            acc[p][0][v] += lane_exchange<0x120 + 4>(acc[p][3][v]);
+          }
+        }
     }
   } else {
     load_set(0, c0);
