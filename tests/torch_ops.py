@@ -81,6 +81,7 @@ def rope_cache_write(qkv, positions, timescale, scale_factor, q_div, num_heads, 
         rows[page, :, off] = k.to(k_pages.dtype)
         k_pages.copy_(rows_to_keys(rows))
         v_pages[page, :, :, off] = v.to(v_pages.dtype)     # value pages are [page, head, hd, page_size]
+    return qkv
 
 
 def rope(x, positions, timescale, scale_factor, div, num_heads, head_dim):
@@ -117,7 +118,8 @@ def squared_relu(x):
 ACTIVATIONS = (gelu_tanh, silu, squared_relu)   # by the kernels' activation codes
 
 
-def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0, activation=0):
+def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0, activation=0, defer_sum=False):
+    # (defer_sum: the kernels may leave a sum to the caller; this stand-in never cuts a product)
     out_dtype = out_dtype or a.dtype
     if getattr(w, "paired", False):
         from simply_amd.kernels.packing import unpack_gate_up
