@@ -498,6 +498,8 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
     if (K == 2048) SA_NORMED_EXACT(EPI, 8);                                                                        \
     if (K == 2304) SA_NORMED_EXACT(EPI, 9);                                                                        \
     if (K == 2560) SA_NORMED_EXACT(EPI, 10);                                                                       \
+    if (K == 3584) SA_NORMED_EXACT(EPI, 14);                                                                       \
+    if (K == 4608) SA_NORMED_EXACT(EPI, 18);                                                                       \
     if (K <= 2560) SA_NORMED(EPI, 10); \
     if (K <= 3584) SA_NORMED(EPI, 14); \
     SA_NORMED(EPI, 18);           \
@@ -549,6 +551,8 @@ extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_
   if (K == 2048) SA_ROTARY_EXACT(8);
   if (K == 2304) SA_ROTARY_EXACT(9);
   if (K == 2560) SA_ROTARY_EXACT(10);
+  if (K == 3584) SA_ROTARY_EXACT(14);
+  if (K == 4608) SA_ROTARY_EXACT(18);
 #undef SA_ROTARY_EXACT
   if (K <= 2560) SA_ROTARY(10);
   if (K <= 3584) SA_ROTARY(14);

@@ -120,7 +120,7 @@ class PendingNorm:
 
 def pending_fits_product(x, w) -> bool:
     """Whether the product kernel with the norms in front takes the pending norm `x` against the weight `w`
-    (bfloat16, up to 16 rows, a tiled weight of rows up to 2560 wide, RMSNorms with bfloat16 scales)."""
+    (bfloat16, up to 16 rows, a tiled weight of rows up to 2560 wide or 3584, RMSNorms with bfloat16 scales)."""
     from ..kernels import ops
     from ..kernels.packing import TiledWeight
 
@@ -131,10 +131,11 @@ def pending_fits_product(x, w) -> bool:
             and nn.scale.dtype == torch.bfloat16
             and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
             and isinstance(w, TiledWeight) and w.rows <= 16 * 2048   # every workgroup redoes the norms
-            # wider rows than 2560 leave the kernel too few registers to have its first weights on their way during
-            # the norms: measured at widths 3584 and 4608, the separate kernels are as fast at 8 rows and 10-20 %
-            # faster at 16
-            and w.cols <= 2560
+            # up to 2560 wide, and 3584 (a whole number of 256-element pieces, for which the kernel has a prologue
+            # without per-piece tests: 5 to 20 % faster than the separate kernels up to 8 rows, even at 16).  Other
+            # widths above 2560 leave the kernel too few registers to have its first weights on their way during the
+            # norms (at 4608 it spills: the separate kernels are 5 % faster at 8 rows)
+            and (w.cols <= 2560 or w.cols == 3584)
             and ops.gemm_normed_takes(x.residual.shape[0], w)
             and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
 
