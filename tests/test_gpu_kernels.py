@@ -851,7 +851,8 @@ def test_bfloat16_rounding_of_the_kernels():
 
 
 @pytest.mark.parametrize("M", [1, 8, 13])
-@pytest.mark.parametrize("H,Kh,hd,P,K", [(8, 4, 256, 16, 2304), (4, 2, 64, 16, 128), (3, 1, 32, 48, 96), (2, 2, 128, 32, 2560)])
+@pytest.mark.parametrize("H,Kh,hd,P,K", [(8, 4, 256, 16, 2304), (4, 2, 64, 16, 128), (3, 1, 32, 48, 96), (2, 2, 128, 32, 2560), (4, 2, 256, 16, 3584),
+                                         (4, 4, 128, 16, 4608)])
 @pytest.mark.parametrize("rotate", [True, False])
 def test_gemm_normed_rotary(M, H, Kh, hd, P, K, rotate):
     """Norms, q/k/v projection, rotation, query scale and cache write in one kernel against the same from the
@@ -867,6 +868,11 @@ def test_gemm_normed_rotary(M, H, Kh, hd, P, K, rotate):
     pages = 5
     slots = torch.randperm(pages * P)[:M].to(torch.int64).cuda()
     norm = dict(post_weight=wp, post_eps=1e-6, post_plus_one=True, next_weight=wn, next_eps=1e-5, next_plus_one=True)
+    if not ops.gemm_normed_takes(M, tw):   # 13 rows of 4,608 do not fit in LDS: refused, with the sizes in the message
+        with pytest.raises(ops.KernelError, match=f"M={M} K={K}"):
+            ops.gemm_normed_rotary(y, h, torch.empty_like(h), tw, **norm, positions=positions, timescale=ts, scale_factor=1.0,
+                                   query_scale=12.0, num_heads=H, num_kv_heads=Kh, head_dim=hd)
+        return
     for with_y in (True, False):
         kp, vp = torch.zeros((pages, Kh, P, hd), dtype=torch.bfloat16).cuda(), torch.zeros((pages, Kh, hd, P), dtype=torch.bfloat16).cuda()
         kp2, vp2 = kp.clone(), vp.clone()
