@@ -181,6 +181,12 @@ __global__ __launch_bounds__(kWaves* kWave) void gemm_normed_kernel(
         }
       }
       const float rr = post ? rsqrtf(wave_sum(ss) / static_cast<float>(K) + eps_post) : 1.f;
+      // (the row's y is converted to float again below, from a value that the compiler takes for a new one: it would
+      // otherwise keep the first loop's 4 NCH floats alive through the sum, which at 14 and 18 pieces is what spills)
+      if constexpr (NCH > 10) {
+  #pragma unroll
+        for (int c = 0; c < NCH; ++c) asm volatile("" : "+v"(yv[c]));
+      }
       float ss2 = 0.f;
   #pragma unroll
       for (int c = 0; c < NCH; ++c) {

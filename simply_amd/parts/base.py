@@ -120,7 +120,7 @@ class PendingNorm:
 
 def pending_fits_product(x, w) -> bool:
     """Whether the product kernel with the norms in front takes the pending norm `x` against the weight `w`
-    (bfloat16, up to 16 rows, a tiled weight of rows up to 2560 wide or 3584, RMSNorms with bfloat16 scales)."""
+    (bfloat16, up to 16 rows, a tiled weight of rows up to 2560 wide, or 3584 or 4608, RMSNorms with bfloat16 scales)."""
     from ..kernels import ops
     from ..kernels.packing import TiledWeight
 
@@ -130,12 +130,12 @@ def pending_fits_product(x, w) -> bool:
     return (x.dtype == torch.bfloat16 and nn is not None and getattr(nn, "fusable_rms", False)
             and nn.scale.dtype == torch.bfloat16
             and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
-            and isinstance(w, TiledWeight) and w.rows <= 16 * 2048   # every workgroup redoes the norms
-            # up to 2560 wide, and 3584 (a whole number of 256-element pieces, for which the kernel has a prologue
-            # without per-piece tests: 5 to 20 % faster than the separate kernels up to 8 rows, even at 16).  Other
-            # widths above 2560 leave the kernel too few registers to have its first weights on their way during the
-            # norms (at 4608 it spills: the separate kernels are 5 % faster at 8 rows)
-            and (w.cols <= 2560 or w.cols == 3584)
+            and isinstance(w, TiledWeight) and w.rows <= 16 * 8192   # (not the head over a large vocabulary)
+            # up to 2560 wide, and 3584 and 4608 (whole numbers of 256-element pieces, for which the kernel has a
+            # prologue without per-piece tests: 5 to 25 % faster than the separate kernels at the 9B and 27B sizes).
+            # Other widths above 2560 leave the kernel too few registers to have its first weights on their way
+            # during the norms
+            and (w.cols <= 2560 or w.cols in (3584, 4608))
             and ops.gemm_normed_takes(x.residual.shape[0], w)
             and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
 
