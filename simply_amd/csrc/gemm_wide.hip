@@ -340,7 +340,7 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     // time fitted to measurements at the 2B, 9B and 27B sizes (64 to 2,048 rows, seven tiles, one to fourteen cuts;
     // it is within 6 % of the best measured choice nearly everywhere, and a fifth faster in sum than either the
     // uncut tiles above or the tiled kernel with its cut: the 2B down projection at 512 rows takes 36 us against 55).
-    if (epi == 0 && M >= 17 && M <= 1536) {
+    if (epi == 0 && M <= 1536) {  // (fewer than 17 rows come here only against a very long K)
       struct Tile { int code, rows, wrows; double eff, start; };  // share of the MFMA rate in the loop; us to start
       static const Tile tiles[7] = {{3128128, 128, 128, 0.425, 1.44}, {3128256, 128, 256, 0.535, 2.03},
                                     {3192128, 192, 128, 0.535, 1.25}, {3256128, 256, 128, 0.615, 1.58},

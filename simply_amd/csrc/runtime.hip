@@ -55,13 +55,16 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
   // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower).  Not from 8 rows on
   // against so many weight rows that the tiled kernel fills the GPU without a cut of K (the head over a large
   // vocabulary: 7 % faster at 8 rows, 30 % at 16, 80 % at 32; up to 6 rows the few-rows kernel wins).
-  // Nor against a very long K (the 27B down projection, 36864: the tiled kernel with its cut of K is 15 % faster at
-  // one row and 40 % at 16; at the 9B size, 14336, the few-rows kernel still wins up to 12 rows).
+  // Nor against a very long K (the 27B down projection, 36864: kernels that cut K over workgroups are 15 % faster at
+  // one row and 40 % at 16), nor from 9 rows on against K of 8192 and more (the 2B and 9B down projections: the
+  // wide kernel with its cut takes 13.0 against 16.8 us and 24.2 against 26.7 at 16 rows; up to 8 rows, where a
+  // load of activations serves several chunks of K, the few-rows kernel wins).
   const bool many_weight_rows = packed && epilogue != 1 && M >= 8 && N >= 65536;
   const bool long_k = packed && epilogue != 1 && K >= 24576;
+  const bool longish_k = packed && epilogue == 0 && M >= 9 && K >= 8192 && N <= 16384;
   const bool tiled_first = many_weight_rows || long_k;
   if (algo == 2 ||
-      (algo == 0 && bf16_in && !tiled_first && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4096)))) {
+      (algo == 0 && bf16_in && !tiled_first && !longish_k && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4096)))) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
@@ -77,7 +80,9 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
   // 17 to 1,536 rows without an epilogue (q/k/v, output and down projections of portions of prompts and of many
   // decoding requests): the wide kernel with a tile and a cut of K that it chooses for the sizes (2B down projection:
   // 13 us at 17 rows, 15 at 64, 36 at 512, against 19, 23 and 55 for the tiled kernel with its cut)
-  const bool small_wide = epilogue == 0 && M >= 17 && M <= 1536 && N <= 16384;
+  // ... and up to 16 rows against a very long K (the 27B down projection: 62 us against 67 for the tiled kernel
+  // with its cut and 74 to 84 for the few-rows kernel)
+  const bool small_wide = epilogue == 0 && N <= 16384 && ((M >= 17 && M <= 1536) || (long_k && M <= 16) || longish_k);
   const bool wide_first = !gemm_streams_weights(M, NW, K) || (epilogue == 1 && M > 16) || small_wide;
   if (algo == 4 || (algo == 0 && bf16_in && packed && wide_first)) {
     const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
