@@ -625,6 +625,24 @@ def test_gemm_dispatch_at_a_few_hundred_rows(M, N, K):
     assert not out[:, N:].any()
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 24576), (8, 1024, 24576), (16, 520, 24640), (9, 2304, 9216), (12, 2304, 8192),
+                                   (16, 2304, 9216), (13, 1000, 8256), (9, 2304, 8200)])
+def test_gemm_dispatch_of_few_rows_against_a_long_k(M, N, K):
+    """Few rows against a very long K, and 9 to 16 rows against a long one, are cut over workgroups by the
+    dispatcher (the wide kernel; where K is no multiple of 64, what takes it): against the reference, also with
+    rows of wider rows in and out."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_tiles
+    a = rand((M, K), torch.bfloat16, 150)
+    w = rand((N, K), torch.bfloat16, 151, 0.03)
+    t = dict(rtol=2e-2, atol=3e-2)
+    torch.testing.assert_close(ops.gemm(a, pack_tiles(w)).float(), ref.gemm(a, w).float(), **t)
+    big, out = rand((M, K + 64), torch.bfloat16, 152), torch.zeros((M, N + 8), dtype=torch.bfloat16, device="cuda")
+    ops.gemm(big[:, 32:32 + K], pack_tiles(w), out=out[:, :N])
+    torch.testing.assert_close(out[:, :N].float(), ref.gemm(big[:, 32:32 + K], w).float(), **t)
+    assert not out[:, N:].any()
+
+
 @pytest.mark.parametrize("activation", [0, 1, 2])
 @pytest.mark.parametrize("M", [5, 16, 40, 300])
 def test_gated_activations_in_every_product_kernel(M, activation):
