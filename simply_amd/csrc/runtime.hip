@@ -61,10 +61,15 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
   // load of activations serves several chunks of K, the few-rows kernel wins).
   const bool many_weight_rows = packed && epilogue != 1 && M >= 8 && N >= 65536;
   const bool long_k = packed && epilogue != 1 && K >= 24576;
-  const bool longish_k = packed && epilogue == 0 && M >= 9 && K >= 8192 && N <= 16384;
+  // (... or against K of 4096 and more where the weight is large, 16 M elements: 27B q/k/v 16.0 against 18.6 us at
+  // 16 rows; the same size decides for 17 to 32 rows: 9B q/k/v 16.0 against 22.5 us at 32 rows with the wide kernel,
+  // 2B q/k/v 9.5 against 9.8 with the few-rows kernel)
+  const bool large = static_cast<int64_t>(N) * K >= (int64_t{16} << 20);
+  const bool longish_k = packed && epilogue == 0 && M >= 9 && N <= 16384 && (K >= 8192 || (K >= 4096 && large));
   const bool tiled_first = many_weight_rows || long_k;
   if (algo == 2 ||
-      (algo == 0 && bf16_in && !tiled_first && !longish_k && (M <= 16 || (M <= 32 && epilogue != 1 && K < 4096)))) {
+      (algo == 0 && bf16_in && !tiled_first && !longish_k &&
+       (M <= 16 || (M <= 32 && epilogue != 1 && K < 4096 && !(packed && epilogue == 0 && large && N <= 16384))))) {
     const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
     SA_REQUIRE(takes || algo == 0,
                "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
