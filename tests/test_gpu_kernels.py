@@ -626,10 +626,11 @@ def test_gemm_dispatch_at_a_few_hundred_rows(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1024, 24576), (8, 1024, 24576), (16, 520, 24640), (9, 2304, 9216), (12, 2304, 8192),
-                                   (16, 2304, 9216), (13, 1000, 8256), (9, 2304, 8200)])
+                                   (16, 2304, 9216), (13, 1000, 8256), (9, 2304, 8200), (24, 8192, 3584), (12, 4608, 4096),
+                                   (32, 5000, 3584)])
 def test_gemm_dispatch_of_few_rows_against_a_long_k(M, N, K):
-    """Few rows against a very long K, and 9 to 16 rows against a long one, are cut over workgroups by the
-    dispatcher (the wide kernel; where K is no multiple of 64, what takes it): against the reference, also with
+    """Few rows against a very long K, 9 to 16 rows against a long one and 9 to 32 rows against a large weight are
+    cut over workgroups by the dispatcher (the wide kernel; where K is no multiple of 64, what takes it): against the reference, also with
     rows of wider rows in and out."""
     from simply_amd.kernels import ops
     from simply_amd.kernels.packing import pack_tiles
