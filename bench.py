@@ -79,8 +79,8 @@ def fill_cache_random(lm, std: float = 0.5, seed: int = 0) -> None:
     gen = torch.Generator(device=lm.executor.device)
     gen.manual_seed(seed)
     for v in lm.executor.cache.views:
-        if v.k_pages is not None and v.write:
-            for t in (v.k_pages, v.v_pages):
+        if v.pages and v.write:
+            for t in v.pages.values():
                 flat = t.view(-1)     # in slices, so that no float32 copy of a whole pool is made
                 step = 1 << 26
                 for i in range(0, flat.numel(), step):

@@ -13,7 +13,10 @@ once (`windowed_pool_pages`), as the reference sizes its local pool by the windo
 simply/serving/page_server.py:180-196).
 
 Bookkeeping is separate from storage: `CacheManager(device=None)` keeps no tensors and runs
-anywhere.
+anywhere.  The manager counts pages and slots only; what a page or a slot holds, and in which layout, is
+said by the need that a mixer declares (simply_amd/parts/base.py: `PagedNeed.page_tensors`,
+`StateNeed.slot_tensor`), as the reference keys its groups by what a layer needs
+(simply/utils/ragged_paged_attention.py:865-867) and leaves the tensors to the layer.
 """
 from __future__ import annotations
 
@@ -23,8 +26,6 @@ from typing import Hashable, Sequence
 
 import numpy as np
 import torch
-
-from ..parts.base import PagedKVNeed, StateNeed
 
 
 class CacheError(RuntimeError):
@@ -89,11 +90,13 @@ class _Sequence:
 
 
 class CacheGroup:
-    """Pages and block tables of the layers that share one `PagedKVNeed`."""
+    """Pages and block tables of the layers whose paged needs are equal."""
 
-    def __init__(self, group_id: int, need: PagedKVNeed, page_size: int, num_pages: int, num_slots: int,
+    def __init__(self, group_id: int, need, page_size: int, num_pages: int, num_slots: int,
                  max_blocks_per_seq: int):
         self.group_id, self.need = group_id, need
+        #: None: every token's page is kept; n: pages that lie wholly before the last n tokens are given back
+        self.window = getattr(need, "window", None)
         self.page_size, self.num_slots, self.max_blocks = int(page_size), int(num_slots), int(max_blocks_per_seq)
         self.pool = PagePool(num_pages)
         #: table[slot, absolute block] = page, -1 where no page is held
@@ -106,9 +109,9 @@ class CacheGroup:
         """Blocks that no query at position >= num_computed can see (windowed groups only):
         the first visible key is num_computed - window + 1
         (simply/utils/ragged_paged_attention.py:441-445 with window_size = window - 1)."""
-        if self.need.window is None:
+        if self.window is None:
             return 0
-        return max(num_computed - self.need.window + 1, 0) // self.page_size
+        return max(num_computed - self.window + 1, 0) // self.page_size
 
     def pages_needed(self, rid: Hashable, num_computed: int, q_len: int) -> int:
         """New pages for tokens [num_computed, num_computed + q_len), net of those that become free first."""
@@ -224,12 +227,22 @@ class StateSlots:
 class CacheView:
     """What one schedule entry's mixer is handed: its own storage (or that of the entry it reads)."""
 
-    need: PagedKVNeed | StateNeed | None
+    need: object | None
     group_id: int | None = None
-    k_pages: torch.Tensor | None = None   # [num_pages, kv heads, page_size, head_dim]
-    v_pages: torch.Tensor | None = None   # [num_pages, kv heads, head_dim, page_size]
-    state: torch.Tensor | None = None     # [num_slots, *need.shape]
+    #: the page tensors that the need asked for, by the need's own names (first dimension: pages of the group's pool)
+    pages: dict = dataclasses.field(default_factory=dict)
+    state: torch.Tensor | None = None     # [num_slots, ...] as the need's `slot_tensor` made it
     write: bool = True                    # False: this entry reads the cache of another entry
+
+    @property
+    def k_pages(self) -> torch.Tensor | None:
+        """Key pages of a `PagedKVNeed`: [num_pages, kv heads, page_size, head_dim]."""
+        return self.pages.get("k")
+
+    @property
+    def v_pages(self) -> torch.Tensor | None:
+        """Value pages of a `PagedKVNeed`: [num_pages, kv heads, head_dim, page_size]."""
+        return self.pages.get("v")
 
 
 class CacheManager:
@@ -260,7 +273,7 @@ class CacheManager:
         self._group_entries: dict[int, list[int]] = {}
         self._device_tables: dict[int, torch.Tensor] = {}
         self._stage_host = self._stage_dev = self._stage_done = None  # what `sync_tables` sends its rows through
-        by_need: dict[PagedKVNeed, CacheGroup] = {}
+        by_need: dict[object, CacheGroup] = {}
         max_blocks = ceil_div(self.max_seq_len, self.page_size)
         for i, (need, cache_from) in enumerate(needs):
             if cache_from is not None:
@@ -272,12 +285,14 @@ class CacheManager:
                 continue
             if need is None:
                 self.views.append(CacheView(None))
-            elif isinstance(need, PagedKVNeed):
+            elif callable(getattr(need, "page_tensors", None)):
+                # something per token, in pages: layers with equal needs share pool, free list and block table
                 group = by_need.get(need)
                 if group is None:
                     pages = self.num_pages
-                    if need.window is not None and max_step_tokens is not None:
-                        pages = min(pages, windowed_pool_pages(need.window, self.page_size, self.num_slots,
+                    window = getattr(need, "window", None)
+                    if window is not None and max_step_tokens is not None:
+                        pages = min(pages, windowed_pool_pages(window, self.page_size, self.num_slots,
                                                                int(max_step_tokens)))
                     if group_pages is not None:
                         pages = int(group_pages(need, pages))
@@ -287,22 +302,27 @@ class CacheManager:
                     self._group_entries[group.group_id] = []
                 view = CacheView(need, group.group_id)
                 if device is not None:
-                    fill = float("nan") if poison else 0.0
                     n = group.pool.num_pages
-                    view.k_pages = torch.full((n, need.num_kv_heads, self.page_size, need.head_dim), fill,
-                                              dtype=dtype, device=device)
-                    # values are stored transposed, so that the keys of a page are contiguous for each dimension
-                    view.v_pages = torch.full((n, need.num_kv_heads, need.head_dim, self.page_size), fill,
-                                              dtype=dtype, device=device)
+                    view.pages = dict(need.page_tensors(n, self.page_size, dtype, device,
+                                                        float("nan") if poison else 0.0))
+                    for name, t in view.pages.items():
+                        if t.dim() < 1 or t.shape[0] != n:
+                            raise CacheError(f"schedule entry {i}: page tensor {name!r} of {need!r} has shape "
+                                             f"{tuple(t.shape)}; its first dimension must be the {n} pages")
                 self._group_entries[group.group_id].append(i)
                 self.views.append(view)
-            elif isinstance(need, StateNeed):
+            elif callable(getattr(need, "slot_tensor", None)):
+                # something of fixed size per request: a row per request slot
                 view = CacheView(need)
                 if device is not None:
-                    view.state = torch.zeros((self.num_slots, *need.shape), dtype=need.dtype, device=device)
+                    view.state = need.slot_tensor(self.num_slots, device)
+                    if view.state.dim() < 1 or view.state.shape[0] != self.num_slots:
+                        raise CacheError(f"schedule entry {i}: the state of {need!r} has shape "
+                                         f"{tuple(view.state.shape)}; its first dimension must be the {self.num_slots} slots")
                 self.views.append(view)
             else:
-                raise CacheError(f"schedule entry {i}: unknown cache need {need!r}")
+                raise CacheError(f"schedule entry {i}: cache need {need!r} says neither page_tensors(...) (something "
+                                 f"per token) nor slot_tensor(...) (something of fixed size per request)")
         if device is not None:
             for g in self.groups:
                 self._device_tables[g.group_id] = torch.full((self.num_slots, g.max_blocks), -1, dtype=torch.int32,
@@ -356,7 +376,7 @@ class CacheManager:
         points = self._release_points(wants)
         for g in self.groups:
             free = g.pool.num_free
-            if g.need.window is not None:
+            if g.window is not None:
                 free += sum(g.releasable(rid, at) for rid, at in points.items())
             if sum(g.new_blocks(rid, nc + q) for rid, nc, q in wants) > free:
                 return False
@@ -370,9 +390,9 @@ class CacheManager:
         for g in self.groups:
             peak = ceil_div(num_tokens, self.page_size)
             free = g.pool.num_free
-            if g.need.window is not None:
+            if g.window is not None:
                 step = min(num_tokens, max(int(max_step_tokens), 1))
-                peak = min(peak, ceil_div(g.need.window - 1 + step, self.page_size) + 1)
+                peak = min(peak, ceil_div(g.window - 1 + step, self.page_size) + 1)
                 free += sum(g.releasable(rid, at) for rid, at in points.items())
             if peak > free:
                 return False
@@ -395,7 +415,7 @@ class CacheManager:
         for rid, nc, _ in wants:
             self.issued[rid] = min(self.issued[rid], nc)    # its queries from nc on are still to come
         for g in self.groups:
-            if g.need.window is not None:
+            if g.window is not None:
                 for rid, at in points.items():
                     self._poison(g, g.release_window(rid, at))
             for rid, nc, q in wants:
@@ -421,8 +441,9 @@ class CacheManager:
             return
         idx = torch.as_tensor(list(pages), dtype=torch.long, device=self.device)
         for e in self._group_entries[g.group_id]:
-            self.views[e].k_pages[idx] = float("nan")
-            self.views[e].v_pages[idx] = float("nan")
+            for t in self.views[e].pages.values():
+                if t.is_floating_point():
+                    t[idx] = float("nan")
 
     def check(self) -> None:
         for g in self.groups:
@@ -450,7 +471,7 @@ class CacheManager:
     def check_readable(self, group_id: int, rid: Hashable, start: int, q_len: int) -> None:
         """Every key that the queries at [start, start + q_len) may read has a page."""
         g = self.groups[group_id]
-        lo = 0 if g.need.window is None else max(start - g.need.window + 1, 0)
+        lo = 0 if g.window is None else max(start - g.window + 1, 0)
         blocks = g.table[g.seqs[rid].slot, lo // g.page_size: ceil_div(start + q_len, g.page_size)]
         if (blocks < 0).any():
             raise CacheError(f"request {rid!r}: keys [{lo}, {start + q_len}) are not all held in group {group_id}")
@@ -494,5 +515,4 @@ class CacheManager:
     def bytes_per_token(self) -> int:
         """Bytes of cache that one token takes over all schedule entries that keep their own."""
         esize = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * v.need.num_kv_heads * v.need.head_dim * esize for v in self.views
-                   if isinstance(v.need, PagedKVNeed) and v.write)
+        return sum(v.need.bytes_per_token(esize) for v in self.views if v.group_id is not None and v.write)

@@ -12,6 +12,7 @@ import math
 from typing import Any, Mapping
 
 from ..registry import ARCHITECTURES
+from ..weights import binding as wb
 from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 
 SLIDING = "sliding_attention"
@@ -67,6 +68,9 @@ class Gemma2Config:
     pad_token_id: int | None
     initializer_range: float
     torch_dtype: str
+    #: how the folder stores the tensors: one of WEIGHT_LAYOUTS ("hf": [out, in] matrices under the names of the
+    #: published Gemma 2 folders)
+    weight_layout: str = "hf"
 
     architecture = "Gemma2ForCausalLM"
 
@@ -123,6 +127,7 @@ class Gemma2Config:
             pad_token_id=d.get("pad_token_id"),
             initializer_range=float(d.get("initializer_range", 0.02)),
             torch_dtype=str(d.get("torch_dtype", d.get("dtype", "bfloat16"))),
+            weight_layout=str(d.get("weight_layout", "hf")),
         )
         cfg.validate()
         return cfg
@@ -147,6 +152,9 @@ class Gemma2Config:
                 raise ConfigError(f"config.json: unknown layer type {t!r}; known: {SLIDING}, {FULL}")
         if SLIDING in self.layer_types and (self.sliding_window is None or self.sliding_window < 1):
             raise ConfigError("config.json: sliding layers need sliding_window >= 1")
+        if self.weight_layout not in WEIGHT_LAYOUTS:
+            raise ConfigError(f"config.json: unknown weight_layout {self.weight_layout!r}; known: "
+                              + ", ".join(sorted(WEIGHT_LAYOUTS)))
         if self.query_pre_attn_scalar <= 0 or self.rms_norm_eps <= 0 or self.rope_theta <= 0:
             raise ConfigError("config.json: query_pre_attn_scalar, rms_norm_eps and rope_theta must be positive")
 
@@ -169,15 +177,16 @@ class Gemma2Config:
         """The parts of Gemma 2 (simply/model_lib.py:2427 TransformerBlock, :1605 Attention,
         :643 FeedForward, :114 LayerNorm) as data."""
         D, H, K, hd = self.hidden_size, self.num_attention_heads, self.num_key_value_heads, self.head_dim
+        names = WEIGHT_LAYOUTS[self.weight_layout](self)
 
-        def norm(name: str) -> PartSpec:
+        def norm(name) -> PartSpec:
             # simply/config_lib.py:863 use_rmsnorm, :296 norm_scale_plus_one
             return PartSpec("rmsnorm", {"dim": D, "eps": self.rms_norm_eps, "scale_plus_one": True},
                             {"scale": name})
 
         layers = []
         for i, kind in enumerate(self.layer_types):
-            p = f"model.layers.{i}."
+            t = names.layer(i)
             mixer = PartSpec(
                 "paged_attention",
                 {
@@ -189,37 +198,35 @@ class Gemma2Config:
                     "position_encoding": PartSpec("rope", {"head_dim": hd, "base": self.rope_theta,
                                                            "scale_factor": 1.0}),
                 },
-                {"q_proj": p + "self_attn.q_proj.weight", "k_proj": p + "self_attn.k_proj.weight",
-                 "v_proj": p + "self_attn.v_proj.weight", "o_proj": p + "self_attn.o_proj.weight"},
+                {n: t[n] for n in ("q_proj", "k_proj", "v_proj", "o_proj")},
             )
             ffn = PartSpec(
                 "gated_dense",
                 {"hidden_size": D, "intermediate_size": self.intermediate_size, "activation": "gelu_tanh"},
-                {"gate_proj": p + "mlp.gate_proj.weight", "up_proj": p + "mlp.up_proj.weight",
-                 "down_proj": p + "mlp.down_proj.weight"},
+                {n: t[n] for n in ("gate_proj", "up_proj", "down_proj")},
             )
             layers.append(LayerSpec(
                 block=PartSpec("sandwich"),  # pre-norm, part, post-norm, then the residual (model_lib.py:2669-2703)
                 mixer=mixer,
                 feed_forward=ffn,
                 norms={
-                    "pre_mixer": norm(p + "input_layernorm.weight"),            # pre_ln_0
-                    "post_mixer": norm(p + "post_attention_layernorm.weight"),  # post_ln_0
-                    "pre_ffn": norm(p + "pre_feedforward_layernorm.weight"),    # pre_ln_1
-                    "post_ffn": norm(p + "post_feedforward_layernorm.weight"),  # post_ln_1
+                    "pre_mixer": norm(t["pre_mixer"]),     # pre_ln_0
+                    "post_mixer": norm(t["post_mixer"]),   # post_ln_0
+                    "pre_ffn": norm(t["pre_ffn"]),         # pre_ln_1
+                    "post_ffn": norm(t["post_ffn"]),       # post_ln_1
                 },
             ))
-        head_tensor = "model.embed_tokens.weight" if self.tie_word_embeddings else "lm_head.weight"
+        head_tensor = names.embedding if self.tie_word_embeddings else names.head
         spec = ModelSpec(
             architecture=self.architecture,
             hidden_size=D,
             vocab_size=self.vocab_size,
             # simply/utils/module.py:472-481: lookup times sqrt(dim)
             embedding=PartSpec("scaled_embedding", {"vocab_size": self.vocab_size, "dim": D, "scale": math.sqrt(D)},
-                               {"table": "model.embed_tokens.weight"}),
+                               {"table": names.embedding}),
             layers=tuple(layers),
             schedule=tuple(ScheduleEntry(i) for i in range(self.num_hidden_layers)),
-            final_norm=norm("model.norm.weight"),
+            final_norm=norm(names.final_norm),
             head=PartSpec("linear_head", {"vocab_size": self.vocab_size, "dim": D,
                                           "soft_cap": self.final_logit_softcapping},
                           {"weight": head_tensor}),
@@ -227,10 +234,104 @@ class Gemma2Config:
             eos_token_ids=self.eos_token_ids,
             initializer_range=self.initializer_range,
             # a folder of a tied model may store the head once more under its own name
-            copies={"lm_head.weight": "model.embed_tokens.weight"} if self.tie_word_embeddings else {},
+            copies={names.head: names.embedding} if self.tie_word_embeddings else {},
         )
         spec.validate()
         return spec
 
+
+# ---------------------------------------------------------------------- how a folder may store the tensors
+@dataclasses.dataclass(frozen=True)
+class TensorNames:
+    """Bindings (simply_amd/weights/binding.py) of the model's tensors for one stored layout: `layer(i)` gives, for
+    the i-th layer, the part's parameter names q_proj, k_proj, v_proj ([heads * head size, width], rows
+    head-major), o_proj ([width, heads * head size]), gate_proj, up_proj ([intermediate, width]), down_proj
+    ([width, intermediate]) and the four norms by their role in the block."""
+
+    embedding: str
+    head: str
+    final_norm: str
+    layer: "callable"
+
+
+def _hf_names(cfg: Gemma2Config) -> TensorNames:
+    """[out, in] matrices under the names of the published Gemma 2 folders: every tensor as it is stored.  (The
+    reference reads a folder of this convention with `nhd->dnh` of the rows split into heads,
+    simply/utils/checkpoint_lib.py:432-458; which of the four norm names plays which role in the block is this
+    engine's reading: no file of the reference names a Gemma 2 folder's norms.)"""
+    def layer(i: int):
+        p = f"model.layers.{i}."
+        t = {n: p + f"self_attn.{n}.weight" for n in ("q_proj", "k_proj", "v_proj", "o_proj")}
+        t.update({n: p + f"mlp.{n}.weight" for n in ("gate_proj", "up_proj", "down_proj")})
+        t.update(pre_mixer=p + "input_layernorm.weight", post_mixer=p + "post_attention_layernorm.weight",
+                 pre_ffn=p + "pre_feedforward_layernorm.weight", post_ffn=p + "post_feedforward_layernorm.weight")
+        return t
+
+    return TensorNames("model.embed_tokens.weight", "lm_head.weight", "model.norm.weight", layer)
+
+
+def _simply_names(cfg: Gemma2Config) -> TensorNames:
+    """The reference's own parameter tree, flattened with '/': projections with separate axes [width, heads, head
+    size] (q/k/v: simply/model_lib.py:2047-2068 `ihd,...i->...hd`; o_proj the same axes, `ihd,...hd->...i`),
+    feed-forward matrices [in, out] (:671-694 `io,...i->...o`), norms pre_ln_0, post_ln_0, pre_ln_1, post_ln_1
+    (:2669-2703)."""
+    D, H, K, hd, F = (cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                      cfg.intermediate_size)
+
+    def layer(i: int):
+        p = f"params/block_{i}/"
+        return {
+            "q_proj": wb.heads_to_rows(wb.stored(p + "attn/q_proj/w", (D, H, hd)), "dnh"),
+            "k_proj": wb.heads_to_rows(wb.stored(p + "attn/k_proj/w", (D, K, hd)), "dnh"),
+            "v_proj": wb.heads_to_rows(wb.stored(p + "attn/v_proj/w", (D, K, hd)), "dnh"),
+            "o_proj": wb.heads_to_cols(wb.stored(p + "attn/o_proj/w", (D, H, hd)), "dnh"),
+            "gate_proj": wb.transpose(wb.stored(p + "ffn/ffn_0_gate/w", (D, F))),
+            "up_proj": wb.transpose(wb.stored(p + "ffn/ffn_0/w", (D, F))),
+            "down_proj": wb.transpose(wb.stored(p + "ffn/ffn_1/w", (F, D))),
+            "pre_mixer": p + "pre_ln_0/scale", "post_mixer": p + "post_ln_0/scale",
+            "pre_ffn": p + "pre_ln_1/scale", "post_ffn": p + "post_ln_1/scale"}
+
+    return TensorNames("params/embed_linear/w", "params/output_layer/w", "params/final_ln/scale", layer)
+
+
+def _gemma_tree_names(transposed_gating: bool):
+    """The Gemma parameter tree that the reference converts with the rules of
+    simply/utils/checkpoint_lib.py:256-335 (Gemma2Format; with `transposed_gating` Gemma2TransposeFormat, whose
+    gating matrices are stored [2, out, in]): q, k and v stacked in `qkv_einsum` [3, heads, width, head size] when
+    the model has as many key heads as query heads, else `q_einsum` [heads, width, head size] and `kv_einsum`
+    [2, key heads, width, head size]; `attn_vec_einsum` [heads, head size, width]; gate and the other factor
+    stacked in `gating_einsum`; `linear` [in, out]; the norms' roles as :249-254 maps them."""
+    def names(cfg: Gemma2Config) -> TensorNames:
+        D, H, K, hd, F = (cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                          cfg.intermediate_size)
+
+        def layer(i: int):
+            p = f"params/transformer/layer_{i}/"
+            if H == K:
+                qkv = wb.stored(p + "attn/qkv_einsum/w", (3, H, D, hd))
+                q, k, v = (wb.select(qkv, j) for j in range(3))
+            else:
+                kv = wb.stored(p + "attn/kv_einsum/w", (2, K, D, hd))
+                q, k, v = wb.stored(p + "attn/q_einsum/w", (H, D, hd)), wb.select(kv, 0), wb.select(kv, 1)
+            gating = wb.stored(p + "mlp/gating_einsum/w", (2, F, D) if transposed_gating else (2, D, F))
+            factor = (lambda j: wb.select(gating, j)) if transposed_gating else (lambda j: wb.transpose(wb.select(gating, j)))
+            return {
+                "q_proj": wb.heads_to_rows(q, "ndh"), "k_proj": wb.heads_to_rows(k, "ndh"),
+                "v_proj": wb.heads_to_rows(v, "ndh"),
+                "o_proj": wb.heads_to_cols(wb.stored(p + "attn/attn_vec_einsum/w", (H, hd, D)), "nhd"),
+                "gate_proj": factor(0), "up_proj": factor(1),
+                "down_proj": wb.transpose(wb.stored(p + "mlp/linear/w", (F, D))),
+                "pre_mixer": p + "pre_attention_norm/scale", "post_mixer": p + "post_attention_norm/scale",
+                "pre_ffn": p + "pre_ffw_norm/scale", "post_ffn": p + "post_ffw_norm/scale"}
+
+        return TensorNames("params/transformer/embedder/input_embedding", "params/transformer/output_layer/w",
+                           "params/transformer/final_norm/scale", layer)
+
+    return names
+
+
+#: config.json "weight_layout" -> the bindings of that stored layout
+WEIGHT_LAYOUTS = {"hf": _hf_names, "simply": _simply_names, "gemma_tree": _gemma_tree_names(False),
+                  "gemma_tree_transposed": _gemma_tree_names(True)}
 
 ARCHITECTURES.register("Gemma2ForCausalLM", Gemma2Config)

@@ -6,6 +6,7 @@ the kind that the spec names.
 """
 from __future__ import annotations
 
+import dataclasses
 from typing import Callable, Mapping
 
 import torch
@@ -15,6 +16,7 @@ from ..config.spec import LayerSpec, ModelSpec, PartSpec
 from ..kernels import ops
 from ..parts.base import Block, ParamSpec, Part, PendingNorm
 from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
+from ..weights import binding
 
 
 def _build_layer(spec: LayerSpec) -> Block:
@@ -46,26 +48,48 @@ class DecoderModel:
         out.append((self.head, self.spec.head))
         return out
 
-    def expected_tensors(self) -> dict[str, ParamSpec]:
-        """Tensor name in the model folder -> what is expected of it, in a fixed order."""
-        expected: dict[str, ParamSpec] = {}
+    def tensor_bindings(self) -> list[tuple[Part, str, ParamSpec, "binding.Binding"]]:
+        """For every parameter of every part: (part, the part's name for it, what the part expects, how it is
+        obtained from stored tensors).  A spec that names a plain tensor means that tensor as it is."""
+        out = []
         for part, ps in self._bindings():
             for local, pspec in part.param_specs().items():
                 if local not in ps.tensors:
                     raise ValueError(f"part {ps.kind!r} needs a tensor {local!r} that its spec does not name")
-                name = ps.tensors[local]
-                if name in expected and expected[name].shape != pspec.shape:
-                    raise ValueError(f"tensor {name!r} is used with shapes {expected[name].shape} and {pspec.shape}")
-                expected.setdefault(name, pspec)
+                b = binding.normalize(ps.tensors[local], pspec.shape)
+                try:
+                    got = binding.shape_of(b)
+                except binding.BindingError as e:
+                    raise ValueError(f"part {ps.kind!r}, tensor {local!r}: {e}") from None
+                if tuple(got) != tuple(pspec.shape):
+                    raise ValueError(f"part {ps.kind!r}, tensor {local!r}: the binding gives shape {list(got)}, the "
+                                     f"part expects {list(pspec.shape)}")
+                out.append((part, local, pspec, b))
+        return out
+
+    def expected_tensors(self) -> dict[str, ParamSpec]:
+        """Stored tensor name in the model folder -> what is expected of it (its stored shape; role and random
+        initialisation of the parameter that it feeds), in a fixed order."""
+        expected: dict[str, ParamSpec] = {}
+        for _, _, pspec, b in self.tensor_bindings():
+            for leaf in binding.leaves(b):
+                if leaf.name in expected and expected[leaf.name].shape != leaf.shape:
+                    raise ValueError(f"tensor {leaf.name!r} is used with shapes {expected[leaf.name].shape} and "
+                                     f"{leaf.shape}")
+                expected.setdefault(leaf.name, dataclasses.replace(pspec, shape=leaf.shape))
         return expected
 
     def load_tensors(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        """`tensors`: name in the model folder -> device tensor in its final dtype."""
+        """`tensors`: stored name -> device tensor in its final dtype.  Every part receives its parameters as its
+        spec's bindings make them from these."""
         from ..kernels import packing
 
+        per_part: dict[int, tuple[Part, dict[str, torch.Tensor]]] = {}
+        for part, local, _, b in self.tensor_bindings():
+            per_part.setdefault(id(part), (part, {}))[1][local] = binding.evaluate(b, tensors.__getitem__)
         try:
-            for part, ps in self._bindings():
-                part.load({local: tensors[ps.tensors[local]] for local in part.param_specs()})
+            for part, _ in self._bindings():
+                part.load(per_part.get(id(part), (part, {}))[1])
         finally:
             packing.clear_cache()   # sharing of re-laid tensors (tied table and head) ends with the load
         self.loaded = True

@@ -26,8 +26,6 @@ class PagedAttention(Mixer):
                  position_encoding: PartSpec | None = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"paged_attention: {num_heads} heads do not split over {num_kv_heads} kv heads")
-        if head_dim % 16:
-            raise ValueError(f"paged_attention: head_dim {head_dim} must be a multiple of 16")
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
         self.query_scale = float(query_scale)
         self.soft_cap = float(soft_cap) if soft_cap else None

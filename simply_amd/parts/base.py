@@ -46,22 +46,62 @@ class ParamSpec:
     init: str = "weight"
 
 
+class PagedNeed:
+    """What a mixer that keeps something for every earlier token asks of the cache manager.  The manager only
+    counts pages (a page holds `page_size` consecutive tokens of one request; layers whose needs are equal share
+    one pool, one free list and one block table); what a page holds and how it is laid out is the need's own
+    business.  A need is hashable (a frozen dataclass) and provides
+
+    window                     None: every token is kept; n: only the last n tokens (older pages are given back)
+    page_tensors(num_pages, page_size, dtype, device, fill)
+                               -> {name: tensor}, every tensor with num_pages as its first dimension, filled with
+                               `fill`; one such set is made for every schedule entry that keeps a cache of its own
+    bytes_per_token(esize)     bytes of storage that a token takes in one schedule entry
+
+    Any class with these (a subclass of this one or not) is accepted."""
+
+    window: "int | None" = None
+
+    def page_tensors(self, num_pages: int, page_size: int, dtype: torch.dtype, device, fill: float) -> dict:
+        raise NotImplementedError
+
+    def bytes_per_token(self, esize: int) -> int:
+        raise NotImplementedError
+
+
 @dataclasses.dataclass(frozen=True)
-class PagedKVNeed:
+class PagedKVNeed(PagedNeed):
     """A mixer that keeps keys and values of earlier tokens: per token `num_kv_heads * head_dim`
-    keys and as many values; `window` None keeps all tokens, else only the last `window`."""
+    keys and as many values; `window` None keeps all tokens, else only the last `window`.
+
+    Pages in the layout that the attention kernels read: keys "k" [page, kv head, page_size, head_dim] (inside a
+    page in 16-key x 32-dimension operand blocks when the sizes allow: simply_amd/kernels/packing.py), values "v"
+    transposed [page, kv head, head_dim, page_size], so that the keys of a page are contiguous for each dimension."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
 
+    def page_tensors(self, num_pages, page_size, dtype, device, fill):
+        K, hd = self.num_kv_heads, self.head_dim
+        return {"k": torch.full((num_pages, K, page_size, hd), fill, dtype=dtype, device=device),
+                "v": torch.full((num_pages, K, hd, page_size), fill, dtype=dtype, device=device)}
+
+    def bytes_per_token(self, esize):
+        return 2 * self.num_kv_heads * self.head_dim * esize
+
 
 @dataclasses.dataclass(frozen=True)
 class StateNeed:
-    """A mixer that keeps a state of fixed size per request (zeroed when a request is admitted)."""
+    """A mixer that keeps a state of fixed size per request (zeroed when a request is admitted).  The manager asks
+    `slot_tensor(num_slots, device)` for the storage, one row per request slot; any class with that method is
+    accepted in its place."""
 
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+    def slot_tensor(self, num_slots: int, device) -> torch.Tensor:
+        return torch.zeros((num_slots, *self.shape), dtype=self.dtype, device=device)
 
 
 def as_product_weight(t: torch.Tensor, shared: bool = False, many_rows: bool = False):
@@ -216,7 +256,9 @@ class Mixer(Part):
     #: True if forward() takes defer_sum=True and may then return an `ops.PartialSums`
     defers_sum = False
 
-    def cache_need(self) -> PagedKVNeed | StateNeed | None:
+    def cache_need(self) -> "PagedNeed | StateNeed | None":
+        """What this mixer keeps between steps: a `PagedNeed` (something per token, in pages), a `StateNeed`
+        (something of fixed size per request) or None."""
         return None
 
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:

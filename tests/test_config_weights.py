@@ -189,144 +189,259 @@ def test_element_types():
 
 
 # ------------------------------------------------------------------ which axis goes where
-REFERENCE_TESTDATA = "/root/reference/simply/utils/testdata"
+def reference_testdata() -> str | None:
+    """The reference's test data folder: $SIMPLY_REFERENCE_TESTDATA, else where this build has the reference
+    mounted.  A folder named by the variable must exist (the test fails, it does not skip)."""
+    named = os.environ.get("SIMPLY_REFERENCE_TESTDATA")
+    if named:
+        assert os.path.isdir(named), f"SIMPLY_REFERENCE_TESTDATA names {named!r}, which is no folder"
+        return named
+    default = os.path.join(os.sep, "root", "reference", "simply", "utils", "testdata")
+    return default if os.path.isdir(default) else None
 
 
-def _tree(path):
-    import json
-
-    def arrays(x):
-        if not isinstance(x, dict):
-            return torch.tensor(x, dtype=torch.float64)
-        out = {}
-        for key, v in x.items():          # a key may be a path ("transformer/layer_0/attn")
-            at = out
-            *parents, last = key.split("/")
-            for part in parents:
-                at = at.setdefault(part, {})
-            at[last] = arrays(v)
-        return out
-
+def _stored(path) -> dict:
+    """A fixture tree as the tensors of a folder: name = the path with '/' (as the reference flattens its trees,
+    simply/utils/checkpoint_lib.py:262), the feed-forward biases left out (Gemma 2 has none,
+    simply/config_lib.py:881-882; the fixtures carry them for the optimizer-state rules)."""
     with open(path) as f:
-        return arrays(json.load(f))
+        tree = json.load(f)
+    out = {}
 
+    def walk(x, at):
+        if isinstance(x, dict):
+            for k, v in x.items():
+                walk(v, at + [k])
+        elif at[-1] != "b":
+            out["/".join(at)] = torch.tensor(x, dtype=torch.float64)
 
-def flax_params_to_simply(params: dict) -> dict:
-    """The Gemma parameter tree in the reference's own layout, by the rules of
-    simply/utils/checkpoint_lib.py:256-335 (written out here for the parameters; the reference's test applies the
-    same rules to the optimizer's trees)."""
-    t = params["transformer"]
-    out = {"embed_linear": {"w": t["embedder"]["input_embedding"]}, "final_ln": {"scale": t["final_norm"]["scale"]}}
-    ln = {"pre_attention_norm": "pre_ln_0", "pre_ffw_norm": "pre_ln_1", "post_attention_norm": "post_ln_0",
-          "post_ffw_norm": "post_ln_1"}                                                  # :249-254
-    for name, layer in t.items():
-        if not name.startswith("layer_"):
-            continue
-        qkv = torch.einsum("kndh->kdnh", layer["attn"]["qkv_einsum"]["w"])             # :272-277, then split in three
-        block = {"attn": {"q_proj": {"w": qkv[0]}, "k_proj": {"w": qkv[1]}, "v_proj": {"w": qkv[2]},
-                          "o_proj": {"w": torch.einsum("nhd->dnh", layer["attn"]["attn_vec_einsum"]["w"])}},   # :283-287
-                 "ffn": {"ffn_0_gate": {"w": layer["mlp"]["gating_einsum"]["w"][0], "b": layer["mlp"]["gating_einsum"]["b"][0]},
-                         "ffn_0": {"w": layer["mlp"]["gating_einsum"]["w"][1], "b": layer["mlp"]["gating_einsum"]["b"][1]},
-                         "ffn_1": {"w": layer["mlp"]["linear"]["w"], "b": layer["mlp"]["linear"]["b"]}}}        # :300-323
-        for theirs, ours in ln.items():
-            block[ours] = {"scale": layer[theirs]["scale"]}
-        out["block_" + name[len("layer_"):]] = block
+    walk(tree["params"], ["params"])
     return out
 
 
-def simply_params_to_folder(params: dict) -> dict:
-    """The model folder's tensors ([out_features, in_features], heads flattened head-major) from the reference's
-    layout: the inverse of the rules by which the reference reads such a folder
-    (simply/utils/checkpoint_lib.py:432-458: q/k/v `nhd->dnh` of the rows split into heads, o the columns split into
-    heads, the feed-forward matrices transposed).  The names of the four norms are the folder's Gemma 2 names in the
-    roles that simply/utils/checkpoint_lib.py:249-254 gives their Flax counterparts; no file of the reference names
-    the Gemma 2 folder's norms, so that part of the mapping is not pinned by it."""
-    out = {"model.embed_tokens.weight": params["embed_linear"]["w"], "model.norm.weight": params["final_ln"]["scale"]}
-    norms = {"pre_ln_0": "input_layernorm", "post_ln_0": "post_attention_layernorm",
-             "pre_ln_1": "pre_feedforward_layernorm", "post_ln_1": "post_feedforward_layernorm"}
-    for name, b in params.items():
-        if not name.startswith("block_"):
-            continue
-        p = f"model.layers.{name[len('block_'):]}."
-        for proj in ("q_proj", "k_proj", "v_proj"):
-            w = b["attn"][proj]["w"]                                                     # [d, n, h]
-            out[p + f"self_attn.{proj}.weight"] = torch.einsum("dnh->nhd", w).reshape(-1, w.shape[0])
-        w = b["attn"]["o_proj"]["w"]
-        out[p + "self_attn.o_proj.weight"] = w.reshape(w.shape[0], -1)
-        out[p + "mlp.gate_proj.weight"] = b["ffn"]["ffn_0_gate"]["w"].T
-        out[p + "mlp.up_proj.weight"] = b["ffn"]["ffn_0"]["w"].T
-        out[p + "mlp.down_proj.weight"] = b["ffn"]["ffn_1"]["w"].T
-        for ours, theirs in norms.items():
-            out[p + theirs + ".weight"] = b[ours]["scale"]
+FIXTURE_SIZES = dict(tiny.TINY_A, hidden_size=4, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=2,
+                     head_dim=4, intermediate_size=8, vocab_size=2)
+
+
+def bound_parameters(layout: str, stored: dict) -> dict:
+    """Every part's parameters as the product's binding table of `layout` makes them from `stored`, keyed by the
+    names of the default layout (so that two layouts can be compared)."""
+    from simply_amd.weights import binding
+
+    model = DecoderModel(config_from_dict(dict(FIXTURE_SIZES, weight_layout=layout)).model_spec())
+    names = DecoderModel(config_from_dict(dict(FIXTURE_SIZES, weight_layout="hf")).model_spec())
+    expected = model.expected_tensors()
+    assert set(expected) == set(stored), (sorted(set(expected) ^ set(stored)))
+    for n, spec in expected.items():
+        assert tuple(stored[n].shape) == tuple(spec.shape), n
+    out = {}
+    for (_, local, pspec, b), (_, local_hf, _, b_hf) in zip(model.tensor_bindings(), names.tensor_bindings()):
+        assert local == local_hf
+        t = binding.evaluate(b, stored.__getitem__)
+        assert tuple(t.shape) == tuple(pspec.shape)
+        out[b_hf.name] = t
     return out
 
 
 def test_axis_order_against_the_reference_fixtures():
-    """The reference holds one pair of files that says which axis of a Gemma tensor goes where: arange-filled trees
-    before and after its own conversion (simply/utils/testdata/ckpt_gemma2_format.json ->
-    ckpt_expected_format.json, compared by simply/utils/checkpoint_lib_test.py).  The rules as read here reproduce
-    the second file from the first; the folder layout derived from them names the tensors that the model expects,
-    with its shapes; and the plain implementation's products on that layout equal the reference's einsums on its
-    own (`ihd,...i->...hd`, `ihd,...hd->...i`, `io,...i->...o`: simply/model_lib.py:2047-2068, :671-694), so that a
-    transposed matrix or heads flattened the other way round would show."""
-    if not os.path.isdir(REFERENCE_TESTDATA):
-        pytest.skip("the reference's test data is not mounted")
-    flax = _tree(os.path.join(REFERENCE_TESTDATA, "ckpt_gemma2_format.json"))
-    expected = _tree(os.path.join(REFERENCE_TESTDATA, "ckpt_expected_format.json"))
-    simply = flax_params_to_simply(flax["params"])
-
-    def same(a, b, path=""):
-        if isinstance(b, dict):
-            assert set(a) == set(b), (path, sorted(a), sorted(b))
-            for k in b:
-                same(a[k], b[k], path + "/" + k)
-        else:
-            assert torch.equal(a, b), path
-
-    same(simply, expected["params"])
-    # the folder: names and shapes are the model's (2 layers, width 4, 2 heads of size 4, feed-forward 8, 2 tokens)
-    folder = simply_params_to_folder(simply)
-    d = dict(tiny.TINY_A, hidden_size=4, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=2, head_dim=4,
-             intermediate_size=8, vocab_size=2)
-    # (the engine's attention wants head sizes in steps of 16; names and shapes do not depend on that)
-    import dataclasses
-    spec = config_from_dict(dict(d, head_dim=16)).model_spec()
-    names = set()
-    for layer in spec.layers:
-        names |= set(layer.mixer.tensors.values()) | set(layer.feed_forward.tensors.values())
-        names |= {n.tensors["scale"] for n in layer.norms.values()}
-    names |= {spec.embedding.tensors["table"], spec.final_norm.tensors["scale"]}
-    assert names == set(folder)
+    """The reference holds files that say which axis of a Gemma tensor goes where: arange-filled trees before and
+    after its own conversion (simply/utils/testdata/ckpt_gemma2_format.json and ckpt_gemma2_transpose_format.json ->
+    ckpt_expected_format.json, compared by simply/utils/checkpoint_lib_test.py:87-128).  The product's binding tables
+    (`weight_layout` gemma_tree, gemma_tree_transposed, simply: simply_amd/config/gemma2.py) read all three files to
+    the same parameters; and on those parameters the plain implementation's products equal the reference's einsums
+    on its own layout (`ihd,...i->...hd`, `ihd,...hd->...i`, `io,...i->...o`: simply/model_lib.py:2047-2068,
+    :671-694), so that a transposed matrix or heads flattened the other way round would show."""
+    data = reference_testdata()
+    if data is None:
+        pytest.skip("the reference's test data is not mounted (set SIMPLY_REFERENCE_TESTDATA)")
+    simply = _stored(os.path.join(data, "ckpt_expected_format.json"))
+    folder = bound_parameters("simply", simply)
+    for layout, file in (("gemma_tree", "ckpt_gemma2_format.json"),
+                         ("gemma_tree_transposed", "ckpt_gemma2_transpose_format.json")):
+        other = bound_parameters(layout, _stored(os.path.join(data, file)))
+        assert set(other) == set(folder)
+        for n in folder:
+            assert torch.equal(other[n], folder[n]), (layout, n)
     assert folder["model.layers.0.self_attn.q_proj.weight"].shape == (8, 4)
     assert folder["model.layers.0.self_attn.o_proj.weight"].shape == (4, 8)
     assert folder["model.layers.1.mlp.down_proj.weight"].shape == (4, 8)
-    # the plain implementation on the folder's layout against the reference's einsums on the reference's layout
+    # the plain implementation on the parts' layout against the reference's einsums on the reference's layout
     x = torch.randn(5, 4, dtype=torch.float64, generator=torch.Generator().manual_seed(0))
-    b = simply["block_1"]
+    b = lambda n: simply["params/block_1/" + n]
     p = "model.layers.1."
     for proj in ("q_proj", "k_proj", "v_proj"):
-        want = torch.einsum("ihd,ti->thd", b["attn"][proj]["w"], x)
+        want = torch.einsum("ihd,ti->thd", b(f"attn/{proj}/w"), x)
         got = (x @ folder[p + f"self_attn.{proj}.weight"].T).reshape(5, 2, 4)       # as plain.attention_layer does
         torch.testing.assert_close(got, want)
     heads = torch.randn(5, 2, 4, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
     torch.testing.assert_close(heads.reshape(5, 8) @ folder[p + "self_attn.o_proj.weight"].T,
-                               torch.einsum("ihd,thd->ti", b["attn"]["o_proj"]["w"], heads))
+                               torch.einsum("ihd,thd->ti", b("attn/o_proj/w"), heads))
     import plain_gemma2 as plain
-    gate = torch.einsum("io,ti->to", b["ffn"]["ffn_0_gate"]["w"], x * 1e-3)
-    up = torch.einsum("io,ti->to", b["ffn"]["ffn_0"]["w"], x * 1e-3)
-    want = torch.einsum("io,ti->to", b["ffn"]["ffn_1"]["w"], plain.gelu_tanh(gate) * up)   # simply/model_lib.py:714-730
+    gate = torch.einsum("io,ti->to", b("ffn/ffn_0_gate/w"), x * 1e-3)
+    up = torch.einsum("io,ti->to", b("ffn/ffn_0/w"), x * 1e-3)
+    want = torch.einsum("io,ti->to", b("ffn/ffn_1/w"), plain.gelu_tanh(gate) * up)   # simply/model_lib.py:714-730
     torch.testing.assert_close(plain.feed_forward(x * 1e-3, folder, p + "mlp."), want)
-    # the roles of the norms: the block of the plain implementation with the folder's names equals the block written
-    # with the reference's names in the reference's order (simply/model_lib.py:2669-2703)
-    cfg = dict(d, rms_norm_eps=1e-6, query_pre_attn_scalar=4, attn_logit_softcapping=None, sliding_window=None)
+    # the roles of the norms: the block of the plain implementation with the default layout's names (no file of the
+    # reference names a published Gemma 2 folder's norms, so that part of the default layout is not pinned by it)
+    # equals the block written with the reference's names in the reference's order (simply/model_lib.py:2669-2703)
+    cfg = dict(FIXTURE_SIZES, rms_norm_eps=1e-6, query_pre_attn_scalar=4, attn_logit_softcapping=None, sliding_window=None)
     small = {k: v * 1e-3 for k, v in folder.items()}
     pos = torch.arange(5)
     h = x
-    y = plain.rms_norm(x, small[p + "input_layernorm.weight"], 1e-6)
+    y = plain.rms_norm(x, b("pre_ln_0/scale") * 1e-3, 1e-6)
     y = plain.attention_layer(y, pos, small, p + "self_attn.", cfg, None)
-    y = plain.rms_norm(y, b["post_ln_0"]["scale"] * 1e-3, 1e-6)
+    y = plain.rms_norm(y, b("post_ln_0/scale") * 1e-3, 1e-6)
     x1 = y + h
-    y = plain.rms_norm(x1, b["pre_ln_1"]["scale"] * 1e-3, 1e-6)
+    y = plain.rms_norm(x1, b("pre_ln_1/scale") * 1e-3, 1e-6)
     y = plain.feed_forward(y, small, p + "mlp.")
-    y = plain.rms_norm(y, b["post_ln_1"]["scale"] * 1e-3, 1e-6)
+    y = plain.rms_norm(y, b("post_ln_1/scale") * 1e-3, 1e-6)
     torch.testing.assert_close(plain.block(x, pos, small, 1, cfg, None), y + x1)
+
+
+def test_every_stored_layout_loads_to_the_same_model(tmp_path):
+    """A folder written in each stored layout (the random-weights mode writes the layout's own tensors) loads,
+    and the same parameters stored in two layouts give the same parts: grouped-query sizes, so that the Gemma
+    tree has `q_einsum` and `kv_einsum`."""
+    from simply_amd.weights import binding
+
+    base = dict(tiny.TINY_A)
+    hf_dir = write_random_model(config_from_dict(base), str(tmp_path / "hf"), 3, torch.float32, norm_std=0.1)
+    hf = load_file(os.path.join(hf_dir, "model.safetensors"))
+    want = DecoderModel(config_from_dict(base).model_spec())
+    load_weights(want, hf_dir, torch.float32, "cpu")
+    D, H, K, hd = 64, 4, 2, 16
+    for layout in ("simply", "gemma_tree", "gemma_tree_transposed"):
+        d = write_random_model(config_from_dict(dict(base, weight_layout=layout)), str(tmp_path / layout), 4,
+                               torch.float32, norm_std=0.1)
+        assert load_config(d).weight_layout == layout
+        m = DecoderModel(load_config(d).model_spec())
+        load_weights(m, d, torch.float32, "cpu")          # names and shapes are the layout's own
+        # now the hf folder's parameters, stored in this layout by hand
+        stored = {}
+        for i in range(2):
+            p, q = f"model.layers.{i}.", f"params/block_{i}/"
+            heads = lambda w, n: w.reshape(n, hd, D)      # [n h, d] -> [n, h, d]
+            qw, kw, vw = (heads(hf[p + f"self_attn.{x}_proj.weight"], n) for x, n in (("q", H), ("k", K), ("v", K)))
+            ow = hf[p + "self_attn.o_proj.weight"].reshape(D, H, hd)
+            g, u, dn = (hf[p + f"mlp.{x}_proj.weight"] for x in ("gate", "up", "down"))
+            if layout == "simply":
+                stored.update({q + "attn/q_proj/w": qw.permute(2, 0, 1), q + "attn/k_proj/w": kw.permute(2, 0, 1),
+                               q + "attn/v_proj/w": vw.permute(2, 0, 1), q + "attn/o_proj/w": ow,
+                               q + "ffn/ffn_0_gate/w": g.T, q + "ffn/ffn_0/w": u.T, q + "ffn/ffn_1/w": dn.T})
+                norms = {"pre_ln_0": "input_layernorm", "post_ln_0": "post_attention_layernorm",
+                         "pre_ln_1": "pre_feedforward_layernorm", "post_ln_1": "post_feedforward_layernorm"}
+                stored.update({q + a + "/scale": hf[p + b + ".weight"] for a, b in norms.items()})
+            else:
+                q = f"params/transformer/layer_{i}/"
+                gating = torch.stack([g, u]) if layout.endswith("transposed") else torch.stack([g.T, u.T])
+                stored.update({q + "attn/q_einsum/w": qw.permute(0, 2, 1),
+                               q + "attn/kv_einsum/w": torch.stack([kw.permute(0, 2, 1), vw.permute(0, 2, 1)]),
+                               q + "attn/attn_vec_einsum/w": ow.permute(1, 2, 0),
+                               q + "mlp/gating_einsum/w": gating, q + "mlp/linear/w": dn.T})
+                norms = {"pre_attention_norm": "input_layernorm", "post_attention_norm": "post_attention_layernorm",
+                         "pre_ffw_norm": "pre_feedforward_layernorm", "post_ffw_norm": "post_feedforward_layernorm"}
+                stored.update({q + a + "/scale": hf[p + b + ".weight"] for a, b in norms.items()})
+        if layout == "simply":
+            stored.update({"params/embed_linear/w": hf["model.embed_tokens.weight"],
+                           "params/final_ln/scale": hf["model.norm.weight"]})
+        else:
+            stored.update({"params/transformer/embedder/input_embedding": hf["model.embed_tokens.weight"],
+                           "params/transformer/final_norm/scale": hf["model.norm.weight"]})
+        out = str(tmp_path / (layout + "_same"))
+        os.makedirs(out)
+        save_file({k: v.contiguous() for k, v in stored.items()}, os.path.join(out, "model.safetensors"))
+        with open(os.path.join(out, "config.json"), "w") as f:
+            json.dump(dict(base, weight_layout=layout), f)
+        got = DecoderModel(load_config(out).model_spec())
+        load_weights(got, out, torch.float32, "cpu")
+        for a, b in zip(got.layers, want.layers):
+            assert torch.equal(a.mixer.qkv_proj, b.mixer.qkv_proj) and torch.equal(a.mixer.o_proj, b.mixer.o_proj)
+            assert torch.equal(a.feed_forward.gate_proj, b.feed_forward.gate_proj)
+            assert torch.equal(a.feed_forward.up_proj, b.feed_forward.up_proj)
+            assert torch.equal(a.feed_forward.down_proj, b.feed_forward.down_proj)
+            for n in a.norms:
+                assert torch.equal(a.norms[n].scale, b.norms[n].scale)
+        assert torch.equal(got.embedding.table, want.embedding.table)
+
+
+def test_binding_expressions():
+    from simply_amd.weights import binding as wb
+
+    a, b = wb.stored("a", (6, 4)), wb.stored("b", (2, 4))
+    t = {"a": torch.arange(24.0).reshape(6, 4), "b": -torch.arange(8.0).reshape(2, 4), "c": torch.arange(24.0).reshape(2, 3, 4)}
+    e = wb.concat_rows(wb.split_rows(a, 4, 6), b, wb.split_rows(a, 0, 1))
+    assert wb.shape_of(e) == (5, 4) and [l.name for l in wb.leaves(e)] == ["a", "b", "a"]
+    assert torch.equal(wb.evaluate(e, t.__getitem__), torch.cat([t["a"][4:6], t["b"], t["a"][0:1]]))
+    assert wb.shape_of(wb.transpose(a)) == (4, 6)
+    c = wb.stored("c", (2, 3, 4))
+    assert wb.shape_of(wb.select(c, 1)) == (3, 4)
+    # [n=2, h=3, d=4] -> rows head-major [n h, d]; -> [d, n h]
+    assert torch.equal(wb.evaluate(wb.heads_to_rows(c, "nhd"), t.__getitem__), t["c"].reshape(6, 4))
+    assert torch.equal(wb.evaluate(wb.heads_to_cols(c, "nhd"), t.__getitem__), t["c"].reshape(6, 4).T)
+    assert wb.shape_of(wb.heads_to_rows(c, "dnh")) == (12, 2)
+    for bad, match in ((wb.split_rows(a, 3, 9), "rows 3..9"), (wb.concat_rows(a, wb.stored("x", (2, 5))), "differ"),
+                       (wb.transpose(c), "2 dimensions"), (wb.heads_to_rows(c, "nnd"), "once each"),
+                       (wb.select(c, 2), "entry 2")):
+        with pytest.raises(wb.BindingError, match=match):
+            wb.shape_of(bad)
+    with pytest.raises(ValueError, match="unknown weight transform"):
+        wb.shape_of(wb.Derived("rot13", (a,)))
+    with pytest.raises(wb.BindingError, match="tensor name or an expression"):
+        wb.normalize(3, (1,))
+
+
+def test_a_folder_with_fused_tensors_loads_through_declared_splits(tmp_path):
+    """A toy folder that stores q, k and v as one tensor and gate and up as one: the spec binds the parts'
+    parameters to row ranges of the stored tensors, and nothing in the loader knows of it.  Errors name the
+    stored tensors with their stored shapes."""
+    import dataclasses as dc
+    from simply_amd.config import PartSpec
+    from simply_amd.weights import binding as wb
+
+    cfg = config_from_dict(tiny.TINY_A)
+    spec = cfg.model_spec()
+    D, H, K, hd, F = 64, 4, 2, 16, 128
+    layers = []
+    for i, layer in enumerate(spec.layers):
+        qkv = wb.stored(f"l{i}.qkv", ((H + 2 * K) * hd, D))
+        gu = wb.stored(f"l{i}.gate_up", (2 * F, D))
+        mixer = dc.replace(layer.mixer, tensors={"q_proj": wb.split_rows(qkv, 0, H * hd),
+                                                 "k_proj": wb.split_rows(qkv, H * hd, (H + K) * hd),
+                                                 "v_proj": wb.split_rows(qkv, (H + K) * hd, (H + 2 * K) * hd),
+                                                 "o_proj": layer.mixer.tensors["o_proj"]})
+        ffn = dc.replace(layer.feed_forward, tensors={"gate_proj": wb.split_rows(gu, 0, F), "up_proj": wb.split_rows(gu, F, 2 * F),
+                                                      "down_proj": layer.feed_forward.tensors["down_proj"]})
+        layers.append(dc.replace(layer, mixer=mixer, feed_forward=ffn))
+    fused = dc.replace(spec, layers=tuple(layers))
+    model = DecoderModel(fused)
+    expected = model.expected_tensors()
+    assert expected["l0.qkv"].shape == (128, 64) and expected["l1.gate_up"].shape == (256, 64)
+    assert not any("q_proj" in n or "gate_proj" in n for n in expected)
+    # the same parameters as a folder of separate tensors
+    plain_dir = write_random_model(cfg, str(tmp_path / "sep"), 0, torch.float32, norm_std=0.1)
+    sep = load_file(os.path.join(plain_dir, "model.safetensors"))
+    stored = {n: t for n, t in sep.items() if not any(x in n for x in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj"))}
+    for i in range(2):
+        p = f"model.layers.{i}."
+        stored[f"l{i}.qkv"] = torch.cat([sep[p + f"self_attn.{x}_proj.weight"] for x in "qkv"])
+        stored[f"l{i}.gate_up"] = torch.cat([sep[p + "mlp.gate_proj.weight"], sep[p + "mlp.up_proj.weight"]])
+    out = tmp_path / "fused"
+    out.mkdir()
+    save_file(stored, str(out / "model.safetensors"))
+    load_weights(model, str(out), torch.float32, "cpu")
+    want = DecoderModel(spec)
+    load_weights(want, plain_dir, torch.float32, "cpu")
+    for a, b in zip(model.layers, want.layers):
+        assert torch.equal(a.mixer.qkv_proj, b.mixer.qkv_proj)
+        assert torch.equal(a.feed_forward.gate_proj, b.feed_forward.gate_proj)
+        assert torch.equal(a.feed_forward.up_proj, b.feed_forward.up_proj)
+    # a stored tensor of the wrong shape is reported by its stored name and shapes
+    stored["l1.qkv"] = stored["l1.qkv"][:100]
+    save_file(stored, str(out / "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_weights(DecoderModel(fused), str(out), torch.float32, "cpu")
+    assert e.value.wrong_shape == [("l1.qkv", (100, 64), (128, 64))]
+    # a binding whose result is not what the part expects is refused when the model is asked for its tensors
+    bad = dc.replace(layers[0].mixer, tensors=dict(layers[0].mixer.tensors, q_proj=wb.split_rows(wb.stored("l0.qkv", (128, 64)), 0, 48)))
+    with pytest.raises(ValueError, match=r"q_proj.*gives shape \[48, 64\].*expects \[64, 64\]"):
+        DecoderModel(dc.replace(spec, layers=(dc.replace(layers[0], mixer=bad), layers[1]))).expected_tensors()

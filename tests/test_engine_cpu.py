@@ -45,6 +45,20 @@ def test_cuts_match_plain(tmp_path, cpu_ops, name):
         assert (got - want).abs().max().item() <= 2e-5 * scale, cuts
 
 
+@pytest.mark.parametrize("head_dim", [2, 6, 24, 40])
+def test_head_sizes_that_are_even_but_no_multiple_of_16(tmp_path, cpu_ops, head_dim):
+    """Every even head size that the configuration allows builds and runs (rotary pairs are all that the
+    architecture asks of it: simply/utils/position_encoding.py:83-84)."""
+    d = tiny.write_config_model(tiny.odd_head_size_config(head_dim), str(tmp_path / "m"), seed=head_dim, std=0.3)
+    w, cfg = plain.load(d)
+    tokens = tiny.random_tokens(30, cfg["vocab_size"], 3)
+    want = plain.forward(w, cfg, tokens)
+    ex = make_executor(d)
+    for cuts in ([30], [12] + [1] * 18, [7, 5, 3, 2, 11, 2]):
+        got = run_cut(ex, "r", tokens, cuts)
+        assert (got - want).abs().max().item() <= 2e-5 * want.abs().max().item(), cuts
+
+
 def test_mixed_with_page_reuse(tmp_path, cpu_ops):
     d = tiny.write_model("B", str(tmp_path / "B"), std=0.3)
     w, cfg = plain.load(d)

@@ -168,6 +168,14 @@ def test_random_configurations_mixed(tmp_path, seed):
     mixed_requests_in_a_tight_pool(d, page, lens, seed)
 
 
+@pytest.mark.parametrize("head_dim", [2, 6, 24, 40, 72])
+def test_head_sizes_that_are_even_but_no_multiple_of_16(tmp_path, head_dim):
+    """Every even head size that the configuration allows runs (on the kernels that take every size), in both
+    element types, mixed in a tight pool (simply/utils/position_encoding.py:83-84 asks only for halves)."""
+    d = tiny.write_config_model(tiny.odd_head_size_config(head_dim), str(tmp_path / "m"), seed=head_dim, std=0.2)
+    mixed_requests_in_a_tight_pool(d, 8 if head_dim != 24 else 16, [33, 70, 9, 51], 300 + head_dim)
+
+
 @pytest.mark.parametrize("case", [4, 11, 21, 36, 94, 135, "smallest"])
 def test_configurations_with_the_largest_bfloat16_error(tmp_path, case):
     """The configurations on which bfloat16 logits lie furthest from the float64 ones (tiny.drawn_case): 4 to 9 % of

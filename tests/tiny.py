@@ -54,6 +54,22 @@ def write_model(name: str, out_dir: str, dtype=torch.float32, std: float | None 
     return write_random_model(cfg, out_dir, seed, dtype, std=std, norm_std=norm_std)
 
 
+def write_config_model(d: dict, out_dir: str, seed: int, dtype=torch.float32, std: float | None = None,
+                       norm_std: float = 0.2) -> str:
+    """Writes the configuration `d` (config.json keys) with random weights."""
+    from simply_amd.config import config_from_dict
+    from simply_amd.weights import write_random_model
+
+    return write_random_model(config_from_dict(d), out_dir, seed, dtype, std=std, norm_std=norm_std)
+
+
+def odd_head_size_config(head_dim: int) -> dict:
+    """A tiny configuration whose head size is even but no multiple of 16 (rotary pairs need no more:
+    simply/utils/position_encoding.py:83-84 splits the head in halves)."""
+    return dict(TINY_C, head_dim=head_dim, query_pre_attn_scalar=head_dim, num_hidden_layers=3,
+                layer_types=["sliding_attention", "full_attention", "sliding_attention"], sliding_window=9)
+
+
 def random_tokens(n: int, vocab: int, seed: int) -> list[int]:
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
