@@ -88,26 +88,36 @@ def fill_cache_random(lm, std: float = 0.5, seed: int = 0) -> None:
                     flat[i:i + n] = (torch.randn(n, generator=gen, device=t.device, dtype=torch.float32) * std).to(t.dtype)
 
 
-def preload(lm, request_id, prompt_token_ids, params):
-    """Admits a request as if all of its prompt but the last token had been run, in portions of the engine's token
-    budget: its pages are reserved and given back as that run would have done (a windowed layer ends up holding its
-    window only) and hold what `fill_cache_random` put there, so the next steps are decode steps at the prompt's
-    length."""
-    from simply_amd.engine.scheduler import Status
-    r = lm.add_request(request_id, prompt_token_ids, params)
-    sched, cache = lm.scheduler, lm.executor.cache
-    sched.waiting.remove(r)
-    cache.admit(r.request_id)
-    n = r.num_tokens - 1
-    for at in range(0, n, sched.budget):
-        q = min(sched.budget, n - at)
-        cache.reserve(r.request_id, at, q)
-        cache.mark_issued([(r.request_id, at, q)])
-    lm.executor.num_computed[r.request_id] = (cache.admission[r.request_id], n)
-    r.num_computed = n
-    r.status = Status.RUNNING
-    sched.running.append(r)
-    return r
+def self_check(lm) -> dict:
+    """Outside the timed steps: the next decode step is run twice, once eagerly (no recorded graph; the kernels plan
+    for the real context) and once as the engine runs it (a replay of the recorded step), over the same cache.  The
+    token that the engine's step draws must be the best of the eager step's logits, or within rounding of it
+    (the two steps may cut the keys differently, so their logits differ in the last bits)."""
+    import dataclasses
+    import torch
+    from simply_amd.engine.executor import StepEntry
+
+    ex, reqs = lm.executor, sorted(lm.scheduler.running, key=lambda r: r.arrival)
+    entries = [StepEntry(r.request_id, [r.all_token_ids[-1]], [0], r.num_computed) for r in reqs]
+    config = ex.config
+    ex.config = dataclasses.replace(config, use_graphs=False)
+    try:
+        eager = ex.step(entries).float().clone()
+    finally:
+        ex.config = config
+    before = [len(r.output_token_ids) for r in reqs]
+    lm.step(max_decode_steps=1)
+    drawn = [r.output_token_ids[-1] for r in reqs]
+    assert all(len(r.output_token_ids) == n + 1 for r, n in zip(reqs, before))
+    assert torch.isfinite(eager).all(), "the eager step's logits are not finite"
+    best = eager.max(dim=1).values
+    of_drawn = eager[torch.arange(len(reqs)), torch.tensor(drawn, device=eager.device)]
+    gap = float((best - of_drawn).max())
+    same = int((eager.argmax(dim=1).cpu() == torch.tensor(drawn)).sum())
+    scale = float(eager.abs().max())
+    assert gap <= 1e-2 * scale, f"the engine's step drew tokens that the eager step's logits do not support: gap {gap}"
+    assert len(set(drawn)) > 1 or len(reqs) == 1, "every request drew the same token"
+    return {"same_token": same, "of": len(reqs), "largest_gap": round(gap, 5), "largest_logit": round(scale, 3)}
 
 
 def percentile(values, p):
@@ -116,22 +126,23 @@ def percentile(values, p):
 
 
 def run_decode(model, cfg, batch, context, steps, warmup, page_size, dtype, latency_steps=0):
-    """Returns (seconds per step, mean kv length over the timed steps, latencies): `steps` decode steps as the engine
-    runs them when nobody waits (several in a row on the device), then `latency_steps` more one at a time, the host
-    reading each step's tokens before the next: their seconds are the latencies."""
+    """Returns (seconds per step, mean kv length over the timed steps, latencies, self-check): `steps` decode steps as
+    the engine runs them when nobody waits (several in a row on the device), then one step whose tokens are checked
+    (`self_check`), then `latency_steps` more one at a time, the host reading each step's tokens before the next:
+    their seconds are the latencies."""
     import torch
     from simply_amd.engine.llm import LMInterface
     from simply_amd.sampling import SamplingParams
 
-    max_len = context + steps + warmup + latency_steps + 8
+    max_len = context + steps + warmup + latency_steps + 10
     lm = LMInterface(config=cfg, random_weights=0, activation_dtype=dtype, batch_size=batch, max_seq_len=max_len,
                      page_size=page_size, max_num_issue_tokens=2048, _model=model)
     fill_cache_random(lm)
     g = torch.Generator().manual_seed(1)
-    params = SamplingParams(temperature=0.0, max_decode_steps=steps + warmup + latency_steps + 4, ignore_eos=True)
+    params = SamplingParams(temperature=0.0, max_decode_steps=steps + warmup + latency_steps + 6, ignore_eos=True)
     for i in range(batch):
         prompt = torch.randint(0, cfg.vocab_size, (context,), generator=g).tolist()
-        preload(lm, f"b{i}", prompt, params)
+        lm.adopt_request(f"b{i}", prompt, context - 1, params)
     def decode(k):
         """Exactly k decode steps (the engine runs several in a row on the device where it can)."""
         target = lm.stats["steps"] + k
@@ -147,6 +158,7 @@ def run_decode(model, cfg, batch, context, steps, warmup, page_size, dtype, late
     first = context + warmup          # kv length seen by the first timed step
     mean_kv = first + (steps - 1) / 2
     assert all(len(r.output_token_ids) == warmup + steps for r in lm.scheduler.running)
+    check = self_check(lm)
     latencies = []
     if latency_steps:
         lm.step(max_decode_steps=1)   # the single-step graph is recorded outside the timed steps
@@ -156,7 +168,7 @@ def run_decode(model, cfg, batch, context, steps, warmup, page_size, dtype, late
         latencies = [sec for _, _, sec in lm.step_log]
     del lm
     torch.cuda.empty_cache()
-    return dt, mean_kv, latencies
+    return dt, mean_kv, latencies, check
 
 
 def run_prefill(model, cfg, tokens, reps, page_size, dtype, portion=None):
@@ -300,8 +312,8 @@ def main():
                           "config": {"model": f"gemma2-{args.shape}-shape", "layers": cfg.num_hidden_layers}}), flush=True)
         return
 
-    dt, mean_kv, latencies = run_decode(model, cfg, args.batch, args.context, args.steps, args.warmup, args.page_size,
-                                        args.dtype, latency_steps=args.latency_steps)
+    dt, mean_kv, latencies, check = run_decode(model, cfg, args.batch, args.context, args.steps, args.warmup,
+                                               args.page_size, args.dtype, latency_steps=args.latency_steps)
     step_bytes = weight_bytes(cfg, esize) + args.batch * kv_bytes_per_request(cfg, mean_kv, esize)
     achieved = step_bytes / dt / 1e9
 
@@ -326,7 +338,7 @@ def main():
     if not args.no_points:
         for b in (1, 64):
             steps_b = max(10, min(args.steps, 30))
-            dtb, _, _ = run_decode(model, cfg, b, args.context, steps_b, 8, args.page_size, args.dtype)
+            dtb, _, _, _ = run_decode(model, cfg, b, args.context, steps_b, 8, args.page_size, args.dtype)
             points[f"decode_b{b}"] = round(b / dtb, 1)
 
     out = {
@@ -349,6 +361,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,
+        "self_check": check,
     }
     print(json.dumps(out), flush=True)
 

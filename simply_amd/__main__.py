@@ -51,7 +51,10 @@ def cmd_generate(argv) -> int:
     _flag(ap, "max_decode_steps", type=int, default=256)
     ap.add_argument("--max-tokens", dest="max_decode_steps", type=int)
     _flag(ap, "page_size", type=int, default=16)
-    _flag(ap, "total_num_pages", type=int, default=None)
+    _flag(ap, "total_num_pages", type=int, default=None, help="pages of a cache group that keeps every token")
+    _flag(ap, "windowed_num_pages", type=int, default=None, help="pages of a cache group that keeps a window only")
+    _flag(ap, "memory_fraction", type=float, default=None,
+          help="size the cache pools to this fraction of the free device memory (when --total_num_pages is not given)")
     _flag(ap, "temperature", type=float, default=1.0)
     _flag(ap, "top_k", type=int, default=-1)
     _flag(ap, "top_p", type=float, default=1.0)
@@ -66,7 +69,8 @@ def cmd_generate(argv) -> int:
 
     kw = dict(activation_dtype=args.activation_dtype, batch_size=args.batch_size, max_seq_len=args.max_seq_len,
               page_size=args.page_size, max_num_issue_tokens=args.max_num_issue_tokens,
-              total_num_pages=args.total_num_pages, seed=args.seed, intermediate_steps=args.intermediate_steps)
+              total_num_pages=args.total_num_pages, windowed_num_pages=args.windowed_num_pages,
+              memory_fraction=args.memory_fraction, seed=args.seed, intermediate_steps=args.intermediate_steps)
     if args.ckpt_dir:
         lm = LMInterface(args.ckpt_dir, **kw)
     elif args.config and args.random_weights is not None:

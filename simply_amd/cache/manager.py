@@ -49,6 +49,28 @@ def windowed_pool_pages(window: int, page_size: int, num_slots: int, max_step_to
     return num_slots * (ceil_div(max(window - 1, 0), page_size) + 2) + ceil_div(max_step_tokens, page_size)
 
 
+def pages_for_memory(needs, *, page_size: int, num_slots: int, max_seq_len: int, max_step_tokens: int, esize: int,
+                     budget_bytes: int) -> int:
+    """How many pages a group that keeps every token gets when `budget_bytes` of device memory go to the cache:
+    the windowed groups take what their requests can hold at once, the others share the rest page for page; never
+    more than `num_slots` sequences of `max_seq_len` need, at least one sequence's worth of one page.  `needs` as
+    `CacheManager` takes them."""
+    per_page_full = per_page_windowed_total = 0
+    for need, cache_from in needs:
+        if cache_from is not None or not callable(getattr(need, "page_tensors", None)):
+            continue
+        page_bytes = need.bytes_per_token(esize) * page_size
+        window = getattr(need, "window", None)
+        if window is None:
+            per_page_full += page_bytes
+        else:
+            per_page_windowed_total += page_bytes * windowed_pool_pages(window, page_size, num_slots, max_step_tokens)
+    most = num_slots * ceil_div(max_seq_len, page_size)
+    if per_page_full == 0:
+        return most
+    return int(max(1, min(most, (int(budget_bytes) - per_page_windowed_total) // per_page_full)))
+
+
 class PagePool:
     """Free pages of one group, handed out from the front and taken back at the end
     (simply/utils/ragged_paged_attention.py:495-511, 530-535)."""

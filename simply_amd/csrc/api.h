@@ -102,6 +102,11 @@ int sa_gemm_planes(const void* A, int a_dtype, int64_t lda, const void* W, const
 // epilogue; epilogue codes as for sa_gemm).
 // h_in, h_out: float32 [M, K], different buffers; y: bfloat16 [M, K]; norm weights float32 or bfloat16 [K].
 int sa_gemm_normed_takes(int M, int N, int K);
+// The most rows that sa_gemm_normed takes, and whether it is expected to be faster than the separate norm and
+// product kernels at these sizes (it takes more sizes than it pays for: rows wider than 2560 elements pay only where
+// the kernel has a prologue for exactly that width, and a weight with very many rows is better served by sa_gemm).
+int sa_gemm_normed_max_rows();
+int sa_gemm_normed_pays(int M, int N, int K);
 
 // The fused q/k/v projection with the norms of sa_gemm_normed in front and the rotation, query scale and cache write
 // of sa_rope_cache_write behind: C receives the queries [M, H * hd] (rows of ldc elements), keys and values go into

@@ -467,9 +467,28 @@ static int launch(const bf16* y, const float* h_in, float* h_out, const void* w_
 
 using namespace sa;
 
+extern "C" int sa_gemm_normed_max_rows() { return 16; }
+
 extern "C" int sa_gemm_normed_takes(int M, int N, int K) {
   const size_t lds = static_cast<size_t>(M <= 8 ? 8 : 16) * (K + 8) * 2 + 8 * 2 * 16 * 17 * 4;
-  return M >= 1 && M <= 16 && K % 32 == 0 && K <= 256 * 18 && lds <= 160 * 1024;
+  return M >= 1 && M <= sa_gemm_normed_max_rows() && K % 32 == 0 && K <= 256 * 18 && lds <= 160 * 1024;
+}
+
+// Widths of a whole number of 256-element pieces for which the prologue without per-piece tests is instantiated
+// (SA_NORMED_K and the rotary dispatch below name the same ones).
+static bool has_exact_prologue(int K) {
+  switch (K) {
+    case 2048: case 2304: case 2560: case 3072: case 3584: case 4096: case 4608: return true;
+    default: return false;
+  }
+}
+
+extern "C" int sa_gemm_normed_pays(int M, int N, int K) {
+  // Up to 2560 wide every width gains (8.1 against 13.3 us for q/k/v at one row of 2304).  Wider rows leave the
+  // kernel too few registers to have its first weights on their way during the norms unless the prologue has no
+  // per-piece tests (5 to 25 % faster than the separate kernels at 3584 and 4608, slower without).  Against very many
+  // weight rows (a head over a large vocabulary) the kernels that fill the GPU without the norms in front win.
+  return sa_gemm_normed_takes(M, N, K) && (K <= 2560 || has_exact_prologue(K)) && N <= 16 * 8192;
 }
 
 extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, const void* w_post, int w_post_dtype,
@@ -504,7 +523,9 @@ extern "C" int sa_gemm_normed(const void* y, const float* h_in, float* h_out, co
     if (K == 2048) SA_NORMED_EXACT(EPI, 8);                                                                        \
     if (K == 2304) SA_NORMED_EXACT(EPI, 9);                                                                        \
     if (K == 2560) SA_NORMED_EXACT(EPI, 10);                                                                       \
+    if (K == 3072) SA_NORMED_EXACT(EPI, 12);                                                                       \
     if (K == 3584) SA_NORMED_EXACT(EPI, 14);                                                                       \
+    if (K == 4096) SA_NORMED_EXACT(EPI, 16);                                                                       \
     if (K == 4608) SA_NORMED_EXACT(EPI, 18);                                                                       \
     if (K <= 2560) SA_NORMED(EPI, 10); \
     if (K <= 3584) SA_NORMED(EPI, 14); \
@@ -557,7 +578,9 @@ extern "C" int sa_gemm_normed_rotary(const void* y, const float* h_in, float* h_
   if (K == 2048) SA_ROTARY_EXACT(8);
   if (K == 2304) SA_ROTARY_EXACT(9);
   if (K == 2560) SA_ROTARY_EXACT(10);
+  if (K == 3072) SA_ROTARY_EXACT(12);
   if (K == 3584) SA_ROTARY_EXACT(14);
+  if (K == 4096) SA_ROTARY_EXACT(16);
   if (K == 4608) SA_ROTARY_EXACT(18);
 #undef SA_ROTARY_EXACT
   if (K <= 2560) SA_ROTARY(10);

@@ -14,7 +14,7 @@ from typing import Hashable, Sequence
 import numpy as np
 import torch
 
-from ..cache import CacheManager
+from ..cache import CacheManager, pages_for_memory
 from ..config import EngineConfig
 from ..models import DecoderModel
 from .context import GroupStep, StepContext
@@ -36,13 +36,27 @@ class Executor:
         self.model, self.config = model, config
         self.device = torch.device(config.device)
         self.dtype = config.dtype
+        needs = model.cache_needs()
         pages = num_pages if num_pages is not None else config.total_num_pages
+        if pages is None and config.memory_fraction is not None and self.device.type == "cuda":
+            # what is free now, the weights being loaded; the kernels' workspace and a step's buffers come off first
+            from ..kernels import ops
+
+            free, _ = torch.cuda.mem_get_info(self.device)
+            reserve = ops.WORKSPACE_BYTES + 8 * config.batch_size * model.spec.vocab_size + (256 << 20)
+            pages = pages_for_memory(needs, page_size=config.page_size, num_slots=config.batch_size,
+                                     max_seq_len=config.max_seq_len, max_step_tokens=config.max_step_tokens,
+                                     esize=torch.empty((), dtype=self.dtype).element_size(),
+                                     budget_bytes=int(free * config.memory_fraction) - reserve)
         if pages is None:
             pages = config.batch_size * -(-config.max_seq_len // config.page_size)
-        self.cache = CacheManager(model.cache_needs(), page_size=config.page_size, num_pages=pages,
+        windowed = config.windowed_num_pages
+        self.cache = CacheManager(needs, page_size=config.page_size, num_pages=pages,
                                   num_slots=config.batch_size, max_seq_len=config.max_seq_len, dtype=self.dtype,
                                   device=self.device, poison=config.poison_freed_pages,
-                                  max_step_tokens=max(config.issue_budget, config.batch_size))
+                                  max_step_tokens=config.max_step_tokens,
+                                  group_pages=None if windowed is None else
+                                  (lambda need, n: windowed if getattr(need, "window", None) is not None else n))
         self.num_computed: dict[Hashable, tuple[int, int]] = {}  # request -> (admission, tokens run)
         self.vocab_size = model.spec.vocab_size
         # one pinned staging buffer and one device buffer for all of a step's integers
@@ -79,6 +93,13 @@ class Executor:
 
     def finish_request(self, rid: Hashable) -> None:
         self.cache.free(rid)
+
+    def adopt(self, rid: Hashable, num_computed: int) -> None:
+        """Records that the cache already holds the keys of the request's first `num_computed` tokens (the request
+        is admitted and its pages are reserved: `Scheduler.adopt`); its next portion may start there."""
+        if rid not in self.cache.requests:
+            raise KeyError(f"request {rid!r} has not been admitted to the cache")
+        self.num_computed[rid] = (self.cache.admission[rid], int(num_computed))
 
     def has_request(self, rid: Hashable) -> bool:
         return rid in self.cache.requests

@@ -53,15 +53,11 @@ class LMInterface:
     def __init__(self, model: str | None = None, *, config=None, random_weights: int | None = None,
                  activation_dtype: str = "bfloat16", batch_size: int = 8, max_seq_len: int | None = None,
                  page_size: int = 16, max_num_issue_tokens: int = 2048, total_num_pages: int | None = None,
-                 seed: int = 0, device: str = "cuda:0", poison_freed_pages: bool = False, use_graphs: bool = True,
-                 library_gemm_min_rows: int | None = None, intermediate_steps: int = 64, _model=None):
+                 windowed_num_pages: int | None = None, memory_fraction: float | None = None, seed: int = 0, device: str = "cuda:0", poison_freed_pages: bool = False, use_graphs: bool = True,
+                 intermediate_steps: int = 64, _model=None):
         from ..kernels import lib
 
         lib.load()  # fails here, loudly, if the kernel library is missing and cannot be built
-        if library_gemm_min_rows is not None:  # before the weights are laid out: they keep a second form for it
-            from ..kernels import ops
-
-            ops.set_library_gemm_min_rows(library_gemm_min_rows)
         dtype = EngineConfig(activation_dtype=activation_dtype).dtype
         if _model is not None:       # a model that is already on the device (several engines over one set of weights)
             self.model, self.model_config = _model, config
@@ -76,7 +72,9 @@ class LMInterface:
             max_seq_len = self.model.spec.max_position
         self.engine_config = EngineConfig(
             activation_dtype=activation_dtype, page_size=page_size, batch_size=batch_size, max_seq_len=max_seq_len,
-            max_num_issue_tokens=max_num_issue_tokens, total_num_pages=total_num_pages, device=device,
+            max_num_issue_tokens=max_num_issue_tokens, total_num_pages=total_num_pages,
+            windowed_num_pages=windowed_num_pages, memory_fraction=memory_fraction,
+            intermediate_steps=max(1, int(intermediate_steps)), device=device,
             poison_freed_pages=poison_freed_pages, use_graphs=use_graphs)
         self.executor = Executor(self.model, self.engine_config)
         self.scheduler = Scheduler(self.executor.cache, max_num_issue_tokens=self.engine_config.issue_budget,
@@ -95,7 +93,23 @@ class LMInterface:
         self.step_log: list[tuple[int, int, float]] | None = None
 
     # ------------------------------------------------------------------ requests
+    def adopt_request(self, request_id, prompt_token_ids: Sequence[int], num_computed: int,
+                      params: SamplingParams | None = None) -> Request:
+        """A request whose first `num_computed` tokens are taken as run already: the cache's pages are reserved as
+        that run would have left them and hold whatever the caller has put there.  For measurements of decode steps
+        over a long context without the prompts that would have written it; what is generated then depends on what
+        the pages hold."""
+        r = self._new_request(request_id, prompt_token_ids, params)
+        self.scheduler.adopt(r, num_computed)
+        self.executor.adopt(r.request_id, num_computed)
+        return r
+
     def add_request(self, request_id, prompt_token_ids: Sequence[int], params: SamplingParams | None = None) -> Request:
+        r = self._new_request(request_id, prompt_token_ids, params)
+        self.scheduler.add(r)
+        return r
+
+    def _new_request(self, request_id, prompt_token_ids: Sequence[int], params: SamplingParams | None) -> Request:
         params = params or SamplingParams()
         seed = params.seed if params.seed is not None else request_seed(self.seed, self._num_requests)
         self._num_requests += 1
@@ -103,9 +117,7 @@ class LMInterface:
         ids = [int(t) for t in prompt_token_ids]
         if any(t < 0 or t >= vocab for t in ids):
             raise ValueError(f"request {request_id!r}: token id outside [0, {vocab})")
-        r = Request(request_id, ids, params, seed=seed, eos_ids=tuple(self.model.spec.eos_token_ids))
-        self.scheduler.add(r)
-        return r
+        return Request(request_id, ids, params, seed=seed, eos_ids=tuple(self.model.spec.eos_token_ids))
 
     def step(self, max_decode_steps: int | None = None) -> list[Request]:
         """One scheduling decision and one run of the step function; when every scheduled request is decoding and

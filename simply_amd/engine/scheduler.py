@@ -120,6 +120,37 @@ class Scheduler:
         request.status = Status.WAITING
         self.waiting.append(request)
 
+    def adopt(self, request: Request, num_computed: int) -> None:
+        """Takes over a request whose first `num_computed` tokens already have their keys in the cache (written by
+        the caller, for instance a benchmark that fills the pages instead of running a long prompt): the request is
+        admitted and its pages are reserved and given back exactly as if those tokens had run in portions of the
+        token budget, one request at a time, so a windowed group ends up holding its window only.  The request goes
+        on from there like any running request.  Raises `OutOfPages` (and leaves nothing behind) if it does not fit."""
+        if not request.prompt_token_ids:
+            raise ValueError(f"request {request.request_id!r} has an empty prompt")
+        request.params.validate()
+        n = int(num_computed)
+        if not 0 <= n < request.num_tokens:
+            raise ValueError(f"request {request.request_id!r}: {n} computed tokens of {request.num_tokens}")
+        if request.num_tokens >= self._limit(request):
+            raise ValueError(f"request {request.request_id!r}: {request.num_tokens} tokens leave no room to generate "
+                             f"under max_seq_len {self._limit(request)}")
+        cache, rid = self.cache, request.request_id
+        cache.admit(rid)
+        try:
+            for at in range(0, n, self.budget):
+                q = min(self.budget, n - at)
+                cache.reserve(rid, at, q)
+                cache.mark_issued([(rid, at, q)])
+        except Exception:
+            cache.free(rid)
+            raise
+        request.arrival = self._arrivals
+        self._arrivals += 1
+        request.num_computed = n
+        request.status = Status.RUNNING
+        self.running.append(request)
+
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 

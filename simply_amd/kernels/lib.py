@@ -44,6 +44,8 @@ _SIGNATURES = {
                                    _P],
     "sa_gemm_normed": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _I, _I, _F, _P],
     "sa_gemm_normed_takes": [_I, _I, _I],
+    "sa_gemm_normed_pays": [_I, _I, _I],
+    "sa_gemm_normed_max_rows": [],
     "sa_paged_attention_prefill_group": [],
     "sa_paged_attention_decode_takes": [_I, _I, _I, _I, _I, _L, _P],
     "sa_gemm_normed_rotary": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _P, _P, _F, _F, _P, _P,

@@ -113,17 +113,29 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, plus_one: bool, o
 
 class PartialSums:
     """A matrix product whose cuts of K have not been added up yet (`gemm(..., defer_sum=True)`): `planes`
-    [cuts, M, N] float32 in the kernels' workspace, valid until the next kernel that uses the workspace, and `out`,
-    the tensor that the sum belongs in.  `add_rmsnorm` takes it in place of y and adds the planes up itself, which
-    saves the sum kernel and its round trip; anyone else calls `materialize()`."""
+    [cuts, M, N] float32 in the kernels' workspace, valid until the next kernel that is handed the workspace, and
+    `out`, the tensor that the sum belongs in.  `add_rmsnorm` takes it in place of y and adds the planes up itself,
+    which saves the sum kernel and its round trip; anyone else calls `materialize()`.  The planes remember how
+    often the workspace had been handed out when they were written: whoever reads them after another kernel has
+    been given the workspace is refused (`check_fresh`), instead of adding up someone else's partial results."""
 
     def __init__(self, planes: torch.Tensor, out: torch.Tensor):
         self.planes, self.out = planes, out
         self.shape, self.dtype, self.device = out.shape, out.dtype, out.device
+        self._written_at = workspace_uses(out.device)
+
+    def check_fresh(self) -> None:
+        if self.planes is not None and workspace_uses(self.device) != self._written_at:
+            raise KernelError(
+                "partial sums of a matrix product were read after another kernel had been given the workspace that "
+                "holds them: add them up (add_rmsnorm, rope_cache_write or materialize()) before anything else "
+                "that uses the workspace runs (a product with K cut over workgroups, attention over key ranges, "
+                "the sampler)")
 
     def materialize(self) -> torch.Tensor:
         """The product itself: the sum kernel, now."""
         if self.planes is not None:
+            self.check_fresh()
             count, M, N = self.planes.shape
             _lib.call("sa_sum_planes", _ptr(self.planes), count, _ptr(self.out), _code(self.out), self.out.stride(0), M, N,
                       _stream())
@@ -142,6 +154,7 @@ def add_rmsnorm(y: "torch.Tensor | PartialSums", residual: torch.Tensor, *, post
         fits = (y.planes is not None and D % 4 == 0 and D <= 5120 and y.dtype == torch.bfloat16
                 and tuple(y.shape) == (T, D) and all(w is None or w.data_ptr() % 16 == 0 for w in (post_weight, next_weight)))
         if fits:
+            y.check_fresh()
             planes, y = y.planes, y.out   # (y stands for shape and type below; it is not read)
         else:
             y = y.materialize()
@@ -195,6 +208,7 @@ def rope_cache_write(qkv: "torch.Tensor | PartialSums", positions: torch.Tensor,
     planes = None
     if isinstance(qkv, PartialSums):
         if qkv.planes is not None and qkv.shape[0] <= 256 and qkv.dtype == torch.bfloat16:
+            qkv.check_fresh()
             planes, qkv = qkv.planes, qkv.out
         else:
             qkv = qkv.materialize()
@@ -327,28 +341,23 @@ def _gated(activation: int) -> int:
 #: device, allocated at first use; kernels on one stream use it one after the other
 WORKSPACE_BYTES = 256 << 20
 _scratch: dict = {}
+_scratch_uses: dict = {}
 
 
 def _workspace(device) -> torch.Tensor:
+    """The device's workspace, for a kernel that is about to be launched with it: what an earlier kernel left there
+    is lost from now on (`workspace_uses` counts these hand-outs)."""
     key = (device.type, device.index)
     if key not in _scratch:
         _scratch[key] = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    _scratch_uses[key] = _scratch_uses.get(key, 0) + 1
     return _scratch[key]
 
 
-# Plain products (no epilogue) of at least this many rows go to the library (hipBLASLt through torch.matmul) when
-# the weight has kept its row-major form; 0 (the default): never, everything runs on this package's kernels.  Set
-# before the weights are loaded: they keep the second form only while this is on.
-_library_gemm_min_rows = 0
-
-
-def set_library_gemm_min_rows(rows: int) -> None:
-    global _library_gemm_min_rows
-    _library_gemm_min_rows = max(0, int(rows))
-
-
-def library_gemm_min_rows() -> int:
-    return _library_gemm_min_rows
+def workspace_uses(device) -> int:
+    """How often the device's workspace has been handed to a kernel."""
+    device = torch.device(device)
+    return _scratch_uses.get((device.type, device.index), 0)
 
 
 def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
@@ -393,10 +402,6 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
     if tuple(out.shape) != (M, N):
         raise KernelError("gemm: bad output shape")
     ldc = _rows(out, "gemm: out")
-    if (algo == ALGO_AUTO and packed and w.row_major is not None and epi == EPILOGUE_NONE and out.dtype == a.dtype
-            and 0 < _library_gemm_min_rows <= M and not torch.cuda.is_current_stream_capturing()):
-        # (not while a graph is recorded: the library may allocate a workspace)
-        return torch.matmul(a, w.row_major.t(), out=out)
     ws = _workspace(a.device)
     if defer_sum and epi == EPILOGUE_NONE and out.dtype == torch.bfloat16 and out.is_contiguous():
         count = ctypes.c_int(1)
@@ -416,6 +421,25 @@ def gemm_normed_takes(M: int, w) -> bool:
     if not isinstance(w, TiledWeight) or not w.data.is_cuda:
         return False
     return bool(_lib.load().sa_gemm_normed_takes(int(M), int(w.rows), int(w.cols)))
+
+
+def gemm_normed_pays(M: int, w) -> bool:
+    """Whether `gemm_normed` takes M rows against the weight `w` and is expected to beat the separate norm and
+    product kernels there (the library's own answer: it knows for which widths it has which prologue)."""
+    if not isinstance(w, TiledWeight) or not w.data.is_cuda:
+        return False
+    return bool(_lib.load().sa_gemm_normed_pays(int(M), int(w.rows), int(w.cols)))
+
+
+_few_rows: int | None = None
+
+
+def few_rows_limit() -> int:
+    """The most rows of a step for which the kernels that fuse the norms into the following product exist."""
+    global _few_rows
+    if _few_rows is None:
+        _few_rows = int(_lib.load().sa_gemm_normed_max_rows())
+    return _few_rows
 
 
 def gemm_normed(y: torch.Tensor | None, h_in: torch.Tensor, h_out: torch.Tensor | None, w: TiledWeight, *,

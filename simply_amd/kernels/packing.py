@@ -19,7 +19,6 @@ class TiledWeight:
     rows: int            # N
     cols: int            # K
     paired: bool = False  # two matrices [N, K], their 16-row tiles in turn (gate, factor, gate, factor, ...)
-    row_major: torch.Tensor | None = None  # the same matrix [N, K] as it was, for the library product of many rows
 
     @property
     def shape(self) -> tuple[int, int]:

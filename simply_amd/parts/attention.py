@@ -44,8 +44,8 @@ class PagedAttention(Mixer):
         # one product for q, k and v: rows [q heads | k heads | v heads]
         device = tensors["o_proj"].device
         self.qkv_proj = as_product_weight(torch.cat([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]], dim=0)
-                                          .contiguous(), many_rows=True)
-        self.o_proj = as_product_weight(tensors["o_proj"], many_rows=True)
+                                          .contiguous())
+        self.o_proj = as_product_weight(tensors["o_proj"])
         if self.position_encoding is not None and hasattr(self.position_encoding, "to_device"):
             self.position_encoding.to_device(device)
 

@@ -104,22 +104,14 @@ class StateNeed:
         return torch.zeros((num_slots, *self.shape), dtype=self.dtype, device=device)
 
 
-def as_product_weight(t: torch.Tensor, shared: bool = False, many_rows: bool = False):
+def as_product_weight(t: torch.Tensor, shared: bool = False):
     """A matrix in the form that the matrix-product kernels read fastest: bfloat16 matrices on the GPU are
     re-laid in tiles (simply_amd/kernels/packing.py), anything else stays row-major.  `shared`: parts that are
-    handed the same tensor during one load (a tied table and head) get the same re-laid copy.  `many_rows`: the
-    weight of a plain product that portions of prompts go through; it also keeps its row-major form when the
-    library product for many rows is switched on (ops.set_library_gemm_min_rows), which reads that form."""
-    import dataclasses as dc
-
-    from ..kernels import ops
+    handed the same tensor during one load (a tied table and head) get the same re-laid copy."""
     from ..kernels.packing import pack_tiles
 
     if t.dtype == torch.bfloat16 and t.is_cuda and t.dim() == 2:
-        tiled = pack_tiles(t, cached=shared)
-        if many_rows and ops.library_gemm_min_rows() > 0:
-            tiled = dc.replace(tiled, row_major=t.contiguous())
-        return tiled
+        return pack_tiles(t, cached=shared)
     return t
 
 
@@ -159,10 +151,10 @@ class PendingNorm:
 
 
 def pending_fits_product(x, w) -> bool:
-    """Whether the product kernel with the norms in front takes the pending norm `x` against the weight `w`
-    (bfloat16, up to 16 rows, a tiled weight of rows up to 2560 wide, or 3584 or 4608, RMSNorms with bfloat16 scales)."""
+    """Whether the product kernel with the norms in front should take the pending norm `x` against the weight `w`:
+    bfloat16 rows, RMSNorms with bfloat16 scales, and sizes for which the kernel library says that its fused
+    kernel takes them and pays (`ops.gemm_normed_pays`)."""
     from ..kernels import ops
-    from ..kernels.packing import TiledWeight
 
     if not isinstance(x, PendingNorm):
         return False
@@ -170,13 +162,7 @@ def pending_fits_product(x, w) -> bool:
     return (x.dtype == torch.bfloat16 and nn is not None and getattr(nn, "fusable_rms", False)
             and nn.scale.dtype == torch.bfloat16
             and (x.y is None or pn is None or (getattr(pn, "fusable_rms", False) and pn.scale.dtype == torch.bfloat16))
-            and isinstance(w, TiledWeight) and w.rows <= 16 * 8192   # (not the head over a large vocabulary)
-            # up to 2560 wide, and 3584 and 4608 (whole numbers of 256-element pieces, for which the kernel has a
-            # prologue without per-piece tests: 5 to 25 % faster than the separate kernels at the 9B and 27B sizes).
-            # Other widths above 2560 leave the kernel too few registers to have its first weights on their way
-            # during the norms
-            and (w.cols <= 2560 or w.cols in (3584, 4608))
-            and ops.gemm_normed_takes(x.residual.shape[0], w)
+            and ops.gemm_normed_pays(x.residual.shape[0], w)
             and (x.y is None or (x.y.dtype == torch.bfloat16 and x.y.is_contiguous())))
 
 

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import ops
 from ..registry import BLOCKS
 from .base import Block, PendingNorm
 
@@ -28,7 +29,7 @@ class SandwichBlock(Block):
 
     def forward(self, h, ctx, cache, normed, next_norm):
         n = self.norms
-        if ctx.dtype == torch.bfloat16 and ctx.num_tokens <= 16:
+        if ctx.dtype == torch.bfloat16 and ctx.positions.is_cuda and ctx.num_tokens <= ops.few_rows_limit():
             return self._forward_few_rows(h, ctx, cache, normed, next_norm)
         if isinstance(normed, PendingNorm):
             normed, h = normed.materialize(), normed.residual

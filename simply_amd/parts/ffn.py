@@ -39,7 +39,7 @@ class GatedDense(FeedForward):
             self.gate_up, self.gate_proj, self.up_proj = pack_gate_up(gate, up), None, None
         else:
             self.gate_up, self.gate_proj, self.up_proj = None, gate, up
-        self.down_proj = as_product_weight(tensors["down_proj"], many_rows=True)
+        self.down_proj = as_product_weight(tensors["down_proj"])
 
     def forward(self, x: torch.Tensor, ctx=None, defer_sum=False) -> torch.Tensor:
         # gelu(x.Wg^T) * (x.Wu^T), one kernel

@@ -51,9 +51,10 @@ class Reference:
             return FP32_TOL
         return MAX_FACTOR * (self.rounded - self.want).abs().max().item() / self.scale
 
-    def check(self, got: torch.Tensor, rows=None, what="") -> float:
+    def check(self, got: torch.Tensor, rows=None, what="", rms: bool = True) -> float:
         """Asserts that `got` (logits at `rows` of the sequence, all rows if None) is within the bound.
-        Returns the largest difference as a fraction of the largest logit."""
+        Returns the largest difference as a fraction of the largest logit.  rms=False: the largest error only (the
+        caller pools the squared errors of several requests in a `Pooled` and checks their RMS together)."""
         got = got.double().cpu()
         assert torch.isfinite(got).all(), (what, "not finite")
         want = self.want if rows is None else self.want[rows]
@@ -61,13 +62,43 @@ class Reference:
         diff = got - want
         err = diff.abs().max().item() / self.scale
         assert err <= self.max_bound(), (what, "largest error", err, "bound", self.max_bound())
-        if self.dtype != "float32" and diff.shape[0] >= RMS_MIN_ROWS and diff.numel() >= RMS_MIN_VALUES:
+        if rms and self.dtype != "float32" and diff.shape[0] >= RMS_MIN_ROWS and diff.numel() >= RMS_MIN_VALUES:
             rounded = self.rounded if rows is None else self.rounded[rows]
             rms = diff.pow(2).mean().sqrt().item()
             rms_ref = (rounded - want).pow(2).mean().sqrt().item()
             assert rms <= RMS_FACTOR * rms_ref, (what, "rms error", rms / self.scale, "rounded plain run",
                                                  rms_ref / self.scale)
         return err
+
+
+class Pooled:
+    """The RMS criterion over many short comparisons of one model (single decode steps, a few rows per request):
+    each `add` contributes its squared errors, the engine's and the rounded plain run's, and `check` compares the
+    two sums once enough rows and values have come together.  A step's rows alone are too few for the ratio of two
+    samples of rounding noise to mean anything; pooled over the requests of a test they are not."""
+
+    def __init__(self):
+        self.engine = self.rounded = 0.0
+        self.rows = self.values = 0
+        self.scale = 0.0
+
+    def add(self, ref: Reference, got: torch.Tensor, rows=None) -> None:
+        if ref.dtype == "float32":
+            return
+        got = got.double().cpu()
+        want = ref.want if rows is None else ref.want[rows]
+        rounded = ref.rounded if rows is None else ref.rounded[rows]
+        self.engine += (got - want).pow(2).sum().item()
+        self.rounded += (rounded - want).pow(2).sum().item()
+        self.rows += want.shape[0]
+        self.values += want.numel()
+        self.scale = max(self.scale, ref.scale)
+
+    def check(self, what="") -> None:
+        if self.rows >= RMS_MIN_ROWS and self.values >= RMS_MIN_VALUES:
+            rms, rms_ref = (self.engine / self.values) ** 0.5, (self.rounded / self.values) ** 0.5
+            assert rms <= RMS_FACTOR * rms_ref, (what, "pooled rms error", rms / self.scale, "rounded plain run",
+                                                 rms_ref / self.scale, "rows", self.rows)
 
 
 def reference(weights: dict, cfg: dict, tokens, dtype: str, device=None, rows=None) -> Reference:

@@ -106,3 +106,108 @@ def test_mixed_with_page_reuse(tmp_path, cpu_ops):
         g = torch.cat(got[r])
         assert (g - want[r]).abs().max().item() <= 2e-5 * want[r].abs().max().item(), r
     assert all(g.pool.num_free == 28 for g in ex.cache.groups)
+
+
+def test_a_mixer_with_pages_of_its_own_layout(cpu_ops):
+    """A toy mixer (tests/toy_parts.py) that keeps one latent vector per token in pages [page, rank, page_size] of
+    float32: its need is a class of the test's own, the cache manager forms groups for it (one windowed, one that
+    keeps everything), counts their pages and poisons what is given back, and knows nothing of the layout.  Whole,
+    cut, and mixed with page reuse give the same logits; the mixer alone equals its whole-sequence formula."""
+    import toy_parts
+    from simply_amd import registry
+    from simply_amd.models import DecoderModel
+    from simply_amd.weights import init_random
+
+    registry.MIXERS.register("toy_latent_mean", toy_parts.LatentMeanMixer)
+    try:
+        model = DecoderModel(toy_parts.latent_model_spec())
+        init_random(model, 0, torch.float32, torch.device("cpu"), std=0.2)
+        cfg = EngineConfig(activation_dtype="float32", page_size=4, batch_size=3, max_seq_len=64, max_num_issue_tokens=32,
+                           total_num_pages=24, device="cpu", use_graphs=False, poison_freed_pages=True, intermediate_steps=1)
+        ex = Executor(model, cfg)
+        assert len(ex.cache.groups) == 3
+        assert [type(g.need).__name__ for g in ex.cache.groups] == ["PagedKVNeed", "LatentNeed", "LatentNeed"]
+        assert [g.window for g in ex.cache.groups] == [7, 6, None]
+        lat = ex.cache.views[1]
+        assert list(lat.pages) == ["latent"] and lat.pages["latent"].shape == (ex.cache.groups[1].pool.num_pages, 12, 4)
+        assert lat.k_pages is None and ex.cache.bytes_per_token() == 2 * 2 * 16 * 4 + 48 + 48
+        assert ex.cache.groups[1].pool.num_pages == 20 and ex.cache.groups[2].pool.num_pages == 24   # a window's worth only
+        reqs = {f"r{i}": tiny.random_tokens(n, 128, 40 + i) for i, n in enumerate((30, 17, 26, 9, 22))}
+        whole = {}
+        for r, t in reqs.items():
+            whole[r] = run_cut(ex, r, t, [len(t)])
+            assert torch.isfinite(whole[r]).all() and whole[r].abs().max() > 0
+        torch.testing.assert_close(run_cut(ex, "x", reqs["r0"], [7, 2, 9, 1, 11]), whole["r0"], rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(run_cut(ex, "y", reqs["r2"], [1] * 26), whole["r2"], rtol=1e-4, atol=1e-4)
+        # mixed, three live at a time in 24 pages of 4 (29 pages' worth in all): pages are used again, poisoned in between
+        pending, live, got = list(reqs), {}, {r: [] for r in reqs}
+        rng = np.random.default_rng(1)
+        while pending or live:
+            while pending and len(live) < 3 and sum(-(-len(reqs[r]) // 4) for r in live) + -(-len(reqs[pending[0]]) // 4) <= 24:
+                live[pending[0]] = 0
+                ex.add_request(pending.pop(0))
+            entries = []
+            for r in list(live):
+                n = min(len(reqs[r]) - live[r], int(rng.integers(1, 8)))
+                entries.append(StepEntry(r, reqs[r][live[r]:live[r] + n], list(range(n))))
+            logits, i = ex.step(entries), 0
+            for e in entries:
+                n = len(e.tokens)
+                got[e.request_id].append(logits[i:i + n])
+                i += n
+                live[e.request_id] += n
+                if live[e.request_id] == len(reqs[e.request_id]):
+                    ex.finish_request(e.request_id)
+                    del live[e.request_id]
+            ex.cache.check()
+        for r in reqs:
+            torch.testing.assert_close(torch.cat(got[r]), whole[r], rtol=1e-4, atol=1e-4)
+        assert all(g.pool.num_free == g.pool.num_pages for g in ex.cache.groups)
+        # the mixer alone against its formula over the whole sequence
+        mixer = model.layers[1].mixer
+        x = torch.randn(19, 64, generator=torch.Generator().manual_seed(3))
+        ex.add_request("m")
+        ex.cache.reserve("m", 0, 19)
+        from simply_amd.engine.context import GroupStep, StepContext
+        tables = ex.cache.sync_tables()
+        slot = ex.cache.slot_of("m")
+        groups = {g.group_id: GroupStep(tables[g.group_id], torch.from_numpy(ex.cache.slot_mapping(g.group_id, "m", 0, 19)))
+                  for g in ex.cache.groups}
+        ctx = StepContext(dtype=torch.float32, num_tokens=19, positions=torch.arange(19, dtype=torch.int32),
+                          token_seq=torch.full((19,), slot, dtype=torch.int32),
+                          seq_meta=torch.tensor([[slot, 0, 19, 0]], dtype=torch.int32), groups=groups, request_ids=["m"],
+                          seq_slots=[slot], seq_starts=[0], q_lens=[19], cu_q_lens=[0, 19])
+        want = toy_parts.latent_mean_reference(x, mixer.w_in, mixer.w_out, 6)
+        torch.testing.assert_close(mixer.forward(x, ctx, ex.cache.views[1]).double(), want, rtol=1e-5, atol=1e-6)
+    finally:
+        registry.MIXERS.unregister("toy_latent_mean")
+
+
+def test_an_unknown_kind_of_need_is_refused_with_what_it_lacks():
+    from simply_amd.cache import CacheError, CacheManager
+
+    class Odd:
+        pass
+
+    with pytest.raises(CacheError, match="neither page_tensors.*nor slot_tensor"):
+        CacheManager([(Odd(), None)], page_size=4, num_pages=4, num_slots=1, max_seq_len=16)
+
+
+def test_partial_sums_are_refused_once_the_workspace_has_been_handed_on():
+    """The cuts of a product lie in the one workspace that every kernel with scratch memory shares: reading them
+    after another kernel has been given the workspace is an error, not a wrong sum."""
+    from simply_amd.kernels import ops
+
+    cpu = torch.device("cpu")
+    out = torch.empty(2, 4, dtype=torch.bfloat16)
+    ps = ops.PartialSums(torch.zeros(3, 2, 4), out)
+    ps.check_fresh()
+    ops._workspace(cpu)                   # (as the next kernel with scratch memory would)
+    with pytest.raises(ops.KernelError, match="after another kernel had been given the workspace"):
+        ps.materialize()
+    with pytest.raises(ops.KernelError, match="workspace"):
+        ops.add_rmsnorm(ps, torch.zeros(2, 4))
+    done = ops.PartialSums(torch.zeros(3, 2, 4), out)
+    done.planes = None                    # added up already: nothing to go stale
+    ops._workspace(cpu)
+    assert done.materialize() is out

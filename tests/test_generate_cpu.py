@@ -42,7 +42,7 @@ def test_windowed_layers_have_a_smaller_pool(tmp_path, cpu_ops):
     w, cfg = plain.load(d)
     prompts = [tiny.random_tokens(n, cfg["vocab_size"], 90 + n) for n in (90, 61, 75)]
     want = [plain.greedy(w, cfg, p, 6) for p in prompts]
-    m = lm(d, max_seq_len=128)
+    m = lm(d, max_seq_len=128, intermediate_steps=1)
     windowed, rest = sorted(m.executor.cache.groups, key=lambda g: g.need.window is None)
     assert windowed.need.window == 8 and rest.need.window is None
     assert rest.pool.num_pages == 3 * 32 and windowed.pool.num_pages == 3 * (2 + 2) + 4
@@ -57,6 +57,71 @@ def test_windowed_layers_have_a_smaller_pool(tmp_path, cpu_ops):
     assert [r.output_token_ids for r in sorted(done, key=lambda r: r.request_id)] == want
     assert m.stats["preemptions"] == 0 and 6 <= most <= windowed.pool.num_pages
     assert windowed.pool.num_free == windowed.pool.num_pages
+
+
+def test_a_full_batch_past_the_window_still_runs_all_its_steps_in_a_row(tmp_path, cpu_ops):
+    """The windowed pool leaves room for `intermediate_steps` tokens ahead of every request: a full batch whose
+    requests are all past the window gets runs of that many decode steps, not runs halved for want of pages."""
+    d = tiny.write_model("A", str(tmp_path / "A"), std=0.5)      # window 8, pages of 4
+    _, cfg = plain.load(d)
+    m = lm(d, max_seq_len=160, intermediate_steps=16)
+    windowed = next(g for g in m.executor.cache.groups if g.need.window is not None)
+    assert windowed.pool.num_pages == 3 * (2 + 2) + 3 * 16 // 4
+    for i, n in enumerate((40, 33, 47)):     # staggered: the requests cross page edges at different steps
+        m.add_request(i, tiny.random_tokens(n, cfg["vocab_size"], 20 + n), SamplingParams(temperature=0.0, max_decode_steps=64,
+                                                                                         ignore_eos=True))
+    m.step_log = []
+    full_runs = 0
+    while m.scheduler.has_work():
+        left = min((64 - len(r.output_token_ids) for r in m.scheduler.running), default=0)
+        decoding = bool(m.scheduler.running) and not m.scheduler.waiting and all(
+            r.num_computed == r.num_tokens - 1 for r in m.scheduler.running)
+        m.step()
+        m.executor.cache.check()
+        if decoding:      # a run is as long as the requests' own limits allow: pages never cut it short
+            assert m.step_log[-1][0] == min(16, left), (m.step_log[-1], left)
+            full_runs += m.step_log[-1][0] == 16
+    assert full_runs == 3
+    assert m.stats["preemptions"] == 0 and windowed.pool.num_free == windowed.pool.num_pages
+
+
+def test_an_adopted_request_goes_on_where_one_that_ran_its_prompt_stands(tmp_path, cpu_ops):
+    """`adopt_request` (what the benchmark uses to start decoding at a long context): the pages are reserved and given
+    back as the prompt's portions would have done, so with the keys and values that the real run left in them the
+    adopted request generates the same tokens, windowed layers included; and nothing is left behind afterwards."""
+    import pytest
+    from simply_amd.cache import OutOfPages
+
+    d = tiny.write_model("A", str(tmp_path / "A"), std=0.5)      # window 8, pages of 4, budget 16
+    _, cfg = plain.load(d)
+    prompt = tiny.random_tokens(45, cfg["vocab_size"], 5)
+    params = SamplingParams(temperature=0.0, max_decode_steps=9, ignore_eos=True)
+    a = lm(d, max_seq_len=128, intermediate_steps=4)
+    want = a.generate([prompt], sampling_params=params)[0].output_token_ids
+    b = lm(d, max_seq_len=128, intermediate_steps=4)
+    r = b.adopt_request("r", prompt, len(prompt) - 1, params)
+    windowed = next(g for g in b.executor.cache.groups if g.need.window is not None)
+    assert len(windowed.pages_of("r")) == 5 and r.num_computed == 44       # blocks 6 to 10: the window and the last portion
+    for va, vb in zip(a.executor.cache.views, b.executor.cache.views):
+        for name, t in va.pages.items():
+            vb.pages[name].copy_(t)                                       # the same pages in the same order: see above
+    while b.scheduler.has_work():
+        b.step()
+        b.executor.cache.check()
+    assert r.output_token_ids == want
+    assert all(g.pool.num_free == g.pool.num_pages for g in b.executor.cache.groups)
+    # what does not fit is refused and leaves nothing behind
+    c = lm(d, max_seq_len=128, total_num_pages=13)
+    c.adopt_request("p", prompt[:20], 19, params)                         # 5 of the 13 pages
+    keeps_all = next(g for g in c.executor.cache.groups if g.need.window is None)
+    assert keeps_all.pool.num_free == 8
+    with pytest.raises(OutOfPages):
+        c.adopt_request("r", prompt, len(prompt) - 1, params)             # 11 more do not fit
+    assert [r.request_id for r in c.scheduler.running] == ["p"] and list(c.executor.cache.requests) == ["p"]
+    assert keeps_all.pool.num_free == 8 and len(keeps_all.pages_of("p")) == 5
+    c.executor.cache.check()
+    with pytest.raises(ValueError, match="computed tokens"):
+        c.adopt_request("q", prompt, len(prompt), params)
 
 
 def test_sampled_tokens_do_not_depend_on_the_batch(tmp_path, cpu_ops):

@@ -11,8 +11,41 @@ pytestmark = pytest.mark.gpu
 DT = [torch.float32, torch.bfloat16]
 
 
+def bf16_step(x: torch.Tensor) -> torch.Tensor:
+    """The spacing of bfloat16 numbers at the magnitude of x (8 bits of significand): 2^(floor(log2 |x|) - 7)."""
+    return torch.exp2(torch.floor(torch.log2(x.abs().clamp_min(1e-30))) - 7)
+
+
 def tol(dtype):
-    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(bf16_steps=1.0)
+
+
+def gated(t):
+    """The tolerance of a gated product: both of its products are rounded to bfloat16 before the activation and
+    the multiplication (act(g) * u with |act'| <= 1.13), and the result once more: three rounding steps."""
+    return dict(t, bf16_steps=3.0 * t["bf16_steps"]) if "bf16_steps" in t else t
+
+
+def check(got, want, *, rtol=None, atol=None, bf16_steps=None, msg=None):
+    """A kernel's result against its plain reference.  With rtol / atol: torch's criterion (32-bit results).  With
+    bf16_steps: both sides were computed in 32-bit from the same bfloat16 inputs and rounded to bfloat16 once, so they
+    differ by a rounding step where the 32-bit values behind them differ in their last bits; every element must lie
+    within that many bfloat16 steps at the largest magnitude of its row (one step there is 0.39 to 0.78 % of that
+    magnitude; the reference's bars for its own attention kernel are 5e-3 and 1e-2 of such outputs:
+    simply/utils/ragged_paged_attention_test.py:471, simply/utils/rpa_shard_window_repro_test.py:234)."""
+    if bf16_steps is None:
+        torch.testing.assert_close(got, want, rtol=rtol, atol=atol, msg=msg)
+        return
+    got, want = got.float(), want.float()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert torch.isfinite(got).all()
+    rows = want.reshape(-1, want.shape[-1])
+    bound = bf16_steps * bf16_step(rows.abs().amax(dim=-1, keepdim=True))
+    excess = (got.reshape(rows.shape) - rows).abs() - bound
+    worst = int(excess.argmax())
+    assert excess.max().item() <= 0, (
+        msg, f"element {worst} of {tuple(want.shape)}: got {got.reshape(-1)[worst].item()}, want "
+             f"{want.reshape(-1)[worst].item()}, allowed {bound[worst // rows.shape[1]].item()}")
 
 
 def rand(shape, dtype, seed, scale=1.0):
@@ -32,7 +65,7 @@ def test_embed(dtype, V, D, T):
     table = rand((V, D), dtype, 0)
     tokens = torch.randint(0, V, (T,), dtype=torch.int32).cuda()
     got = ops.embed(table, tokens, 3.25)
-    torch.testing.assert_close(got, ref.embed(table, tokens, 3.25), rtol=1e-6, atol=1e-6)
+    check(got, ref.embed(table, tokens, 3.25), rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -43,10 +76,10 @@ def test_rmsnorm(dtype, T, D):
     w = rand((D,), dtype, 2, 0.3)
     for plus_one in (True, False):
         got = ops.rmsnorm(x, w, 1e-5, plus_one, dtype)
-        torch.testing.assert_close(got.float(), ref.rmsnorm(x, w, 1e-5, plus_one, dtype).float(), **tol(dtype))
+        check(got.float(), ref.rmsnorm(x, w, 1e-5, plus_one, dtype).float(), **tol(dtype))
     xa = x.to(dtype)
     got = ops.rmsnorm(xa, w, 1e-6, True, dtype)
-    torch.testing.assert_close(got.float(), ref.rmsnorm(xa, w, 1e-6, True, dtype).float(), **tol(dtype))
+    check(got.float(), ref.rmsnorm(xa, w, 1e-6, True, dtype).float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -64,10 +97,10 @@ def test_add_rmsnorm(dtype, T, D):
                       next_eps=1e-5, out_dtype=dtype)
             o_got = ops.add_rmsnorm(y, h_got, **kw)
             o_ref = ref.add_rmsnorm(y, h_ref, **kw)
-            torch.testing.assert_close(h_got, h_ref, rtol=1e-5, atol=1e-5)
+            check(h_got, h_ref, rtol=1e-5, atol=1e-5)
             assert (o_got is None) == (o_ref is None)
             if o_got is not None:
-                torch.testing.assert_close(o_got.float(), o_ref.float(), **tol(dtype))
+                check(o_got.float(), o_ref.float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -97,15 +130,15 @@ def test_rope_cache_write(dtype, H, K, hd, P, T, order):
     ops.rope_cache_write(qkv, positions, ts, 1.0, 12.0, H, K, hd, slots, kp, vp)
     ref.rope_cache_write(qkv2, positions, ts, 1.0, 12.0, H, K, hd, slots, kp2, vp2)
     t = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else tol(dtype)  # sin/cos of angles up to 8000 rad
-    torch.testing.assert_close(qkv[:, :H * hd].float(), qkv2[:, :H * hd].float(), **t)
-    torch.testing.assert_close(kp.float(), kp2.float(), **t)
-    torch.testing.assert_close(vp, vp2, rtol=0, atol=0)
+    check(qkv[:, :H * hd].float(), qkv2[:, :H * hd].float(), **t)
+    check(kp.float(), kp2.float(), **t)
+    check(vp, vp2, rtol=0, atol=0)
     # without rotation and without a cache: only the query scale
     q3 = rand((T, (H + 2 * K) * hd), dtype, 8)
     q4 = q3.clone()
     ops.rope_cache_write(q3, positions, None, 1.0, 3.0, H, K, hd)
-    torch.testing.assert_close(q3[:, :H * hd].float(), (q4[:, :H * hd].float() / 3.0).to(dtype).float(), **tol(dtype))
-    torch.testing.assert_close(q3[:, H * hd:], q4[:, H * hd:], rtol=0, atol=0)
+    check(q3[:, :H * hd].float(), (q4[:, :H * hd].float() / 3.0).to(dtype).float(), **tol(dtype))
+    check(q3[:, H * hd:], q4[:, H * hd:], rtol=0, atol=0)
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -115,14 +148,14 @@ def test_gemm_generic(dtype, M, N, K):
     a, w, w2 = rand((M, K), dtype, 9), rand((N, K), dtype, 10, 0.1), rand((N, K), dtype, 11, 0.1)
     t = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else tol(dtype)
     for algo in (ops.ALGO_AUTO, ops.ALGO_GENERIC):
-        torch.testing.assert_close(ops.gemm(a, w, algo=algo).float(), ref.gemm(a, w).float(), **t)
-        torch.testing.assert_close(ops.gemm(a, w, w2=w2, algo=algo).float(), ref.gemm(a, w, w2=w2).float(), **t)
+        check(ops.gemm(a, w, algo=algo).float(), ref.gemm(a, w).float(), **t)
+        check(ops.gemm(a, w, w2=w2, algo=algo).float(), ref.gemm(a, w, w2=w2).float(), **gated(t))
         got = ops.gemm(a, w, soft_cap=2.0, out_dtype=torch.float32, algo=algo)
         assert got.dtype == torch.float32
-        torch.testing.assert_close(got, ref.gemm(a, w, soft_cap=2.0, out_dtype=torch.float32), **t)
+        check(got, ref.gemm(a, w, soft_cap=2.0, out_dtype=torch.float32), **t)
     # rows of a wider buffer as input (a view), as the attention output is
     wide = rand((M, K + 24), dtype, 12)
-    torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], w).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
+    check(ops.gemm(wide[:, 8:8 + K], w).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
 
 
 def test_gemm_rows_do_not_depend_on_the_batch():
@@ -151,8 +184,7 @@ def paged_setup(dtype, S, H, Kh, hd, P, lens, seed):
             n = min(P, l - b * P)
             kp[page, :, :n] = torch.randn((Kh, n, hd), generator=g).to(dtype)
             vp[page, :, :, :n] = torch.randn((Kh, hd, n), generator=g).to(dtype)
-    from simply_amd.kernels.packing import rows_to_keys
-    return rows_to_keys(kp).cuda(), vp.cuda(), table.cuda()
+    return ref.rows_as_stored_keys(kp).cuda(), vp.cuda(), table.cuda()
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -177,7 +209,27 @@ def test_paged_attention_generic(dtype, H, Kh, hd, P, window, cap):
     want = ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap)
     assert torch.isfinite(got.float()).all()
     t = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else tol(dtype)
-    torch.testing.assert_close(got.float(), want.float(), **t)
+    check(got.float(), want.float(), **t)
+
+
+@pytest.mark.parametrize("P,hd", [(16, 32), (32, 256), (48, 64), (16, 48), (4, 32), (24, 64)])
+def test_key_page_layout(P, hd):
+    """The layout of a stored page of keys, three ways: the index arithmetic of the tests' reference (written from
+    the interface's description), the product's re-layout functions, and the kernel that writes keys into pages."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
+    rows = torch.arange(3 * 2 * P * hd, dtype=torch.float32).reshape(3, 2, P, hd).cuda()
+    assert torch.equal(rows_to_keys(rows), ref.rows_as_stored_keys(rows))
+    assert torch.equal(keys_to_rows(rows_to_keys(rows)), rows) and torch.equal(ref.stored_keys_as_rows(rows_to_keys(rows)), rows)
+    # the kernel: token t's key (no rotation) lands where the arithmetic says
+    T, K = 3 * P, 2
+    qkv = rand((T, (1 + 2 * K) * hd), torch.float32, 5)
+    slots = torch.randperm(3 * P).to(torch.int64).cuda()
+    kp, vp = torch.zeros((3, K, P, hd)).cuda(), torch.zeros((3, K, hd, P)).cuda()
+    ops.rope_cache_write(qkv, torch.zeros(T, dtype=torch.int32).cuda(), None, 1.0, 1.0, 1, K, hd, slots, kp, vp)
+    got = ref.stored_keys_as_rows(kp)
+    want = qkv[:, hd:(1 + K) * hd].reshape(T, K, hd)
+    assert torch.equal(got[slots // P, :, slots % P], want)
 
 
 def test_paged_attention_far_key_and_window_edge():
@@ -186,14 +238,13 @@ def test_paged_attention_far_key_and_window_edge():
     from simply_amd.kernels import ops
     H = Kh = 1
     hd, P, L = 32, 16, 300
-    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
     kp, vp, table = paged_setup(torch.float32, 1, H, Kh, hd, P, [L], 31)
-    kp = keys_to_rows(kp) * 0.01
+    kp = ref.stored_keys_as_rows(kp) * 0.01
     far = 37
     page, off = int(table[0, far // P]), far % P
     kp[page, 0, off] = 0.0
     kp[page, 0, off, 3] = 50.0
-    kp = rows_to_keys(kp)
+    kp = ref.rows_as_stored_keys(kp)
     vp[page, 0, :, off] = 7.0
     q = torch.zeros((1, hd)).cuda()
     q[0, 3] = 1.0
@@ -202,7 +253,7 @@ def test_paged_attention_far_key_and_window_edge():
         ps = torch.tensor([pos], dtype=torch.int32).cuda()
         out = ops.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=None)
         assert (abs(out.mean().item() - 7.0) < 1e-3) == sees, (window, pos, out.mean().item())
-        torch.testing.assert_close(out, ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=None),
+        check(out, ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=None),
                                    rtol=1e-4, atol=1e-5)
 
 
@@ -218,7 +269,7 @@ def test_sampling_kernel():
     tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
     rtok, rlp = ref.sample(logits, temperature, top_k, top_p, seed, counter)
     assert tok.tolist() == rtok.tolist()
-    torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+    check(lp, rlp, rtol=1e-4, atol=1e-4)
     assert tok[0].item() == int(logits[0].argmax()) and tok[3].item() == int(logits[3].argmax())
     # same seed and counter: same token; another counter: (almost surely) another stream
     tok2, _ = ops.sample(logits, temperature, top_k, top_p, seed, counter)
@@ -254,16 +305,16 @@ def test_gemm_skinny(M, N, K):
         if (shape % 100) * 2 * blocks * 16 * 17 * 4 > 65536:
             continue   # the waves' tiles of the gated product would not fit in LDS: the library refuses that
         kw = dict(algo=ops.ALGO_SKINNY, shape=shape)
-        torch.testing.assert_close(ops.gemm(a, w, **kw).float(), ref.gemm(a, w).float(), rtol=2e-2, atol=2e-2)
-        torch.testing.assert_close(ops.gemm(a, w, w2=w2, **kw).float(), ref.gemm(a, w, w2=w2).float(), rtol=2e-2, atol=2e-2)
+        check(ops.gemm(a, w, **kw).float(), ref.gemm(a, w).float(), bf16_steps=1.0)
+        check(ops.gemm(a, w, w2=w2, **kw).float(), ref.gemm(a, w, w2=w2).float(), bf16_steps=3.0)
         got = ops.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32, **kw)
-        torch.testing.assert_close(got, ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
+        check(got, ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
     # the same call twice gives the same bits (the order of the partial sums is fixed)
     assert torch.equal(ops.gemm(a, w, algo=ops.ALGO_SKINNY, shape=804), ops.gemm(a, w, algo=ops.ALGO_SKINNY, shape=804))
     # a view with a row stride, as the attention output is
     wide = rand((M, K + 16), torch.bfloat16, 53)
-    torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], w, algo=ops.ALGO_SKINNY).float(), ref.gemm(wide[:, 8:8 + K], w).float(),
-                               rtol=2e-2, atol=2e-2)
+    check(ops.gemm(wide[:, 8:8 + K], w, algo=ops.ALGO_SKINNY).float(), ref.gemm(wide[:, 8:8 + K], w).float(),
+                               bf16_steps=1.0)
 
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 7, 8, 9])
@@ -279,18 +330,18 @@ def test_gemm_skinny_with_tiled_weights_and_few_rows(M, N, K):
     a, w, w2 = rand((M, K), torch.bfloat16, 58), rand((N, K), torch.bfloat16, 59, 0.05), rand((N, K), torch.bfloat16, 60, 0.05)
     a[M - 1, K // 3] = 40.0      # one activation that stands out: its chunk must meet its own weights
     a[0, K - 1] = -30.0
-    t = dict(rtol=2e-2, atol=2e-2)
+    t = dict(bf16_steps=1.0)
     for waves in (0, 1, 3, 8):
         kw = dict(algo=ops.ALGO_SKINNY, shape=1600 + waves if waves else 0)
         if waves and waves > K // 64:
             continue
-        torch.testing.assert_close(ops.gemm(a, pack_tiles(w), **kw).float(), ref.gemm(a, w).float(), **t)
-        torch.testing.assert_close(ops.gemm(a, pack_gate_up(w, w2), **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
-        torch.testing.assert_close(ops.gemm(a, pack_tiles(w), soft_cap=3.0, out_dtype=torch.float32, **kw),
+        check(ops.gemm(a, pack_tiles(w), **kw).float(), ref.gemm(a, w).float(), **t)
+        check(ops.gemm(a, pack_gate_up(w, w2), **kw).float(), ref.gemm(a, w, w2=w2).float(), **gated(t))
+        check(ops.gemm(a, pack_tiles(w), soft_cap=3.0, out_dtype=torch.float32, **kw),
                                    ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
     # rows of wider rows, as the attention output is
     big = rand((M, K + 32), torch.bfloat16, 61)
-    torch.testing.assert_close(ops.gemm(big[:, 16:16 + K], pack_tiles(w), algo=ops.ALGO_SKINNY).float(),
+    check(ops.gemm(big[:, 16:16 + K], pack_tiles(w), algo=ops.ALGO_SKINNY).float(),
                                ref.gemm(big[:, 16:16 + K], w).float(), **t)
     # the same rows to the bit whoever else is in the batch, within the kernel's variants of up to 4, up to 8 and more rows
     if M in (2, 3, 4):
@@ -303,7 +354,7 @@ def test_gemm_skinny_refuses_what_it_does_not_take():
     a, w = rand((4, 100), torch.bfloat16, 54), rand((8, 100), torch.bfloat16, 55)   # K is no multiple of 8
     with pytest.raises(KernelError, match="few-rows"):
         ops.gemm(a, w, algo=ops.ALGO_SKINNY)
-    torch.testing.assert_close(ops.gemm(a, w).float(), ref.gemm(a, w).float(), rtol=2e-2, atol=2e-2)   # auto falls back
+    check(ops.gemm(a, w).float(), ref.gemm(a, w).float(), bf16_steps=1.0)   # auto falls back
     with pytest.raises(KernelError):
         ops.gemm(rand((65, 64), torch.bfloat16, 56), rand((8, 64), torch.bfloat16, 57), algo=ops.ALGO_SKINNY)
 
@@ -344,7 +395,7 @@ def test_paged_attention_decode(H, Kh, hd, P, window, cap, splits):
                                max_kv_len=max(lens), max_q_len=max(q_lens), out=out, num_splits=splits)
     want = ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap)
     assert torch.isfinite(out.float()).all()
-    torch.testing.assert_close(out.float(), want.float(), rtol=2e-2, atol=2e-2)
+    check(out.float(), want.float(), bf16_steps=2.0)
     # a sub-range of the requests: the others' rows stay untouched
     out2 = torch.full_like(out, 7.0)
     ops.paged_attention_decode(q, kp, vp, table, meta, 2, 3, H, window=window, soft_cap=cap, max_kv_len=max(lens),
@@ -353,7 +404,7 @@ def test_paged_attention_decode(H, Kh, hd, P, window, cap, splits):
     # (with its own choice of key ranges the library cuts differently for 3 requests than for 8: equal up to rounding)
     if splits:
         assert torch.equal(out2[a:b], out[a:b])
-    torch.testing.assert_close(out2[a:b].float(), out[a:b].float(), rtol=2e-2, atol=2e-2)
+    check(out2[a:b].float(), out[a:b].float(), bf16_steps=2.0)
     assert (out2[:a] == 7).all() and (out2[b:] == 7).all()
 
 
@@ -361,14 +412,13 @@ def test_paged_attention_decode_far_key():
     """A key 3000 positions back with a score that stands out, among keys cut over many workgroups."""
     from simply_amd.kernels import ops
     H, Kh, hd, P, L = 2, 1, 128, 16, 3100
-    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
     kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 63)
-    kp = keys_to_rows(kp) * 0.01
+    kp = ref.stored_keys_as_rows(kp) * 0.01
     far = 71
     page, off = int(table[0, far // P]), far % P
     kp[page, 0, off] = 0.0
     kp[page, 0, off, 5] = 60.0
-    kp = rows_to_keys(kp)
+    kp = ref.rows_as_stored_keys(kp)
     vp[page, 0, :, off] = 3.0
     meta, ts, ps = seq_meta_for([L], [1])
     q = torch.zeros((1, 4 * hd), dtype=torch.bfloat16).cuda()
@@ -391,15 +441,15 @@ def test_gemm_tiled_weights(M, N, K):
     tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
     assert torch.equal(unpack_tiles(tw), w)
     assert all(torch.equal(x, y) for x, y in zip(unpack_gate_up(tw2), (w, w2)))
-    t = dict(rtol=2e-2, atol=2e-2)
-    torch.testing.assert_close(ops.gemm(a, tw).float(), ref.gemm(a, w).float(), **t)
-    torch.testing.assert_close(ops.gemm(a, tw2).float(), ref.gemm(a, w, w2=w2).float(), **t)
-    torch.testing.assert_close(ops.gemm(a, tw2, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w, w2=w2).float(), **t)
-    torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32),
+    t = dict(bf16_steps=1.0)
+    check(ops.gemm(a, tw).float(), ref.gemm(a, w).float(), **t)
+    check(ops.gemm(a, tw2).float(), ref.gemm(a, w, w2=w2).float(), **gated(t))
+    check(ops.gemm(a, tw2, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w, w2=w2).float(), **gated(t))
+    check(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32),
                                ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
-    torch.testing.assert_close(ops.gemm(a, tw, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w).float(), **t)
+    check(ops.gemm(a, tw, algo=ops.ALGO_GENERIC).float(), ref.gemm(a, w).float(), **t)
     tokens = torch.randint(0, N, (9,), dtype=torch.int32).cuda()
-    torch.testing.assert_close(ops.embed(tw, tokens, 1.5), ref.embed(w, tokens, 1.5), rtol=1e-6, atol=1e-6)
+    check(ops.embed(tw, tokens, 1.5), ref.embed(w, tokens, 1.5), rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 48, 64), (100, 100, 72), (128, 333, 1000), (300, 2304, 2048), (1, 130, 96),
@@ -410,17 +460,17 @@ def test_gemm_tiled(M, N, K):
     from simply_amd.kernels.packing import pack_gate_up, pack_tiles
     a, w, w2 = rand((M, K), torch.bfloat16, 80), rand((N, K), torch.bfloat16, 81, 0.05), rand((N, K), torch.bfloat16, 82, 0.05)
     tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
-    t = dict(rtol=2e-2, atol=2e-2)
+    t = dict(bf16_steps=1.0)
     kw = dict(algo=ops.ALGO_TILED)
     for cuts in (0, 1, 3):   # K whole, or cut over workgroups with the partial tiles added by a second kernel
         kw = dict(algo=ops.ALGO_TILED, shape=cuts)
-        torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), ref.gemm(a, w).float(), **t)
-        torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **t)
-        torch.testing.assert_close(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw),
+        check(ops.gemm(a, tw, **kw).float(), ref.gemm(a, w).float(), **t)
+        check(ops.gemm(a, tw2, **kw).float(), ref.gemm(a, w, w2=w2).float(), **gated(t))
+        check(ops.gemm(a, tw, soft_cap=3.0, out_dtype=torch.float32, **kw),
                                    ref.gemm(a, w, soft_cap=3.0, out_dtype=torch.float32), rtol=2e-3, atol=2e-3)
     kw = dict(algo=ops.ALGO_TILED)
     wide = rand((M, K + 16), torch.bfloat16, 83)
-    torch.testing.assert_close(ops.gemm(wide[:, 8:8 + K], tw, **kw).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
+    check(ops.gemm(wide[:, 8:8 + K], tw, **kw).float(), ref.gemm(wide[:, 8:8 + K], w).float(), **t)
     from simply_amd.kernels.lib import KernelError
     with pytest.raises(KernelError, match="tiled"):
         ops.gemm(a, w, **kw)     # row-major weights are refused
@@ -436,18 +486,18 @@ def test_gemm_wide(M, N, K):
     from simply_amd.kernels.packing import pack_gate_up, pack_tiles
     a, w, w2 = rand((M, K), torch.bfloat16, 90), rand((N, K), torch.bfloat16, 91, 0.05), rand((N, K), torch.bfloat16, 92, 0.05)
     tw, tw2 = pack_tiles(w), pack_gate_up(w, w2)
-    t = dict(rtol=2e-2, atol=2e-2)
+    t = dict(bf16_steps=1.0)
     want, want_gated = ref.gemm(a, w).float(), ref.gemm(a, w, w2=w2).float()
     # large tiles, and the small ones with deeper pipelines that products of a few hundred rows get
     for shape in (0, 2256192, 3256128, 3128256, 3192128, 2128192, 3128128, 3128064, 3064128, 3064064, 6064064, 5128064,
                   4128128, 6064128):
         kw = dict(algo=ops.ALGO_WIDE, shape=shape)
-        torch.testing.assert_close(ops.gemm(a, tw, **kw).float(), want, **t)
-        torch.testing.assert_close(ops.gemm(a, tw2, **kw).float(), want_gated, **t)
+        check(ops.gemm(a, tw, **kw).float(), want, **t)
+        check(ops.gemm(a, tw2, **kw).float(), want_gated, **gated(t))
     # K cut over two, three and seven workgroups per tile (their partial tiles summed by a second kernel); a cut
     # that K is too short for shrinks to what it allows
     for shape in (20000000 + 3128128, 30000000 + 6064064, 70000000 + 3256128, 20000000 + 5128064, 30000000 + 3192128):
-        torch.testing.assert_close(ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=shape).float(), want, **t)
+        check(ops.gemm(a, tw, algo=ops.ALGO_WIDE, shape=shape).float(), want, **t)
     if K >= 128:
         with pytest.raises(KernelError, match="cuts K only without"):
             ops.gemm(a, tw2, algo=ops.ALGO_WIDE, shape=20000000 + 3128128)
@@ -462,7 +512,7 @@ def test_gemm_wide(M, N, K):
     big = rand((M, K + 16), torch.bfloat16, 93)
     out = torch.full((M, N + 12), 7.0, dtype=torch.bfloat16, device="cuda")
     ops.gemm(big[:, 8:8 + K], tw, out=out[:, 4:4 + N], **kw)
-    torch.testing.assert_close(out[:, 4:4 + N].float(), ref.gemm(big[:, 8:8 + K], w).float(), **t)
+    check(out[:, 4:4 + N].float(), ref.gemm(big[:, 8:8 + K], w).float(), **t)
     assert (out[:, :4] == 7.0).all() and (out[:, 4 + N:] == 7.0).all()
     with pytest.raises(KernelError, match="wide"):
         ops.gemm(a, w, **kw)                                     # row-major weights
@@ -474,7 +524,7 @@ def test_gemm_wide(M, N, K):
         ops.gemm(a, pack_tiles(w[:N - 2].contiguous()), **kw)  # N that is no multiple of 4
     # it is what the library chooses by itself for products that are not bound by streaming the weights; for what it
     # refuses, the tiled kernel
-    torch.testing.assert_close(ops.gemm(a, pack_tiles(w[:N - 2].contiguous())).float(), want[:, :N - 2], **t)
+    check(ops.gemm(a, pack_tiles(w[:N - 2].contiguous())).float(), want[:, :N - 2], **t)
 
 
 @pytest.mark.parametrize("D", [5000, 5200])
@@ -487,8 +537,8 @@ def test_add_rmsnorm_wide_rows(D):
     h_ref = h.clone()
     o = ops.add_rmsnorm(y, h, post_weight=w1, post_eps=1e-6, next_weight=w2, next_eps=1e-6, out_dtype=torch.bfloat16)
     o_ref = ref.add_rmsnorm(y, h_ref, post_weight=w1, post_eps=1e-6, next_weight=w2, next_eps=1e-6, out_dtype=torch.bfloat16)
-    torch.testing.assert_close(h, h_ref, rtol=1e-5, atol=1e-5)
-    torch.testing.assert_close(o.float(), o_ref.float(), rtol=2e-2, atol=2e-2)
+    check(h, h_ref, rtol=1e-5, atol=1e-5)
+    check(o.float(), o_ref.float(), bf16_steps=1.0)
 
 
 def test_sampling_rows_at_odd_addresses():
@@ -506,7 +556,7 @@ def test_sampling_rows_at_odd_addresses():
     tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
     rtok, rlp = ref.sample(logits, temperature, top_k, top_p, seed, counter)
     assert tok.tolist() == rtok.tolist()
-    torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+    check(lp, rlp, rtol=1e-4, atol=1e-4)
     for r in (0, 2, 4):
         assert tok[r].item() == int(logits[r].argmax())
 
@@ -536,7 +586,7 @@ def test_sampling_greedy_rows_of_a_large_vocabulary(V, offset):
     assert tok.tolist() == rtok.tolist()
     assert tok.tolist()[:3] == [V - 1, part - 1, 3] and tok[4].item() == 0
     assert tok[5].item() == int(logits[5].argmax())
-    torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+    check(lp, rlp, rtol=1e-4, atol=1e-4)
 
 
 @pytest.mark.parametrize("V", [20000, 256000])
@@ -561,7 +611,7 @@ def test_sampling_top_k_and_top_p_of_a_large_vocabulary(V):
         for modes in (7, 1, 3, 5, 0):
             tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter, modes=modes)
             assert tok.tolist() == rtok.tolist(), (modes, tok.tolist(), rtok.tolist())
-            torch.testing.assert_close(lp, rlp, rtol=1e-4, atol=1e-4)
+            check(lp, rlp, rtol=1e-4, atol=1e-4)
     assert rtok[6].item() in range(100, 105) and rtok[7].item() == 7
     # rows that ask for one thing only, with the kernels for exactly that
     for modes, rows in ((ops.SAMPLE_DRAWN | ops.SAMPLE_TOP_K, [0, 3, 6]), (ops.SAMPLE_DRAWN | ops.SAMPLE_TOP_P, [1, 7]),
@@ -571,7 +621,7 @@ def test_sampling_top_k_and_top_p_of_a_large_vocabulary(V):
         tok, lp = ops.sample(logits[idx].contiguous(), temperature[idx], top_k[idx], top_p[idx], seed[idx], counter,
                              modes=modes)
         assert tok.tolist() == rtok[idx].tolist()
-        torch.testing.assert_close(lp, rlp[idx], rtol=1e-4, atol=1e-4)
+        check(lp, rlp[idx], rtol=1e-4, atol=1e-4)
 
 
 @pytest.mark.parametrize("V", [333, 1001, 20000])
@@ -590,7 +640,7 @@ def test_score(V):
     seed = torch.arange(R, dtype=torch.int64).cuda() * 5 + 3
     counter = torch.full((R,), 2, dtype=torch.int32).cuda()
     tok, lp = ops.sample(logits, temperature, top_k, top_p, seed, counter)
-    torch.testing.assert_close(ops.score(logits, temperature, top_k, top_p, tok), lp, rtol=1e-5, atol=1e-5)
+    check(ops.score(logits, temperature, top_k, top_p, tok), lp, rtol=1e-5, atol=1e-5)
     best, worst = logits.argmax(-1).int(), logits.argmin(-1).int()
     fifth = logits.topk(5).indices[:, 4].int().contiguous()
     for given in (tok, best, worst, fifth, torch.full((R,), 104, dtype=torch.int32).cuda()):
@@ -598,7 +648,7 @@ def test_score(V):
         want = ref.score(logits, temperature, top_k, top_p, given)
         masked = want < -1e37
         assert torch.equal(got < -1e37, masked), (given.tolist(), got.tolist(), want.tolist())
-        torch.testing.assert_close(got[~masked], want[~masked], rtol=1e-4, atol=1e-4)
+        check(got[~masked], want[~masked], rtol=1e-4, atol=1e-4)
         assert (got[masked] == ops.SCORE_MASKED).all()
     got = ops.score(logits, temperature, top_k, top_p, worst)
     assert got[4] == ops.SCORE_MASKED and got[8] == ops.SCORE_MASKED and got[5] > -1e3   # greedy rows; a plain draw
@@ -614,14 +664,14 @@ def test_gemm_dispatch_at_a_few_hundred_rows(M, N, K):
     from simply_amd.kernels.packing import pack_gate_up, pack_tiles
     a = rand((M, K), torch.bfloat16, 140)
     w, w2 = rand((N, K), torch.bfloat16, 141, 0.03), rand((N, K), torch.bfloat16, 142, 0.03)
-    t = dict(rtol=2e-2, atol=2e-2)
-    torch.testing.assert_close(ops.gemm(a, pack_tiles(w)).float(), ref.gemm(a, w).float(), **t)
+    t = dict(bf16_steps=1.0)
+    check(ops.gemm(a, pack_tiles(w)).float(), ref.gemm(a, w).float(), **t)
     if N <= 2304:
-        torch.testing.assert_close(ops.gemm(a, pack_gate_up(w, w2)).float(), ref.gemm(a, w, w2=w2).float(), **t)
+        check(ops.gemm(a, pack_gate_up(w, w2)).float(), ref.gemm(a, w, w2=w2).float(), **gated(t))
     # rows of wider rows in and out, as the attention output and the fused projection are
     big, out = rand((M, K + 64), torch.bfloat16, 143), torch.zeros((M, N + 8), dtype=torch.bfloat16, device="cuda")
     ops.gemm(big[:, 32:32 + K], pack_tiles(w), out=out[:, :N])
-    torch.testing.assert_close(out[:, :N].float(), ref.gemm(big[:, 32:32 + K], w).float(), **t)
+    check(out[:, :N].float(), ref.gemm(big[:, 32:32 + K], w).float(), **t)
     assert not out[:, N:].any()
 
 
@@ -636,11 +686,11 @@ def test_gemm_dispatch_of_few_rows_against_a_long_k(M, N, K):
     from simply_amd.kernels.packing import pack_tiles
     a = rand((M, K), torch.bfloat16, 150)
     w = rand((N, K), torch.bfloat16, 151, 0.03)
-    t = dict(rtol=2e-2, atol=3e-2)
-    torch.testing.assert_close(ops.gemm(a, pack_tiles(w)).float(), ref.gemm(a, w).float(), **t)
+    t = dict(bf16_steps=1.0)
+    check(ops.gemm(a, pack_tiles(w)).float(), ref.gemm(a, w).float(), **t)
     big, out = rand((M, K + 64), torch.bfloat16, 152), torch.zeros((M, N + 8), dtype=torch.bfloat16, device="cuda")
     ops.gemm(big[:, 32:32 + K], pack_tiles(w), out=out[:, :N])
-    torch.testing.assert_close(out[:, :N].float(), ref.gemm(big[:, 32:32 + K], w).float(), **t)
+    check(out[:, :N].float(), ref.gemm(big[:, 32:32 + K], w).float(), **t)
     assert not out[:, N:].any()
 
 
@@ -660,24 +710,25 @@ def test_gated_activations_in_every_product_kernel(M, activation):
     assert want.abs().max() > 0.5
     if activation:
         assert not torch.allclose(want, ref.gemm(a, w, w2=w2).float(), rtol=2e-2, atol=2e-2)   # the activations differ
-    t = dict(rtol=2e-2, atol=2e-2)
+    # (the squared relu doubles the relative error of its argument: one step more than gelu and silu)
+    t = dict(bf16_steps=4.0 if activation == 2 else 3.0)
     a32, w32, w232 = a.float(), w.float(), w2.float()
-    torch.testing.assert_close(ops.gemm(a32, w32, w2=w232, activation=activation),
+    check(ops.gemm(a32, w32, w2=w232, activation=activation),
                                ref.gemm(a32, w32, w2=w232, activation=activation), rtol=1e-4, atol=1e-4)
-    torch.testing.assert_close(ops.gemm(a, w, w2=w2, activation=activation, algo=ops.ALGO_GENERIC).float(), want, **t)
-    torch.testing.assert_close(ops.gemm(a, tg, activation=activation).float(), want, **t)      # the dispatcher's choice
+    check(ops.gemm(a, w, w2=w2, activation=activation, algo=ops.ALGO_GENERIC).float(), want, **t)
+    check(ops.gemm(a, tg, activation=activation).float(), want, **t)      # the dispatcher's choice
     if M <= 16:
-        torch.testing.assert_close(ops.gemm(a, tg, activation=activation, algo=ops.ALGO_SKINNY).float(), want, **t)
+        check(ops.gemm(a, tg, activation=activation, algo=ops.ALGO_SKINNY).float(), want, **t)
         h = a.float() * 3.0
         wn = rand((K,), torch.bfloat16, 133, 0.3)
         normed = ref.rmsnorm(h, wn, 1e-6, True, torch.bfloat16)
         got = ops.gemm_normed(None, h, None, tg, post_weight=None, post_eps=0.0, post_plus_one=True, next_weight=wn,
                               next_eps=1e-6, next_plus_one=True, activation=activation)
-        torch.testing.assert_close(got.float(), ref.gemm(normed, w, w2=w2, activation=activation).float(), **t)
+        check(got.float(), ref.gemm(normed, w, w2=w2, activation=activation).float(), **t)
     for cuts in (1, 2):
         got = ops.gemm(a, tg, activation=activation, algo=ops.ALGO_TILED, shape=cuts)
-        torch.testing.assert_close(got.float(), want, **t)
-    torch.testing.assert_close(ops.gemm(a, tg, activation=activation, algo=ops.ALGO_WIDE).float(), want, **t)
+        check(got.float(), want, **t)
+    check(ops.gemm(a, tg, activation=activation, algo=ops.ALGO_WIDE).float(), want, **t)
     from simply_amd.kernels.lib import KernelError
     with pytest.raises(KernelError, match="activation"):
         ops.gemm(a, tg, activation=3)
@@ -685,7 +736,7 @@ def test_gated_activations_in_every_product_kernel(M, activation):
 
 @pytest.mark.parametrize("M", [1, 3, 8, 9, 13, 16])
 @pytest.mark.parametrize("K,N", [(128, 96), (2304, 4096), (2560, 512), (2048, 200), (3584, 512), (4608, 64), (4640, 64),
-                                 (96, 40), (72, 64)])
+                                 (96, 40), (72, 64), (3072, 200), (4096, 512), (2816, 96), (3328, 64)])
 def test_gemm_normed(M, K, N):
     """Residual sum, two norms and the product in one kernel against the separate references."""
     from simply_amd.kernels import ops
@@ -696,28 +747,33 @@ def test_gemm_normed(M, K, N):
     tw, tg = pack_tiles(w), pack_gate_up(w, w2)
     fits = (8 if M <= 8 else 16) * (K + 8) * 2 + 8 * 2 * 16 * 17 * 4 <= 160 * 1024   # activations and tiles in LDS
     assert ops.gemm_normed_takes(M, tw) == (fits and K % 32 == 0 and K <= 4608)
+    # what it takes it computes; it says that it pays where it has a prologue for the width (the widths of the three
+    # Gemma 2 sizes and other multiples of 256 such as 3072 and 4096) or the row is at most 2560 wide
+    assert ops.gemm_normed_pays(M, tw) == (ops.gemm_normed_takes(M, tw)
+                                           and (K <= 2560 or K in (3072, 3584, 4096, 4608)))
+    assert not ops.gemm_normed_pays(M, pack_tiles(torch.zeros((16 * 8192 + 16, 64), dtype=torch.bfloat16).cuda()))
     if not ops.gemm_normed_takes(M, tw):
         return
     kw = dict(post_weight=wp, post_eps=1e-6, post_plus_one=True, next_weight=wn, next_eps=1e-5, next_plus_one=True)
-    t = dict(rtol=2e-2, atol=2e-2)
+    t = dict(bf16_steps=1.0)
     for with_y in (True, False):
         h_ref = h.clone()
         a_ref = ref.add_rmsnorm(y, h_ref, post_weight=wp, post_eps=1e-6, next_weight=wn, next_eps=1e-5,
                                 out_dtype=torch.bfloat16) if with_y else ref.rmsnorm(h, wn, 1e-5, True, torch.bfloat16)
         h_out = torch.full_like(h, 7.0)
         got = ops.gemm_normed(y if with_y else None, h, h_out if with_y else None, tw, **kw)
-        torch.testing.assert_close(got.float(), ref.gemm(a_ref, w).float(), **t)
+        check(got.float(), ref.gemm(a_ref, w).float(), **t)
         if with_y:
-            torch.testing.assert_close(h_out, h_ref, rtol=1e-5, atol=1e-5)
+            check(h_out, h_ref, rtol=1e-5, atol=1e-5)
         got = ops.gemm_normed(y if with_y else None, h, h_out if with_y else None, tg, **kw)
-        torch.testing.assert_close(got.float(), ref.gemm(a_ref, w, w2=w2).float(), **t)
+        check(got.float(), ref.gemm(a_ref, w, w2=w2).float(), **gated(t))
         got = ops.gemm_normed(y if with_y else None, h, h_out if with_y else None, tw, soft_cap=3.0,
                               out_dtype=torch.float32, **kw)
-        torch.testing.assert_close(got, ref.gemm(a_ref, w, soft_cap=3.0, out_dtype=torch.float32), rtol=5e-3, atol=5e-3)
+        check(got, ref.gemm(a_ref, w, soft_cap=3.0, out_dtype=torch.float32), rtol=5e-3, atol=5e-3)
     # without a post-norm the residual takes y as it is
     h_out = torch.empty_like(h)
     ops.gemm_normed(y, h, h_out, tw, **dict(kw, post_weight=None))
-    torch.testing.assert_close(h_out, h + y.float(), rtol=1e-6, atol=1e-6)
+    check(h_out, h + y.float(), rtol=1e-6, atol=1e-6)
     assert not ops.gemm_normed_takes(17, tw) and not ops.gemm_normed_takes(M, w)
 
 
@@ -758,12 +814,12 @@ def test_paged_attention_prefill(H, Kh, hd, P, window, cap, splits):
                                 max_kv_len=max(lens), max_q_len=per_unit, out=out, num_splits=splits)
     want = ref.paged_attention(q, kp, vp, table, ts, ps, H, window=window, soft_cap=cap)
     assert torch.isfinite(out.float()).all()
-    torch.testing.assert_close(out.float(), want.float(), rtol=2e-2, atol=2e-2)
+    check(out.float(), want.float(), bf16_steps=2.0)
     # the few-rows kernel on the same units gives the same up to rounding
     out2 = torch.zeros_like(out)
     ops.paged_attention_decode(q, kp, vp, table, units, 0, units.shape[0], H, window=window, soft_cap=cap,
                                max_kv_len=max(lens), max_q_len=per_unit, out=out2)
-    torch.testing.assert_close(out.float(), out2.float(), rtol=2e-2, atol=2e-2)
+    check(out.float(), out2.float(), bf16_steps=2.0)
     # a sub-range of the units: the other rows stay untouched
     first = next(i for i in range(units.shape[0]) if int(units[i, 0]) == 2)
     count = sum(1 for i in range(units.shape[0]) if int(units[i, 0]) == 2)
@@ -771,7 +827,7 @@ def test_paged_attention_prefill(H, Kh, hd, P, window, cap, splits):
     ops.paged_attention_prefill(q, kp, vp, table, units, first, count, H, window=window, soft_cap=cap,
                                 max_kv_len=max(lens), max_q_len=per_unit, out=out3, num_splits=splits)
     a, b = sum(q_lens[:2]), sum(q_lens[:3])
-    torch.testing.assert_close(out3[a:b].float(), out[a:b].float(), rtol=2e-2, atol=2e-2)
+    check(out3[a:b].float(), out[a:b].float(), bf16_steps=2.0)
     assert (out3[:a] == 7).all() and (out3[b:] == 7).all()
     with pytest.raises(Exception, match="groups of"):
         ops.paged_attention_prefill(q, kp, vp, table, units, 0, 3, H, window=window, soft_cap=cap,
@@ -782,15 +838,14 @@ def test_paged_attention_prefill_far_key_and_window_edge():
     """Every query row of a long portion must find one key far back whose score stands out, and a windowed
     layer must see it exactly while it is inside each row's own window."""
     from simply_amd.kernels import ops
-    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
     H, Kh, hd, P, L, Q = 2, 1, 128, 16, 2500, 600
     kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 73)
-    kp = keys_to_rows(kp) * 0.01
+    kp = ref.stored_keys_as_rows(kp) * 0.01
     far = 1871
     page, off = int(table[0, far // P]), far % P
     kp[page, 0, off] = 0.0
     kp[page, 0, off, 5] = 60.0
-    kp = rows_to_keys(kp)
+    kp = ref.rows_as_stored_keys(kp)
     vp[page, 0, :, off] = 3.0
     units = prefill_units([L], [Q], 8)
     q = torch.zeros((Q, 4 * hd), dtype=torch.bfloat16).cuda()
@@ -812,17 +867,16 @@ def test_paged_attention_far_keys_of_a_long_context(window):
     whose score stands out for it; in the prompt-portion kernel, the few-rows kernel (keys cut over workgroups) and
     the generic kernel, with and without a window."""
     from simply_amd.kernels import ops
-    from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
     H, Kh, hd, P, L, Q = 2, 1, 128, 16, 70000, 64
     kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 75)
-    kp = keys_to_rows(kp) * 0.01
+    kp = ref.stored_keys_as_rows(kp) * 0.01
     far = [3, 40001, 65535, 65536, 69000, L - 70]
     for f, at in enumerate(far):
         page, off = int(table[0, at // P]), at % P
         kp[page, 0, off] = 0.0
         kp[page, 0, off, 5 + f] = 60.0
         vp[page, 0, :, off] = float(f + 1)
-    kp = rows_to_keys(kp)
+    kp = ref.rows_as_stored_keys(kp)
     q = torch.zeros((Q, 4 * hd), dtype=torch.bfloat16).cuda()
     which = torch.arange(Q) % len(far)
     for i in range(Q):
@@ -871,7 +925,7 @@ def test_bfloat16_rounding_of_the_kernels():
 
 @pytest.mark.parametrize("M", [1, 8, 13])
 @pytest.mark.parametrize("H,Kh,hd,P,K", [(8, 4, 256, 16, 2304), (4, 2, 64, 16, 128), (3, 1, 32, 48, 96), (2, 2, 128, 32, 2560), (4, 2, 256, 16, 3584),
-                                         (4, 4, 128, 16, 4608)])
+                                         (4, 4, 128, 16, 4608), (6, 2, 128, 16, 3072), (4, 1, 64, 16, 4096), (2, 1, 32, 16, 2816)])
 @pytest.mark.parametrize("rotate", [True, False])
 def test_gemm_normed_rotary(M, H, Kh, hd, P, K, rotate):
     """Norms, q/k/v projection, rotation, query scale and cache write in one kernel against the same from the
@@ -902,14 +956,14 @@ def test_gemm_normed_rotary(M, H, Kh, hd, P, K, rotate):
         want = ops.gemm_normed(y if with_y else None, h, h_out2 if with_y else None, tw, **norm)
         ops.rope_cache_write(want, positions, ts, 1.0, 12.0, H, Kh, hd, slots, kp2, vp2)
         t = dict(rtol=1e-2, atol=1e-3)   # the same sums; the rotation's products may round one bfloat16 step apart
-        torch.testing.assert_close(got[:, :H * hd].float(), want[:, :H * hd].float(), **t)
-        torch.testing.assert_close(kp.float(), kp2.float(), **t)
+        check(got[:, :H * hd].float(), want[:, :H * hd].float(), **t)
+        check(kp.float(), kp2.float(), **t)
         assert torch.equal(vp, vp2)
         assert torch.equal(h_out, h_out2)
     # without pages only the queries are produced
     got = ops.gemm_normed_rotary(None, h, None, tw, **norm, positions=positions, timescale=ts, scale_factor=1.0,
                                  query_scale=12.0, num_heads=H, num_kv_heads=Kh, head_dim=hd)
-    torch.testing.assert_close(got[:, :H * hd].float(), want[:, :H * hd].float(), rtol=1e-2, atol=1e-3)
+    check(got[:, :H * hd].float(), want[:, :H * hd].float(), rtol=1e-2, atol=1e-3)
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 2304, 2048), (64, 2304, 9216), (64, 2304, 2048), (100, 3584, 4096), (512, 2304, 9216),

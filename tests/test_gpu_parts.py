@@ -338,6 +338,67 @@ def test_toy_state_advances_once_per_step_under_graphs(toy_registry):
         torch.testing.assert_close(replayed[r], whole, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_pages_of_its_own_layout(dtype):
+    """A toy mixer (tests/toy_parts.py) that keeps one latent vector per token in float32 pages [page, rank,
+    page_size], through a need class of the test's own: two more cache groups beside the attention layer's, one of
+    them windowed.  Whole, cut and mixed in a pool so small that pages are used again (poisoned in between) give the
+    same logits, in both element types; the framework's files know nothing of the layout."""
+    import numpy as np
+    import toy_parts
+
+    registry.MIXERS.register("toy_latent_mean", toy_parts.LatentMeanMixer)
+    try:
+        model = DecoderModel(toy_parts.latent_model_spec())
+        tdtype = torch.float32 if dtype == "float32" else torch.bfloat16
+        init_random(model, 0, tdtype, torch.device(DEV), std=0.2)
+        cfg = EngineConfig(activation_dtype=dtype, page_size=4, batch_size=3, max_seq_len=64, max_num_issue_tokens=32,
+                           total_num_pages=24, device=DEV, use_graphs=False, poison_freed_pages=True, intermediate_steps=1)
+        ex = Executor(model, cfg)
+        assert [type(g.need).__name__ for g in ex.cache.groups] == ["PagedKVNeed", "LatentNeed", "LatentNeed"]
+        assert ex.cache.views[1].pages["latent"].dtype == torch.float32 and ex.cache.views[0].k_pages.dtype == tdtype
+        reqs = {f"r{i}": tiny.random_tokens(n, 128, 40 + i) for i, n in enumerate((30, 17, 26, 9, 22))}
+        tol = dict(rtol=1e-4, atol=1e-4) if dtype == "float32" else dict(rtol=5e-2, atol=5e-2)
+
+        def run(rid, t, cuts):
+            ex.add_request(rid)
+            out, i = [], 0
+            for c in cuts:
+                out.append(ex.step([StepEntry(rid, t[i:i + c], list(range(c)))]).cpu())
+                i += c
+            ex.finish_request(rid)
+            return torch.cat(out)
+
+        whole = {r: run(r, t, [len(t)]) for r, t in reqs.items()}
+        assert all(torch.isfinite(v).all() and v.abs().max() > 0 for v in whole.values())
+        torch.testing.assert_close(run("x", reqs["r0"], [7, 2, 9, 1, 11]), whole["r0"], **tol)
+        pending, live, got = list(reqs), {}, {r: [] for r in reqs}
+        rng = np.random.default_rng(1)
+        while pending or live:
+            while pending and len(live) < 3 and sum(-(-len(reqs[r]) // 4) for r in live) + -(-len(reqs[pending[0]]) // 4) <= 24:
+                live[pending[0]] = 0
+                ex.add_request(pending.pop(0))
+            entries = []
+            for r in list(live):
+                n = min(len(reqs[r]) - live[r], int(rng.integers(1, 8)))
+                entries.append(StepEntry(r, reqs[r][live[r]:live[r] + n], list(range(n))))
+            logits, i = ex.step(entries).cpu(), 0
+            for e in entries:
+                n = len(e.tokens)
+                got[e.request_id].append(logits[i:i + n])
+                i += n
+                live[e.request_id] += n
+                if live[e.request_id] == len(reqs[e.request_id]):
+                    ex.finish_request(e.request_id)
+                    del live[e.request_id]
+            ex.cache.check()
+        for r in reqs:
+            torch.testing.assert_close(torch.cat(got[r]), whole[r], **tol)
+        assert all(g.pool.num_free == g.pool.num_pages for g in ex.cache.groups)
+    finally:
+        registry.MIXERS.unregister("toy_latent_mean")
+
+
 def test_unknown_part_names_are_refused():
     spec = toy_spec()   # the toy kinds are not registered here
     with pytest.raises(ValueError, match="unknown (mixer|feed-forward|position encoding)"):

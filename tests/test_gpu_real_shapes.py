@@ -54,12 +54,10 @@ def test_real_layer_shapes(tmp_path, gpu_lib, shape, dtype):
             ref.check(got, what=cuts)
 
 
-@pytest.mark.parametrize("library_rows", [256, 0])
-def test_long_portions(tmp_path, gpu_lib, library_rows):
-    """Portions of several hundred tokens at the 2B layer sizes: the kernels for many rows (the library's or the
-    tiled product, the residual/norm and rotary kernels with a wave per row and a block per token, attention with
+def test_long_portions(tmp_path, gpu_lib):
+    """Portions of several hundred tokens at the 2B layer sizes: the kernels for many rows (the wide
+    product, the residual/norm and rotary kernels with a wave per row and a block per token, attention with
     64 query rows per workgroup over a history and a window), against the plain implementation."""
-    from simply_amd.kernels import ops
     d = dict(architectures=["Gemma2ForCausalLM"], num_hidden_layers=2, vocab_size=2000, rms_norm_eps=1e-6,
              rope_theta=10000.0, sliding_window=200, attn_logit_softcapping=50.0, final_logit_softcapping=30.0,
              max_position_embeddings=8192, initializer_range=0.02, **SHAPES["2b"])
@@ -69,18 +67,13 @@ def test_long_portions(tmp_path, gpu_lib, library_rows):
     ref = bounds.reference(w, cfg, tokens, "bfloat16")
     ecfg = EngineConfig(activation_dtype="bfloat16", page_size=16, batch_size=2, max_seq_len=704, max_num_issue_tokens=704,
                         total_num_pages=48, device="cuda:0", use_graphs=False, poison_freed_pages=True)
-    before = ops.library_gemm_min_rows()
-    ops.set_library_gemm_min_rows(library_rows)
-    try:
-        model, _ = load_model(folder, ecfg.dtype, "cuda:0")
-        ex = Executor(model, ecfg)
-        for cuts in ([700], [600, 98, 2]):
-            ex.add_request("r")
-            out, i = [], 0
-            for c in cuts:
-                out.append(ex.step([StepEntry("r", tokens[i:i + c], list(range(c)))]).cpu())
-                i += c
-            ex.finish_request("r")
-            ref.check(torch.cat(out), what=cuts)
-    finally:
-        ops.set_library_gemm_min_rows(before)
+    model, _ = load_model(folder, ecfg.dtype, "cuda:0")
+    ex = Executor(model, ecfg)
+    for cuts in ([700], [600, 98, 2]):
+        ex.add_request("r")
+        out, i = [], 0
+        for c in cuts:
+            out.append(ex.step([StepEntry("r", tokens[i:i + c], list(range(c)))]).cpu())
+            i += c
+        ex.finish_request("r")
+        ref.check(torch.cat(out), what=cuts)

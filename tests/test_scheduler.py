@@ -185,3 +185,68 @@ def test_decoding_requests_ask_the_cache_once():
         [(f"r{i}", 1, True) for i in range(32)]
     assert len(calls) <= 3 and max(calls) == 32
     cache.check()
+
+
+@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("window,page_size,slots,budget,ahead", [(8, 4, 4, 16, 8), (50, 16, 6, 64, 16)])
+def test_a_windowed_pool_as_tight_as_the_engine_makes_it(seed, window, page_size, slots, budget, ahead):
+    """The engine gives a windowed group only the pages that its requests can hold at once
+    (`CacheManager(max_step_tokens=...)`), not as many as the group that keeps everything.  Random long prompts and
+    runs of decode steps that reserve ahead and end early, as `LMInterface.step` and `Executor.decode_many` do them
+    (pages for the whole run reserved first, `mark_issued` for the steps that ran): admission, portions that shrink
+    to the free pages, requests left out of a step and preemption never run the tight pool dry, lose a page or
+    finish a request for want of room."""
+    import numpy as np
+
+    from simply_amd.cache import OutOfPages
+
+    rng = np.random.default_rng(1000 * window + seed)
+    max_len = 40 * page_size
+    needs = [(PagedKVNeed(1, 16, window), None), (PagedKVNeed(1, 16, None), None)]
+    pages = slots * (max_len // page_size)
+    cache = CacheManager(needs, page_size=page_size, num_pages=pages, num_slots=slots, max_seq_len=max_len,
+                         max_step_tokens=max(budget, slots * ahead))
+    windowed = next(g for g in cache.groups if g.window is not None)
+    assert windowed.pool.num_pages < pages // 2
+    sched = Scheduler(cache, max_num_issue_tokens=budget, max_seq_len=max_len)
+    todo = [req(f"r{i}", int(rng.integers(1, max_len - 40)), steps=int(rng.integers(1, 40)), ignore_eos=True)
+            for i in range(14)]
+    finished, arrivals = [], 0
+    for _ in range(4000):
+        while todo and rng.random() < 0.3:
+            sched.add(todo.pop())
+        if not sched.has_work():
+            if not todo:
+                break
+            sched.add(todo.pop())
+        out = sched.schedule()
+        finished += out.finished
+        if not out.scheduled:
+            continue
+        cache.check()
+        decoding = all(s.num_tokens == 1 and s.samples for s in out.scheduled)
+        n = 1
+        if decoding and not sched.waiting and len(out.scheduled) == len(sched.running):
+            n = ahead
+            for s in out.scheduled:
+                n = min(n, s.request.params.max_decode_steps - len(s.request.output_token_ids))
+            while n > 1 and not cache.can_reserve([(s.request.request_id, s.start, n) for s in out.scheduled]):
+                n //= 2
+        wants = [(s.request.request_id, s.start, max(s.num_tokens, n)) for s in out.scheduled]
+        cache.reserve_all(wants)       # as the step function does (OutOfPages here would fail the test)
+        ran = int(rng.integers(1, n + 1)) if n > 1 else 1        # a run may end early
+        live = list(out.scheduled)
+        for k in range(ran):
+            now = [type(s)(s.request, s.start + k, s.num_tokens, s.samples) for s in live]
+            finished += sched.update(now, [7] * len(now), [0.0] * len(now)) if n > 1 else run_step(sched, out)
+            live = [s for s in live if s.request.status is Status.RUNNING]
+            if len(live) < len(now):
+                ran = k + 1
+                break
+        cache.mark_issued([(s.request.request_id, s.start, s.num_tokens if n == 1 else ran) for s in out.scheduled
+                           if s.request.request_id in cache.requests])
+        cache.check()
+    assert not sched.has_work() and not todo
+    assert len(finished) == 14 and all(r.finish_reason in ("length", "max_seq_len") for r in finished), \
+        [(r.request_id, r.finish_reason) for r in finished]
+    assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups) and cache.slots.num_free == slots

@@ -79,6 +79,14 @@ def test_static_scratch_equals_workspace(window):
             want, got = run_both(lib, case, H, Kh, hd, page, window, max_len, num_splits, workspace)
             assert torch.isfinite(want.float()).all() and want.float().abs().max() > 0
             assert torch.equal(want, got), (num_splits, max_len, (want.float() - got.float()).abs().max().item())
+            # ... and both against the plain torch attention over the same pages (a fault that the two entry points
+            # shared would pass the comparison above): within two bfloat16 steps at each row's largest value
+            import torch_ops
+            q, k_pages, v_pages, table, meta = case
+            plain = torch_ops.paged_attention(q, k_pages, v_pages, table, meta[:, 0].contiguous(), meta[:, 3].contiguous(), H,
+                                              window=window or None, soft_cap=50.0).float()
+            bound = 2 * torch.exp2(torch.floor(torch.log2(plain.abs().amax(dim=-1, keepdim=True))) - 7)
+            assert ((got.float() - plain).abs() <= bound).all(), (num_splits, max_len)
 
 
 def test_static_scratch_refuses_what_does_not_fit():

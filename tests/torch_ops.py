@@ -74,12 +74,12 @@ def rope_cache_write(qkv, positions, timescale, scale_factor, q_div, num_heads, 
     q = q / q_div
     qkv[:, :H * hd] = q.reshape(T, H * hd).to(qkv.dtype)
     if k_pages is not None:
-        from simply_amd.kernels.packing import keys_to_rows, rows_to_keys
         P = k_pages.shape[2]
         page, off = slot_mapping[:T] // P, slot_mapping[:T] % P
-        rows = keys_to_rows(k_pages)      # the kernels' storage order of keys -> row-major, and back
-        rows[page, :, off] = k.to(k_pages.dtype)
-        k_pages.copy_(rows_to_keys(rows))
+        # element d of the key goes where the layout of a stored page puts it (key_element_index below)
+        at = key_element_index(P, hd, off[:, None], torch.arange(hd, device=off.device)[None, :])    # [T, hd]
+        flat = k_pages.view(k_pages.shape[0], K, P * hd)
+        flat[page[:, None, None], torch.arange(K, device=off.device)[None, :, None], at[:, None, :]] = k.to(k_pages.dtype)
         v_pages[page, :, :, off] = v.to(v_pages.dtype)     # value pages are [page, head, hd, page_size]
     return qkv
 
@@ -137,12 +137,43 @@ def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shap
     return c
 
 
+def key_element_index(P: int, hd: int, key: torch.Tensor, d: torch.Tensor) -> torch.Tensor:
+    """Where element d of key `key` (its offset inside a page) lies in a stored page of keys, by the layout's own
+    definition (simply_amd/csrc/api.h, sa_paged_attention): row-major [P][hd], unless P % 16 == 0 and hd % 32 == 0;
+    then in blocks of 16 keys x 32 dimensions, block (key // 16, d // 32) a contiguous 512 elements holding element
+    [(d % 32) // 8 * 16 + key % 16][d % 8] of a [64][8] array, the blocks of a group of 16 keys one after the other.
+    (Index arithmetic of the test's own: the product's re-layout functions are not used.)"""
+    if P % 16 or hd % 32:
+        return key * hd + d
+    block = (key // 16) * (hd // 32) + d // 32
+    return block * 512 + ((d % 32) // 8 * 16 + key % 16) * 8 + d % 8
+
+
+def stored_keys_as_rows(k_pages: torch.Tensor) -> torch.Tensor:
+    """Pages of keys as the kernels store them [pages, heads, P, hd] -> row-major [pages, heads, P, hd]."""
+    n, Kh, P, hd = k_pages.shape
+    key = torch.arange(P, device=k_pages.device)[:, None].expand(P, hd)
+    d = torch.arange(hd, device=k_pages.device)[None, :].expand(P, hd)
+    index = key_element_index(P, hd, key, d).reshape(-1)
+    return k_pages.reshape(n, Kh, P * hd)[:, :, index].reshape(n, Kh, P, hd)
+
+
+def rows_as_stored_keys(rows: torch.Tensor) -> torch.Tensor:
+    """Row-major pages of keys [pages, heads, P, hd] -> the kernels' storage order (same shape)."""
+    n, Kh, P, hd = rows.shape
+    key = torch.arange(P, device=rows.device)[:, None].expand(P, hd)
+    d = torch.arange(hd, device=rows.device)[None, :].expand(P, hd)
+    index = key_element_index(P, hd, key, d).reshape(-1)
+    out = torch.empty_like(rows).reshape(n, Kh, P * hd)
+    out[:, :, index] = rows.reshape(n, Kh, P * hd)
+    return out.reshape(n, Kh, P, hd)
+
+
 def paged_attention(q, k_pages, v_pages, block_table, token_seq, positions, num_heads, *, window, soft_cap, out=None,
                     algo=0):
-    from simply_amd.kernels.packing import keys_to_rows
     T = q.shape[0]
     _, Kh, P, hd = k_pages.shape
-    k_pages = keys_to_rows(k_pages)
+    k_pages = stored_keys_as_rows(k_pages)
     H = num_heads
     G = H // Kh
     res = torch.empty((T, H * hd), dtype=q.dtype, device=q.device)
