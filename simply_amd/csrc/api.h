@@ -138,8 +138,10 @@ int sa_paged_attention(const void* q, int dtype, int64_t q_stride, const void* k
 // The same attention for requests seq_begin .. seq_begin + seq_count - 1 of seq_meta (int32 [S, 4]: block-table
 // row, index of the request's first token in this step, number of its tokens, position of its first token), each
 // with (query heads per key head) * tokens <= 16: bfloat16, head size 64, 128 or 256, page size a multiple of 16.
-// max_kv_len bounds the keys of any of them (for the choice of how many ways to cut the keys; num_splits > 0 fixes
-// it).  workspace (bytes): scratch memory for the partial results of the key ranges.
+// max_kv_len bounds the keys of any of them: it is what the cut of the keys into ranges is planned for (num_splits > 0
+// fixes the number of ranges).  A request with more keys than that is still computed in full, only slower (its
+// ranges are longer than planned; a range of more than 32768 keys is worked through in several passes).
+// workspace (bytes): scratch memory for the partial results of the key ranges.
 int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                               const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
                               int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,

@@ -72,21 +72,30 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   const int tb = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * split / num_splits);
   const int te = tile0 + static_cast<int>(static_cast<int64_t>(ntiles) * (split + 1) / num_splits);
 
-  // Where every sub-tile of 16 keys of the range lies: looked up here once, so that the loop below has no load
-  // whose address depends on another load.  (A sub-tile lies within one page: page_size is a multiple of 16.)
-  const int sub0 = 2 * tb;
-  const int nsub = 2 * (te - tb) < kMaxRangeSubTiles ? 2 * (te - tb) : kMaxRangeSubTiles;  // (the host has seen to it)
-  for (int i = tid; i < nsub; i += 256) {
-    const int key = (sub0 + i) * 16;
-    int2 w = {0, 0};
-    if (key < hi && key + 16 > lo) {
-      const int block = key / page_size;
-      w.x = table[block];
-      w.y = (key - block * page_size) / 16;
+  // Where every sub-tile of 16 keys of the range lies is looked up once per pass, into LDS, so that the loop below
+  // has no load whose address depends on another load.  (A sub-tile lies within one page: page_size is a multiple
+  // of 16.)  The host cuts the keys so that a range fits one pass; a range that is longer all the same (a caller
+  // that understates max_kv_len) takes further passes, each with its own look-up, instead of reading beyond the
+  // array.
+  constexpr int kPassTiles = kMaxRangeSubTiles / 2;
+  int pass_b = tb;                                        // this pass covers tiles [pass_b, pass_e)
+  int pass_e = te - tb > kPassTiles ? tb + kPassTiles : te;
+  int sub0 = 2 * pass_b;
+  auto look_up = [&]() {
+    const int nsub = 2 * (pass_e - pass_b);
+    for (int i = tid; i < nsub; i += 256) {
+      const int key = (sub0 + i) * 16;
+      int2 w = {0, 0};
+      if (key < hi && key + 16 > lo) {
+        const int block = key / page_size;
+        w.x = table[block];
+        w.y = (key - block * page_size) / 16;
+      }
+      where_s[i] = w;
     }
-    where_s[i] = w;
-  }
-  __syncthreads();
+    __syncthreads();
+  };
+  look_up();
 
   // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
   bf16x8 qf[NDC];
@@ -115,7 +124,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   auto locate = [&](int tile, int t) {
     SubTile st;
     const int sk0 = tile * kTile + t * 16;
-    st.ok = tile < te && sk0 < hi && sk0 + 16 > lo;  // wave-uniform
+    st.ok = tile < pass_e && sk0 < hi && sk0 + 16 > lo;  // wave-uniform
     // A sub-tile outside the range is loaded all the same, from the pool's first page: every load of the loop is
     // unconditional, the loop straight-line code, and the compiler counts the loads in flight (with a branch
     // around a load it waits for all of them, and loads and products do not overlap).  What is loaded there is
@@ -224,14 +233,22 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   };
 
   TileRegs A, B;
-  int tile = tb + wave;
-  request_keys(A, tile);
-  request_values(A);
-  request_keys(B, tile + 4);
-  request_values(B);
-  for (; tile < te; tile += 8) {
-    process(A, tile, tile + 8);
-    if (tile + 4 < te) process(B, tile + 4, tile + 12);
+  for (;;) {
+    int tile = pass_b + wave;
+    request_keys(A, tile);
+    request_values(A);
+    request_keys(B, tile + 4);
+    request_values(B);
+    for (; tile < pass_e; tile += 8) {
+      process(A, tile, tile + 8);
+      if (tile + 4 < pass_e) process(B, tile + 4, tile + 12);
+    }
+    if (pass_e >= te) break;  // (the usual case: one pass)
+    __syncthreads();          // every wave has done with this pass's look-ups
+    pass_b = pass_e;
+    pass_e = te - pass_b > kPassTiles ? pass_b + kPassTiles : te;
+    sub0 = 2 * pass_b;
+    look_up();
   }
 
   // ---- merge the four waves in two rounds through LDS (waves 2, 3 into 0, 1; then 1 into 0).
@@ -427,11 +444,8 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   int KS = paged_attention_decode_ranges(seq_count, Kh, window, max_kv_len, num_splits);
   const size_t per_split = static_cast<size_t>(units) * 16 * (hd + kRowExtra) * sizeof(float);
   while (KS > 1 && (workspace == nullptr || per_split * KS > workspace_bytes)) --KS;
-  if (2 * ((decode_max_tiles(window, max_kv_len) + KS - 1) / KS + 1) > kMaxRangeSubTiles) {
-    set_error("paged_attention_decode: %d keys in %d ranges are more than %d keys per range; the workspace of %zu bytes "
-              "holds no more ranges", max_kv_len, KS, kMaxRangeSubTiles * 16, workspace_bytes);
-    return 1;
-  }
+  // (ranges of more than kMaxRangeSubTiles sub-tiles, which a small workspace or a caller's own num_splits may
+  // leave, take several passes inside the kernel)
   const dim3 grid(KS, Kh, seq_count);
   const bf16* qp = static_cast<const bf16*>(q);
   const bf16* kp = static_cast<const bf16*>(k_pages);

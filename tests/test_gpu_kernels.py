@@ -408,6 +408,35 @@ def test_paged_attention_decode(H, Kh, hd, P, window, cap, splits):
     assert (out2[:a] == 7).all() and (out2[b:] == 7).all()
 
 
+@pytest.mark.parametrize("stated", [40000, 700])
+def test_paged_attention_decode_with_a_range_longer_than_one_look_up(stated):
+    """One range of 40,000 keys (more than the 32,768 whose pages a workgroup looks up at a time), and a caller that
+    understates the longest context: the kernel works through the range in passes and reads every key."""
+    from simply_amd.kernels import ops
+    H, Kh, hd, P, L = 2, 1, 64, 16, 40000
+    kp, vp, table = paged_setup(torch.bfloat16, 1, H, Kh, hd, P, [L], 77)
+    q = rand((1, H * hd), torch.bfloat16, 78, 0.5)
+    meta = torch.tensor([[0, 0, 1, L - 1]], dtype=torch.int32).cuda()
+    out = torch.zeros((1, H * hd), dtype=torch.bfloat16).cuda()
+    ops.paged_attention_decode(q, kp, vp, table, meta, 0, 1, H, window=None, soft_cap=30.0, max_kv_len=stated, max_q_len=1,
+                               out=out, num_splits=1)
+    want = ref.paged_attention(q, kp, vp, table, torch.zeros(1, dtype=torch.int32).cuda(),
+                               torch.tensor([L - 1], dtype=torch.int32).cuda(), H, window=None, soft_cap=30.0)
+    check(out.float(), want.float(), bf16_steps=2.0)
+    # a key in the second pass that stands out is found
+    rows = ref.stored_keys_as_rows(kp) * 0.01
+    far = 36000
+    page, off = int(table[0, far // P]), far % P
+    rows[page, 0, off] = 0.0
+    rows[page, 0, off, 5] = 60.0
+    vp[page, 0, :, off] = 9.0
+    q2 = torch.zeros((1, H * hd), dtype=torch.bfloat16).cuda()
+    q2[0, 5] = q2[0, hd + 5] = 1.0
+    ops.paged_attention_decode(q2, ref.rows_as_stored_keys(rows), vp, table, meta, 0, 1, H, window=None, soft_cap=None,
+                               max_kv_len=stated, max_q_len=1, out=out, num_splits=1)
+    assert abs(out.float().mean().item() - 9.0) < 0.1, out.float().mean().item()
+
+
 def test_paged_attention_decode_far_key():
     """A key 3000 positions back with a score that stands out, among keys cut over many workgroups."""
     from simply_amd.kernels import ops
