@@ -238,6 +238,67 @@ def run_requests(model, cfg, requests, prompt_min, prompt_max, new_tokens, page_
     return dt, sum(lengths), requests * new_tokens, stats
 
 
+def run_products(which: str):
+    """Times of the three bfloat16 product kernels (few-rows, tiled, wide) and of the library's own choice, for 1 to 64
+    rows against weights of many sizes streamed from HBM (several copies of a weight in turn, so that no cache holds
+    them), beside the times that the library expects: one JSON line per size and number of rows.  This is the sweep
+    that the kernels' time models (`sa_gemm_plan`) are fitted to and judged by."""
+    import torch
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.packing import pack_gate_up, pack_tiles
+
+    def graph_time(fs, reps=8):
+        for f in fs:
+            f()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for f in fs:
+                f()
+        g.replay()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            g.replay()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / reps / len(fs) * 1e3
+
+    # q/k/v, output and down projections of the 2B, 9B and 27B sizes, sizes of no model, the head; gated: the three
+    # feed-forwards and two sizes of no model
+    plain = [(4096, 2304), (2304, 2048), (2304, 9216), (8192, 3584), (3584, 4096), (3584, 14336), (8192, 4608),
+             (4608, 4096), (4608, 36864), (3072, 3072), (5120, 8192), (1024, 1024), (11008, 4096), (2048, 16384),
+             (256000, 2304)]
+    gated = [(9216, 2304), (14336, 3584), (36864, 4608), (8192, 3072), (4096, 1024)]
+    names = {ops.ALGO_SKINNY: "skinny", ops.ALGO_TILED: "tiled", ops.ALGO_WIDE: "wide"}
+    for (N, K) in (gated if which == "gated" else plain):
+        nbytes = N * K * 2 * (2 if which == "gated" else 1)
+        copies = max(1, min(12, -(-(700 << 20) // nbytes)))
+        ws = []
+        for _ in range(copies):
+            w = (torch.randn(N, K, device="cuda") * 0.03).to(torch.bfloat16)
+            ws.append(pack_gate_up(w, (torch.randn(N, K, device="cuda") * 0.03).to(torch.bfloat16))
+                      if which == "gated" else pack_tiles(w))
+            del w
+        for M in (1, 2, 4, 8, 9, 12, 16, 17, 24, 32, 48, 64):
+            a = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+            out = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            res = {}
+            for name, algo in (("skinny", ops.ALGO_SKINNY), ("tiled", ops.ALGO_TILED), ("wide", ops.ALGO_WIDE),
+                               ("chosen", ops.ALGO_AUTO)):
+                try:
+                    fs = [(lambda w=w: ops.gemm(a, w, out=out, algo=algo)) for w in ws]
+                    res[name] = round(graph_time(fs * (2 if copies < 4 else 1)), 2)
+                except ops.KernelError:
+                    res[name] = None
+            kernel, expected = ops.gemm_plan(M, N, K, gated=which == "gated")
+            print(json.dumps({"product": which, "M": M, "N": N, "K": K, "us": res, "choice": names.get(kernel),
+                              "expected_us": {k: round(v, 1) for k, v in expected.items()}}), flush=True)
+        del ws
+        torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -250,8 +311,10 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prefill-chunked"],
-                    help="measure one part alone (for profiles); the line then holds that part only")
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prefill-chunked", "products",
+                                                      "gated-products"],
+                    help="measure one part alone (for profiles); the line then holds that part only.  products / "
+                         "gated-products: the sweep of the product kernels over rows and weight sizes")
     ap.add_argument("--latency-steps", type=int, default=100,
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
@@ -271,6 +334,9 @@ def main():
     from simply_amd.kernels import lib
 
     lib.load()
+    if args.only in ("products", "gated-products"):
+        run_products("gated" if args.only == "gated-products" else "plain")
+        return
     d = dict(GEMMA2_2B, **SHAPES[args.shape])
     full_layers = d["num_hidden_layers"]
     if args.layers:

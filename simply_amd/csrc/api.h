@@ -92,6 +92,11 @@ int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* 
 // == 1: C holds the product as after sa_gemm.
 // C = the sum of `count` planes [M][N] float32 in their order, rounded to C's type: the kernel that sa_gemm_planes
 // leaves out.
+// Which kernel sa_gemm would run for bfloat16 operands of these sizes with tiled weights and 16-byte aligned
+// operands (2: few-rows, 3: tiled, 4: wide), and, in us[0..2] if it is not null, the microseconds that the library
+// expects of the three (negative: not eligible).  c_dtype is the output's element type (the wide kernel writes
+// bfloat16 only).  A host function: nothing is launched.
+int sa_gemm_plan(int M, int N, int K, int epilogue, int c_dtype, int64_t workspace_bytes, double* us);
 int sa_sum_planes(const float* planes, int count, void* C, int c_dtype, int64_t ldc, int M, int N, hipStream_t stream);
 int sa_gemm_planes(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
                    int c_dtype, int64_t ldc, int M, int N, int K, int epilogue, float cap, int algo, int packed,
@@ -202,6 +207,12 @@ int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const v
                  int c_dtype, int64_t ldc, int M, int N, int K, int epi, int act, float cap, int packed,
                  hipStream_t stream);
 bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2);
+// Expected microseconds of each bfloat16 product kernel for these sizes (epi: 0 none, 1 gated, 2 soft-cap); negative:
+// the kernel is not made for them.  The dispatcher runs the kernel with the smallest figure among those that take
+// the arguments.
+double gemm_skinny_predict_us(int M, int N, int K, int epi);
+double gemm_tiled_predict_us(int M, int N, int K, int epi);
+double gemm_wide_predict_us(int M, int N, int K, int epi, bool have_workspace, size_t workspace_bytes);
 int gemm_skinny(const void* A, int64_t lda, const void* W, const void* W2, void* C, int c_dtype, int64_t ldc, int M,
                 int N, int K, int epi, int act, float cap, int packed, int shape, hipStream_t stream);
 bool paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q);

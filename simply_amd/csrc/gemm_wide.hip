@@ -292,6 +292,81 @@ bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* 
          static_cast<int64_t>(M) * lda < (int64_t{1} << 31);  // byte offsets of rows are kept in 32 bits
 }
 
+// The tile and the cut of K for a product whose caller fixes neither, and the time that this kernel is expected to
+// take with them in microseconds (the figure by which the library chooses between its product kernels).
+static double plan_shape(int M, int N, int K, int epi, bool have_workspace, size_t workspace_bytes, int& shape, int& ks) {
+  const int NW_all = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
+  // without a fitted model below: the weights streamed once at the rate this kernel reaches for few rows, or the
+  // products at its rate for many, whichever takes longer, after its start
+  double us = 5.0 + 0.02 * (M < 64 ? M : 64) +
+              fmax(2.0 * NW_all * K / 5.8e6, static_cast<double>(M) * NW_all * K / (1.05e9 / 2));
+  // The cost of a shape: the workgroups that the busiest CU gets times the size of the tile; of equals the first.
+  // Workgroups of four waves run two to a CU, where one's epilogue and first loads overlap the other's
+  // products (measured: 7-9 % faster than one workgroup of twice the tile once every CU has two of them;
+  // slower when it has one; from one and a half per CU on it is also the best for few rows of very many weight
+  // rows, which are bound by streaming them).
+  const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
+  const int shapes[5][4] = {{2128192, 128, 192, 93}, {2256192, 256, 192, 100}, {3256128, 256, 128, 100},
+                            {3128256, 128, 256, 100}, {3192128, 192, 128, 100}};
+  int64_t best = -1;
+  for (const auto& sh : shapes) {
+    const int64_t tiles = static_cast<int64_t>((M + sh[1] - 1) / sh[1]) * ((NW + sh[2] - 1) / sh[2]);
+    if (sh[3] < 100 && tiles < wide::kCUs * 3 / 2) continue;
+    const int64_t cost = ((tiles + wide::kCUs - 1) / wide::kCUs) * sh[1] * sh[2] * sh[3];
+    if (best < 0 || cost < best) {
+      best = cost;
+      shape = sh[0];
+    }
+  }
+  // A gated product of few rows whose tiles of 128 weight rows make one round at most (the 2B and 9B feed-forward
+  // for up to 128 decoding requests) streams its weights: rows of 64 (or 128) with the deepest pipeline that fits
+  // are 5 to 25 % faster there than the large tiles (2B at 64 rows: 23 against 28 us; 9B: 39 against 48).
+  if (epi == 1 && M <= 128) {
+    const int rows = M <= 64 ? 64 : 128;
+    if (static_cast<int64_t>((M + rows - 1) / rows) * ((NW + 127) / 128) <= wide::kCUs) shape = M <= 64 ? 6064128 : 3128128;
+  }
+  // 17 to 1,536 rows without an epilogue (portions of prompts, many decoding requests): the tiles above are too few
+  // for 256 CUs, and every workgroup walks all of K at the pace of its own slabs.  Smaller tiles with deeper
+  // pipelines, and K cut over workgroups so that about one round of them covers the GPU, chosen by a model of the
+  // time fitted to measurements at the 2B, 9B and 27B sizes (64 to 2,048 rows, seven tiles, one to fourteen cuts;
+  // it is within 6 % of the best measured choice nearly everywhere, and a fifth faster in sum than either the
+  // uncut tiles above or the tiled kernel with its cut: the 2B down projection at 512 rows takes 36 us against 55).
+  if (epi == 0 && M <= 1536) {  // (fewer than 17 rows come here only against a very long K)
+    struct Tile { int code, rows, wrows; double eff, start; };  // share of the MFMA rate in the loop; us to start
+    static const Tile tiles[7] = {{3128128, 128, 128, 0.425, 1.44}, {3128256, 128, 256, 0.535, 2.03},
+                                  {3192128, 192, 128, 0.535, 1.25}, {3256128, 256, 128, 0.615, 1.58},
+                                  {5128064, 128, 64, 0.326, 0.85},  {6064064, 64, 64, 0.234, 0.80},
+                                  {6064128, 64, 128, 0.277, 1.08}};
+    const int slabs = K / wide::BK;
+    double best_us = -1.0;
+    int best_ks = 1;
+    for (const Tile& t : tiles) {
+      const int64_t count = static_cast<int64_t>((M + t.rows - 1) / t.rows) * ((N + t.wrows - 1) / t.wrows);
+      const int cuts[3] = {1, static_cast<int>(wide::kCUs / count), static_cast<int>(2 * wide::kCUs / count)};
+      for (int c = 0; c < 3; ++c) {
+        const int cut = cuts[c];
+        if (cut < 1 || (c > 0 && (cut < 2 || cut == cuts[c - 1])) || cut > slabs / 4) continue;
+        const double partial_bytes = static_cast<double>(cut) * M * N * 4;
+        if (cut > 1 && (!have_workspace || partial_bytes > static_cast<double>(workspace_bytes))) continue;
+        const int64_t rounds = (count * cut + wide::kCUs - 1) / wide::kCUs;
+        const int per = (slabs + cut - 1) / cut;
+        // a CU's MFMA rate: 4.9 M multiply-adds of bfloat16 a microsecond
+        double us = rounds * (static_cast<double>(per) * t.rows * t.wrows * wide::BK / (4.9e6 * t.eff) + t.start) + 3.2;
+        if (cut > 1) us += partial_bytes / 5.5e6 + partial_bytes / 4.9e6 + 3.7;  // written, read again, the sum kernel
+        if (best_us < 0 || us < best_us) {
+          best_us = us;
+          shape = t.code;
+          best_ks = cut;
+        }
+      }
+    }
+    if (ks == 1) ks = best_ks;
+    // (the model of the tiles knows nothing of memory: the weights streamed once from HBM are a floor under it)
+    if (best_us >= 0) us = fmax(best_us, 5.0 + 0.02 * (M < 64 ? M : 64) + 2.0 * NW_all * K / 5.8e6);
+  }
+  return us;
+}
+
 // shape: 0: chosen here; else stages * 1000000 + rows * 1000 + weight rows of a workgroup's tile (2256192, 3256128,
 // 3128256, 3192128; 2128192: workgroups of four waves, two to a CU).
 // ks > 1 cuts K over that many workgroups per tile (no epilogue only; the partial tiles go through `workspace`,
@@ -308,70 +383,7 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
   const bf16* a = static_cast<const bf16*>(A);
   const bf16* w = static_cast<const bf16*>(W);
   bf16* c = static_cast<bf16*>(C);
-  if (shape == 0) {
-    // The cost of a shape: the workgroups that the busiest CU gets times the size of the tile; of equals the first.
-    // Workgroups of four waves run two to a CU, where one's epilogue and first loads overlap the other's
-    // products (measured: 7-9 % faster than one workgroup of twice the tile once every CU has two of them;
-    // slower when it has one; from one and a half per CU on it is also the best for few rows of very many weight
-    // rows, which are bound by streaming them).
-    const int NW = epi == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-    const int shapes[5][4] = {{2128192, 128, 192, 93}, {2256192, 256, 192, 100}, {3256128, 256, 128, 100},
-                              {3128256, 128, 256, 100}, {3192128, 192, 128, 100}};
-    int64_t best = -1;
-    for (const auto& sh : shapes) {
-      const int64_t tiles = static_cast<int64_t>((M + sh[1] - 1) / sh[1]) * ((NW + sh[2] - 1) / sh[2]);
-      if (sh[3] < 100 && tiles < wide::kCUs * 3 / 2) continue;
-      const int64_t cost = ((tiles + wide::kCUs - 1) / wide::kCUs) * sh[1] * sh[2] * sh[3];
-      if (best < 0 || cost < best) {
-        best = cost;
-        shape = sh[0];
-      }
-    }
-    // A gated product of few rows whose tiles of 128 weight rows make one round at most (the 2B and 9B feed-forward
-    // for up to 128 decoding requests) streams its weights: rows of 64 (or 128) with the deepest pipeline that fits
-    // are 5 to 25 % faster there than the large tiles (2B at 64 rows: 23 against 28 us; 9B: 39 against 48).
-    if (epi == 1 && M <= 128) {
-      const int rows = M <= 64 ? 64 : 128;
-      if (static_cast<int64_t>((M + rows - 1) / rows) * ((NW + 127) / 128) <= wide::kCUs) shape = M <= 64 ? 6064128 : 3128128;
-    }
-    // 17 to 1,536 rows without an epilogue (portions of prompts, many decoding requests): the tiles above are too few
-    // for 256 CUs, and every workgroup walks all of K at the pace of its own slabs.  Smaller tiles with deeper
-    // pipelines, and K cut over workgroups so that about one round of them covers the GPU, chosen by a model of the
-    // time fitted to measurements at the 2B, 9B and 27B sizes (64 to 2,048 rows, seven tiles, one to fourteen cuts;
-    // it is within 6 % of the best measured choice nearly everywhere, and a fifth faster in sum than either the
-    // uncut tiles above or the tiled kernel with its cut: the 2B down projection at 512 rows takes 36 us against 55).
-    if (epi == 0 && M <= 1536) {  // (fewer than 17 rows come here only against a very long K)
-      struct Tile { int code, rows, wrows; double eff, start; };  // share of the MFMA rate in the loop; us to start
-      static const Tile tiles[7] = {{3128128, 128, 128, 0.425, 1.44}, {3128256, 128, 256, 0.535, 2.03},
-                                    {3192128, 192, 128, 0.535, 1.25}, {3256128, 256, 128, 0.615, 1.58},
-                                    {5128064, 128, 64, 0.326, 0.85},  {6064064, 64, 64, 0.234, 0.80},
-                                    {6064128, 64, 128, 0.277, 1.08}};
-      const int slabs = K / wide::BK;
-      double best_us = -1.0;
-      int best_ks = 1;
-      for (const Tile& t : tiles) {
-        const int64_t count = static_cast<int64_t>((M + t.rows - 1) / t.rows) * ((N + t.wrows - 1) / t.wrows);
-        const int cuts[3] = {1, static_cast<int>(wide::kCUs / count), static_cast<int>(2 * wide::kCUs / count)};
-        for (int c = 0; c < 3; ++c) {
-          const int cut = cuts[c];
-          if (cut < 1 || (c > 0 && (cut < 2 || cut == cuts[c - 1])) || cut > slabs / 4) continue;
-          const double partial_bytes = static_cast<double>(cut) * M * N * 4;
-          if (cut > 1 && (ws == nullptr || partial_bytes > static_cast<double>(workspace_bytes))) continue;
-          const int64_t rounds = (count * cut + wide::kCUs - 1) / wide::kCUs;
-          const int per = (slabs + cut - 1) / cut;
-          // a CU's MFMA rate: 4.9 M multiply-adds of bfloat16 a microsecond
-          double us = rounds * (static_cast<double>(per) * t.rows * t.wrows * wide::BK / (4.9e6 * t.eff) + t.start) + 3.2;
-          if (cut > 1) us += partial_bytes / 5.5e6 + partial_bytes / 4.9e6 + 3.7;  // written, read again, the sum kernel
-          if (best_us < 0 || us < best_us) {
-            best_us = us;
-            shape = t.code;
-            best_ks = cut;
-          }
-        }
-      }
-      if (ks == 1) ks = best_ks;
-    }
-  }
+  if (shape == 0) plan_shape(M, N, K, epi, ws != nullptr, workspace_bytes, shape, ks);
   switch (shape) {
     case 2256192: wide::launch<4, 6, 4, 2>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
     case 3256128: wide::launch<4, 4, 4, 3>(a, lda, w, c, ldc, M, N, K, epi, act, ks, ws, stream); break;
@@ -399,6 +411,12 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
   }
   if (ks > 1) return gemm_sum_partials(ws, ks, C, kBF16, ldc, M, N, N, 0, 0, 0.f, stream);
   return 0;
+}
+
+
+double gemm_wide_predict_us(int M, int N, int K, int epi, bool have_workspace, size_t workspace_bytes) {
+  int shape = 0, ks = 1;
+  return plan_shape(M, N, K, epi, have_workspace, workspace_bytes, shape, ks);
 }
 
 }  // namespace sa

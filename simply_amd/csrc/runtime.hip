@@ -50,66 +50,45 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
   SA_REQUIRE(algo >= 0 && algo <= 4, "gemm: unknown algorithm %d", algo);
   const bool bf16_in = a_dtype == kBF16 && w_dtype == kBF16;
-  // up to 16 rows, and up to 32 for products without the gated epilogue and with K below 4096 (measured at the
-  // 2B, 9B and 27B sizes: the few-rows kernel, whose waves read the activations from L2, beats the kernels with
-  // K cut over workgroups there; for longer K, the down projections, it is up to 2x slower).  Not from 8 rows on
-  // against so many weight rows that the tiled kernel fills the GPU without a cut of K (the head over a large
-  // vocabulary: 7 % faster at 8 rows, 30 % at 16, 80 % at 32; up to 6 rows the few-rows kernel wins).
-  // Nor against a very long K (the 27B down projection, 36864: kernels that cut K over workgroups are 15 % faster at
-  // one row and 40 % at 16), nor from 9 rows on against K of 8192 and more (the 2B and 9B down projections: the
-  // wide kernel with its cut takes 13.0 against 16.8 us and 24.2 against 26.7 at 16 rows; up to 8 rows, where a
-  // load of activations serves several chunks of K, the few-rows kernel wins).
-  const bool many_weight_rows = packed && epilogue != 1 && M >= 8 && N >= 65536;
-  const bool long_k = packed && epilogue != 1 && K >= 24576;
-  // (... or against K of 4096 and more where the weight is large, 16 M elements: 27B q/k/v 16.0 against 18.6 us at
-  // 16 rows; the same size decides for 17 to 32 rows: 9B q/k/v 16.0 against 22.5 us at 32 rows with the wide kernel,
-  // 2B q/k/v 9.5 against 9.8 with the few-rows kernel)
-  const bool large = static_cast<int64_t>(N) * K >= (int64_t{16} << 20);
-  const bool longish_k = packed && epilogue == 0 && M >= 9 && N <= 16384 && (K >= 8192 || (K >= 4096 && large));
-  const bool tiled_first = many_weight_rows || long_k;
-  if (algo == 2 ||
-      (algo == 0 && bf16_in && !tiled_first && !longish_k &&
-       (M <= 16 || (M <= 32 && epilogue != 1 && K < 4096 && !(packed && epilogue == 0 && large && N <= 16384))))) {
-    const bool takes = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
-    SA_REQUIRE(takes || algo == 0,
-               "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
-               "operands; got M=%d K=%d lda=%lld", M, K, (long long)lda);
-    if (takes)
-      return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, shape, stream);
+  const size_t ws_bytes = static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes);
+  // Which of the three bfloat16 kernels take these arguments; a kernel that the caller names must take them.
+  const bool skinny_ok = bf16_in && gemm_skinny_takes(M, N, K, lda, A, W, W2);
+  const bool wide_ok = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
+  const bool tiled_ok = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
+  SA_REQUIRE(algo != 2 || skinny_ok,
+             "gemm: the few-rows kernel takes bfloat16 with M <= 64, K and lda multiples of 8 and 16-byte aligned "
+             "operands; got M=%d K=%d lda=%lld", M, K, (long long)lda);
+  SA_REQUIRE(algo != 4 || wide_ok,
+             "gemm: the wide MFMA kernel takes bfloat16 in and out with tiled weights, no soft-cap, K a multiple of "
+             "64, N and ldc of 4, lda of 8; got N=%d K=%d lda=%lld ldc=%lld tiled=%d", N, K, (long long)lda,
+             (long long)ldc, packed);
+  SA_REQUIRE(algo != 3 || tiled_ok,
+             "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
+             "aligned operands; got K=%d lda=%lld tiled=%d", K, (long long)lda, packed);
+  int kernel = algo;
+  if (algo == 0) {
+    // The kernel that is expected to be fastest: every kernel says how long it expects to take for these sizes (a
+    // model of its own time, fitted to measurements, beside its code), and the smallest figure wins.  No size of any
+    // model stands here.
+    kernel = 1;
+    double best = -1.0;
+    const double us[3] = {skinny_ok ? gemm_skinny_predict_us(M, N, K, epilogue) : -1.0,
+                          tiled_ok ? gemm_tiled_predict_us(M, N, K, epilogue) : -1.0,
+                          wide_ok ? gemm_wide_predict_us(M, N, K, epilogue, workspace != nullptr, ws_bytes) : -1.0};
+    for (int i = 0; i < 3; ++i)
+      if (us[i] >= 0.0 && (best < 0.0 || us[i] < best)) {
+        best = us[i];
+        kernel = 2 + i;
+      }
   }
-  // once the product is no longer bound by streaming the weights: the wide tiles (both operands through LDS); and
-  // the gated product from 17 rows on, whose very many weight rows fill the GPU with the wide kernel's workgroups
-  // without a cut of K (measured at 32 and 64 rows: 10-20 % faster than the tiled kernel with its sum kernel at the
-  // 2B, 9B and 27B sizes)
-  const int NW = epilogue == 1 ? 2 * ((N + 15) / 16) * 16 : N;
-  // 17 to 1,536 rows without an epilogue (q/k/v, output and down projections of portions of prompts and of many
-  // decoding requests): the wide kernel with a tile and a cut of K that it chooses for the sizes (2B down projection:
-  // 13 us at 17 rows, 15 at 64, 36 at 512, against 19, 23 and 55 for the tiled kernel with its cut)
-  // ... and up to 16 rows against a very long K (the 27B down projection: 62 us against 67 for the tiled kernel
-  // with its cut and 74 to 84 for the few-rows kernel)
-  const bool small_wide = epilogue == 0 && N <= 16384 && ((M >= 17 && M <= 1536) || (long_k && M <= 16) || longish_k);
-  const bool wide_first = !gemm_streams_weights(M, NW, K) || (epilogue == 1 && M > 16) || small_wide;
-  if (algo == 4 || (algo == 0 && bf16_in && packed && wide_first)) {
-    const bool takes = bf16_in && gemm_wide_takes(M, N, K, lda, ldc, A, W, W2, C, c_dtype, epilogue, packed);
-    SA_REQUIRE(takes || algo == 0,
-               "gemm: the wide MFMA kernel takes bfloat16 in and out with tiled weights, no soft-cap, K a multiple of "
-               "64, N and ldc of 4, lda of 8; got N=%d K=%d lda=%lld ldc=%lld tiled=%d", N, K, (long long)lda,
-               (long long)ldc, packed);
-    // (a shape given by the caller may carry a cut of K in front: cuts * 10000000 + shape)
-    if (takes)
-      return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape % 10000000 : 0,
-                       algo == 4 ? shape / 10000000 : 1, workspace,
-                       static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream, planes_left);
-  }
-  if (algo == 3 || (algo == 0 && bf16_in && packed && (M > 16 || tiled_first))) {
-    const bool takes = bf16_in && gemm_tiled_takes(M, N, K, lda, A, W, W2, packed);
-    SA_REQUIRE(takes || algo == 0,
-               "gemm: the tiled MFMA kernel takes bfloat16 with tiled weights, K and lda multiples of 8 and 16-byte "
-               "aligned operands; got K=%d lda=%lld tiled=%d", K, (long long)lda, packed);
-    if (takes)
-      return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, act, cap, shape, workspace,
-                        static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream);
-  }
+  if (kernel == 2)
+    return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, shape, stream);
+  // (a shape given by the caller for the wide kernel may carry a cut of K in front: cuts * 10000000 + shape)
+  if (kernel == 4)
+    return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape % 10000000 : 0,
+                     algo == 4 ? shape / 10000000 : 1, workspace, ws_bytes, stream, planes_left);
+  if (kernel == 3)
+    return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, act, cap, shape, workspace, ws_bytes, stream);
   return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, stream);
 }
 
@@ -118,6 +97,31 @@ extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, c
                        int packed, int shape, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   return gemm_routed(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, cap, algo, packed, shape,
                      workspace, workspace_bytes, nullptr, stream);
+}
+
+extern "C" int sa_gemm_plan(int M, int N, int K, int epilogue, int c_dtype, int64_t workspace_bytes, double* us_out) {
+  if (M < 1 || N < 1 || K < 1) return 0;
+  const int epi = epilogue_kind(epilogue);
+  const size_t ws_bytes = static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes);
+  alignas(16) static const char aligned_stand_in[16] = {};   // an address that every alignment test passes
+  const void* p = aligned_stand_in;
+  const int64_t lda = K, ldc = N;
+  const bool skinny_ok = gemm_skinny_takes(M, N, K, lda, p, p, nullptr);
+  const bool wide_ok = gemm_wide_takes(M, N, K, lda, ldc, p, p, nullptr, p, c_dtype, epi, 1);
+  const bool tiled_ok = gemm_tiled_takes(M, N, K, lda, p, p, nullptr, 1);
+  const double us[3] = {skinny_ok ? gemm_skinny_predict_us(M, N, K, epi) : -1.0,
+                        tiled_ok ? gemm_tiled_predict_us(M, N, K, epi) : -1.0,
+                        wide_ok ? gemm_wide_predict_us(M, N, K, epi, ws_bytes > 0, ws_bytes) : -1.0};
+  int kernel = 1;
+  double best = -1.0;
+  for (int i = 0; i < 3; ++i) {
+    if (us_out != nullptr) us_out[i] = us[i];
+    if (us[i] >= 0.0 && (best < 0.0 || us[i] < best)) {
+      best = us[i];
+      kernel = 2 + i;
+    }
+  }
+  return kernel;
 }
 
 extern "C" int sa_sum_planes(const float* planes, int count, void* C, int c_dtype, int64_t ldc, int M, int N,

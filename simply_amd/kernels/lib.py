@@ -88,6 +88,8 @@ def load() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes = args
             fn.restype = c_int
+        lib.sa_gemm_plan.argtypes = [_I, _I, _I, _I, _I, _L, _P]
+        lib.sa_gemm_plan.restype = c_int
         lib.sa_philox4x32_10.argtypes = [_P, _P, _P]
         lib.sa_philox4x32_10.restype = None
         _lib, _path = lib, path

@@ -416,6 +416,17 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
     return out
 
 
+def gemm_plan(M: int, N: int, K: int, *, gated: bool = False, soft_cap: bool = False,
+              out_dtype: torch.dtype = torch.bfloat16) -> tuple[int, dict[str, float]]:
+    """Which kernel `gemm` would run for bfloat16 rows against a tiled [N, K] weight (ALGO_SKINNY, ALGO_TILED or
+    ALGO_WIDE), and the microseconds that the library expects of each (negative: not eligible).  A host function:
+    it needs no GPU."""
+    us = (ctypes.c_double * 3)()
+    epi = EPILOGUE_GATED if gated else (EPILOGUE_SOFT_CAP if soft_cap else EPILOGUE_NONE)
+    kernel = _lib.load().sa_gemm_plan(int(M), int(N), int(K), epi, _CODES[out_dtype], WORKSPACE_BYTES, us)
+    return kernel, {"skinny": us[0], "tiled": us[1], "wide": us[2]}
+
+
 def gemm_normed_takes(M: int, w) -> bool:
     """Whether `gemm_normed` takes M rows against the weight `w`."""
     if not isinstance(w, TiledWeight) or not w.data.is_cuda:
