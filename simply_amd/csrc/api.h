@@ -27,6 +27,13 @@ int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, int w_post_dt
                    int plus_one_post, float* residual, const void* w_next, int w_next_dtype, float eps_next,
                    int plus_one_next, void* out, int out_dtype, int T, int D, hipStream_t stream);
 
+// For the rows index[0..R-1] only, and without storing the sum: out[r] = norm(residual[index[r]] + norm(y[index[r]];
+// w_post); w_next) (w_post null: + y as it is).  What a model's end needs: the rows whose logits are wanted.
+int sa_add_rmsnorm_rows(const void* y, int y_dtype, const void* w_post, int w_post_dtype, float eps_post,
+                        int plus_one_post, const float* residual, const void* w_next, int w_next_dtype, float eps_next,
+                        int plus_one_next, void* out, int out_dtype, const int* index, int R, int D,
+                        hipStream_t stream);
+
 // The same with y given as `planes` partial results [planes][T][D] float32 (sa_gemm_planes): y is their sum in the
 // order of the planes, rounded to bfloat16, as the sum kernel of the product would have left it.  D % 4 == 0.
 int sa_add_rmsnorm_planes(const float* y_planes, int planes, const void* w_post, int w_post_dtype, float eps_post,
@@ -64,6 +71,13 @@ int sa_fill_u32(void* p, uint32_t value, int64_t n, hipStream_t stream);
 int sa_decode_advance(int B, int* step_counter, const int* sampled_tokens, const float* sampled_logprobs,
                       int* tokens_in, int* positions, int* seq_meta, int* draw_counters, int* out_tokens,
                       float* out_logprobs, int max_steps, hipStream_t stream);
+// sa_decode_advance and, in the same launch, sa_decode_slots at the new positions for num_groups (at most 4) cache
+// groups: block_tables, table_strides and slot_mappings are host arrays of num_groups entries.
+int sa_decode_advance_slots(int B, int* step_counter, const int* sampled_tokens, const float* sampled_logprobs,
+                            int* tokens_in, int* positions, int* seq_meta, int* draw_counters, int* out_tokens,
+                            float* out_logprobs, int max_steps, const int* token_seq, int num_groups,
+                            const int* const* block_tables, const int* table_strides, int64_t* const* slot_mappings,
+                            int page_size, hipStream_t stream);
 // slot_mapping[b] = block_table[token_seq[b], positions[b] / page_size] * page_size + positions[b] % page_size
 int sa_decode_slots(int B, const int* positions, const int* token_seq, const int* block_table, int table_stride,
                     int page_size, int64_t* slot_mapping, hipStream_t stream);

@@ -55,9 +55,14 @@ constexpr int kRowRegs = 5;  // (1024 threads hold 5120: the width of the 27B sh
 __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, const void* __restrict__ w_post,
                                    int w_post_dtype, float eps_post, float plus_one_post, float* __restrict__ residual,
                                    const void* __restrict__ w_next, int w_next_dtype, float eps_next,
-                                   float plus_one_next, void* __restrict__ out, int out_dtype, int D) {
+                                   float plus_one_next, void* __restrict__ out, int out_dtype, int D,
+                                   const int* __restrict__ index) {
+  // index: block b works on row index[b] of y and of the residual, which it only reads, and writes row b of out
+  // (the rows whose logits are wanted, at a model's end: the other rows' sums are of no use to anyone)
   __shared__ float scratch[16];
-  const size_t rb = static_cast<size_t>(blockIdx.x) * D;
+  const size_t rb = static_cast<size_t>(index != nullptr ? index[blockIdx.x] : static_cast<int>(blockIdx.x)) * D;
+  const size_t ob = static_cast<size_t>(blockIdx.x) * D;
+  const bool keep = index == nullptr;  // the residual stream is updated
   if (D <= kRowRegs * static_cast<int>(blockDim.x)) {
     float yv[kRowRegs], hv[kRowRegs], wp[kRowRegs], wn[kRowRegs];
 #pragma unroll
@@ -84,7 +89,7 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
       const float v = w_post != nullptr ? yv[j] * r * wp[j] : yv[j];
       hv[j] += v;
       if (d < D) {
-        residual[rb + d] = hv[j];
+        if (keep) residual[rb + d] = hv[j];
         ss2 += hv[j] * hv[j];
       }
     }
@@ -94,7 +99,7 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
 #pragma unroll
     for (int j = 0; j < kRowRegs; ++j) {
       const int d = threadIdx.x + j * blockDim.x;
-      if (d < D) store_f(out, out_dtype, rb + d, hv[j] * r2 * wn[j]);
+      if (d < D) store_f(out, out_dtype, ob + d, hv[j] * r2 * wn[j]);
     }
     return;
   }
@@ -112,15 +117,20 @@ __global__ void add_rmsnorm_kernel(const void* __restrict__ y, int y_dtype, cons
     float v = load_f(y, y_dtype, rb + d);
     if (w_post != nullptr) v = v * r * (load_f(w_post, w_post_dtype, d) + plus_one_post);
     const float h = residual[rb + d] + v;
-    residual[rb + d] = h;  // re-read below by the same thread only
+    if (keep) residual[rb + d] = h;  // re-read below by the same thread only
     ss2 += h * h;
   }
   if (w_next == nullptr) return;
   ss2 = block_sum(ss2, scratch);
   const float r2 = rsqrtf(ss2 / static_cast<float>(D) + eps_next);
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    const float h = residual[rb + d] * r2;
-    store_f(out, out_dtype, rb + d, h * (load_f(w_next, w_next_dtype, d) + plus_one_next));
+    float h = residual[rb + d];
+    if (!keep) {  // the sum was not stored: made once more
+      float v = load_f(y, y_dtype, rb + d);
+      if (w_post != nullptr) v = v * r * (load_f(w_post, w_post_dtype, d) + plus_one_post);
+      h += v;
+    }
+    store_f(out, out_dtype, ob + d, h * r2 * (load_f(w_next, w_next_dtype, d) + plus_one_next));
   }
 }
 
@@ -611,6 +621,44 @@ __global__ void decode_advance_kernel(int B, int* __restrict__ step_counter, con
   if (b == 0) *step_counter = k + 1;
 }
 
+// The same, and where the next token's keys go in up to kMaxSlotGroups cache groups (what decode_slots_kernel
+// computes, for every group, from the positions just moved on): one launch between two decode steps instead of one
+// and one per group.
+constexpr int kMaxSlotGroups = 4;
+struct SlotGroups {
+  const int* table[kMaxSlotGroups];
+  int table_stride[kMaxSlotGroups];
+  int64_t* slot_mapping[kMaxSlotGroups];
+  int count, page_size;
+};
+__global__ void decode_advance_slots_kernel(int B, int* __restrict__ step_counter, const int* __restrict__ sampled_tokens,
+                                            const float* __restrict__ sampled_logprobs, int* __restrict__ tokens_in,
+                                            int* __restrict__ positions, int* __restrict__ seq_meta,
+                                            int* __restrict__ draw_counters, int* __restrict__ out_tokens,
+                                            float* __restrict__ out_logprobs, int max_steps,
+                                            const int* __restrict__ token_seq, SlotGroups groups) {
+  const int b = threadIdx.x;
+  const int k = *step_counter;
+  __syncthreads();
+  if (b < B) {
+    if (k < max_steps) {
+      out_tokens[static_cast<size_t>(k) * B + b] = sampled_tokens[b];
+      out_logprobs[static_cast<size_t>(k) * B + b] = sampled_logprobs[b];
+    }
+    tokens_in[b] = sampled_tokens[b];
+    const int pos = positions[b] + 1;
+    positions[b] = pos;
+    seq_meta[4 * b + 3] += 1;
+    draw_counters[b] += 1;
+    const int row = token_seq[b];
+    for (int g = 0; g < groups.count; ++g) {
+      const int page = groups.table[g][static_cast<size_t>(row) * groups.table_stride[g] + pos / groups.page_size];
+      groups.slot_mapping[g][b] = static_cast<int64_t>(page) * groups.page_size + pos % groups.page_size;
+    }
+  }
+  if (b == 0) *step_counter = k + 1;
+}
+
 // slot_mapping[b] = where the key of token b goes: page (from its request's block-table row) * page_size + offset
 __global__ void decode_slots_kernel(int B, const int* __restrict__ positions, const int* __restrict__ token_seq,
                                     const int* __restrict__ block_table, int table_stride, int page_size,
@@ -690,8 +738,23 @@ extern "C" int sa_add_rmsnorm(const void* y, int y_dtype, const void* w_post, in
   }
   add_rmsnorm_kernel<<<T, row_threads(D), 0, stream>>>(y, y_dtype, w_post, w_post_dtype, eps_post,
                                                        plus_one_post ? 1.f : 0.f, residual, w_next, w_next_dtype,
-                                                       eps_next, plus_one_next ? 1.f : 0.f, out, out_dtype, D);
+                                                       eps_next, plus_one_next ? 1.f : 0.f, out, out_dtype, D, nullptr);
   return check_launch("add_rmsnorm");
+}
+
+extern "C" int sa_add_rmsnorm_rows(const void* y, int y_dtype, const void* w_post, int w_post_dtype, float eps_post,
+                                   int plus_one_post, const float* residual, const void* w_next, int w_next_dtype,
+                                   float eps_next, int plus_one_next, void* out, int out_dtype, const int* index, int R,
+                                   int D, hipStream_t stream) {
+  if (R == 0) return 0;
+  SA_REQUIRE(R > 0 && D > 0 && index != nullptr && w_next != nullptr && out != nullptr && y != nullptr &&
+                 residual != nullptr,
+             "add_rmsnorm_rows: bad arguments (R=%d D=%d)", R, D);
+  add_rmsnorm_kernel<<<R, row_threads(D), 0, stream>>>(y, y_dtype, w_post, w_post_dtype, eps_post,
+                                                       plus_one_post ? 1.f : 0.f, const_cast<float*>(residual), w_next,
+                                                       w_next_dtype, eps_next, plus_one_next ? 1.f : 0.f, out,
+                                                       out_dtype, D, index);
+  return check_launch("add_rmsnorm_rows");
 }
 
 extern "C" int sa_add_rmsnorm_planes(const float* y_planes, int planes, const void* w_post, int w_post_dtype,
@@ -846,6 +909,33 @@ extern "C" int sa_decode_advance(int B, int* step_counter, const int* sampled_to
                                                    positions, seq_meta, draw_counters, out_tokens, out_logprobs,
                                                    max_steps);
   return check_launch("decode_advance");
+}
+
+extern "C" int sa_decode_advance_slots(int B, int* step_counter, const int* sampled_tokens, const float* sampled_logprobs,
+                                       int* tokens_in, int* positions, int* seq_meta, int* draw_counters, int* out_tokens,
+                                       float* out_logprobs, int max_steps, const int* token_seq, int num_groups,
+                                       const int* const* block_tables, const int* table_strides,
+                                       int64_t* const* slot_mappings, int page_size, hipStream_t stream) {
+  if (B == 0) return 0;
+  SA_REQUIRE(B > 0 && B <= 1024 && max_steps > 0, "decode_advance: 1..1024 requests and a positive number of steps");
+  SA_REQUIRE(num_groups >= 0 && num_groups <= kMaxSlotGroups && page_size > 0 && (num_groups == 0 || token_seq != nullptr),
+             "decode_advance_slots: 0..%d cache groups, a positive page size", kMaxSlotGroups);
+  SlotGroups groups{};
+  groups.count = num_groups;
+  groups.page_size = page_size;
+  for (int g = 0; g < num_groups; ++g) {
+    SA_REQUIRE(block_tables[g] != nullptr && slot_mappings[g] != nullptr && table_strides[g] > 0,
+               "decode_advance_slots: group %d lacks a table or a slot mapping", g);
+    groups.table[g] = block_tables[g];
+    groups.table_stride[g] = table_strides[g];
+    groups.slot_mapping[g] = slot_mappings[g];
+  }
+  int threads = 64;
+  while (threads < B) threads *= 2;
+  decode_advance_slots_kernel<<<1, threads, 0, stream>>>(B, step_counter, sampled_tokens, sampled_logprobs, tokens_in,
+                                                         positions, seq_meta, draw_counters, out_tokens, out_logprobs,
+                                                         max_steps, token_seq, groups);
+  return check_launch("decode_advance_slots");
 }
 
 extern "C" int sa_decode_slots(int B, const int* positions, const int* token_seq, const int* block_table,

@@ -231,11 +231,14 @@ class Executor:
         def one_step():
             logits = self.model.forward(dev[:T], ctx, self.cache.views, logit_rows, logits_out=shared)
             toks, lps = sampler.launch(logits)
+            groups = [(ctx.groups[g.group_id].block_table, ctx.groups[g.group_id].slot_mapping) for g in self.cache.groups]
+            # what was drawn becomes the next step's input, positions move on, and every cache group learns where
+            # the next keys go: one launch for up to four groups
             ops.decode_advance(counter, toks, lps, dev[:T], dev[cap:cap + T], ctx.seq_meta, sampler.draw_counters,
-                               out_tok, out_lp)
-            for g in self.cache.groups:
-                ops.decode_slots(dev[cap:cap + T], dev[2 * cap:2 * cap + T], ctx.groups[g.group_id].block_table,
-                                 self.cache.page_size, ctx.groups[g.group_id].slot_mapping)
+                               out_tok, out_lp, token_seq=dev[2 * cap:2 * cap + T], page_size=self.cache.page_size,
+                               groups=groups[:4])
+            for table, slots in groups[4:]:
+                ops.decode_slots(dev[cap:cap + T], dev[2 * cap:2 * cap + T], table, self.cache.page_size, slots)
 
         ops.fill_(counter, 0)
         key = ("many", B, self._context_bucket(ctx, num_steps - 1), max_steps, id(sampler), sampler.modes)

@@ -26,6 +26,8 @@ _SIGNATURES = {
     "sa_embed": [_P, _I, _P, _P, _I, _I, _I, _F, _I, _P],
     "sa_rmsnorm": [_P, _I, _L, _P, _I, _P, _I, _L, _I, _I, _F, _I, _P],
     "sa_add_rmsnorm": [_P, _I, _P, _I, _F, _I, _P, _P, _I, _F, _I, _P, _I, _I, _I, _P],
+    "sa_add_rmsnorm_rows": [_P, _I, _P, _I, _F, _I, _P, _P, _I, _F, _I, _P, _I, _P, _I, _I, _P],
+    "sa_decode_advance_slots": [_I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _P],
     "sa_rope_cache_write": [_P, _I, _L, _P, _P, _F, _F, _P, _P, _P, _I, _I, _I, _I, _I, _P],
     "sa_rope_cache_write_planes": [_P, _I, _P, _L, _P, _P, _F, _F, _P, _P, _P, _I, _I, _I, _I, _I, _P],
     "sa_rope": [_P, _I, _L, _P, _P, _F, _F, _I, _I, _I, _P],

@@ -186,6 +186,30 @@ def add_rmsnorm(y: "torch.Tensor | PartialSums", residual: torch.Tensor, *, post
     return out
 
 
+def add_rmsnorm_rows(y: torch.Tensor, residual: torch.Tensor, index: torch.Tensor, *, post_weight: torch.Tensor | None,
+                     post_eps: float = 0.0, post_plus_one: bool = True, next_weight: torch.Tensor, next_eps: float,
+                     next_plus_one: bool = True, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """out[r] = norm(residual[index[r]] + norm(y[index[r]]; post_weight); next_weight), the residual left as it is:
+    `add_rmsnorm` followed by a gather of the rows that are wanted, in one kernel that touches those rows only."""
+    _dev(y, residual, index, post_weight, next_weight)
+    T, D = residual.shape
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("add_rmsnorm_rows: the residual stream must be contiguous float32")
+    if tuple(y.shape) != (T, D) or not y.is_contiguous():
+        raise KernelError(f"add_rmsnorm_rows: y {tuple(y.shape)} does not match the residual {T, D}")
+    for w in (post_weight, next_weight):
+        if w is not None and (w.numel() != D or not w.is_contiguous()):
+            raise KernelError("add_rmsnorm_rows: a norm weight does not match the width")
+    _i32(index, "add_rmsnorm_rows: index")
+    R = index.numel()
+    out = torch.empty((R, D), dtype=out_dtype or y.dtype, device=y.device)
+    _lib.call("sa_add_rmsnorm_rows", _ptr(y), _code(y), _ptr(post_weight),
+              _code(post_weight) if post_weight is not None else 0, float(post_eps), int(post_plus_one), _ptr(residual),
+              _ptr(next_weight), _code(next_weight), float(next_eps), int(next_plus_one), _ptr(out), _code(out),
+              _ptr(index), R, D, _stream())
+    return out
+
+
 def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtype, what: str) -> int:
     """Key pages [pages, K, page_size, hd], value pages [pages, K, hd, page_size]; returns page_size."""
     if k_pages.dim() != 4 or v_pages.dim() != 4 or not k_pages.is_contiguous() or not v_pages.is_contiguous() \
@@ -284,10 +308,14 @@ def fill_(t: torch.Tensor, value_bits: int = 0) -> None:
 
 def decode_advance(step_counter: torch.Tensor, sampled_tokens: torch.Tensor, sampled_logprobs: torch.Tensor,
                    tokens_in: torch.Tensor, positions: torch.Tensor, seq_meta: torch.Tensor,
-                   draw_counters: torch.Tensor, out_tokens: torch.Tensor, out_logprobs: torch.Tensor) -> None:
+                   draw_counters: torch.Tensor, out_tokens: torch.Tensor, out_logprobs: torch.Tensor, *,
+                   token_seq: torch.Tensor | None = None, page_size: int = 0,
+                   groups: "list[tuple[torch.Tensor, torch.Tensor]] | None" = None) -> None:
     """Between two decode steps that the host does not see: what was drawn is recorded as row step_counter[0] of
     out_tokens / out_logprobs [max_steps, B] and becomes the next step's input; positions, the requests' first
-    positions (seq_meta[:, 3]), their draw counters and the step counter go up by one."""
+    positions (seq_meta[:, 3]), their draw counters and the step counter go up by one.  groups: (block table, slot
+    mapping) of up to four cache groups, whose slot mappings are set for the new positions in the same launch (what
+    `decode_slots` does for one group): needs token_seq and page_size."""
     _dev(step_counter, sampled_tokens, sampled_logprobs, tokens_in, positions, seq_meta, draw_counters, out_tokens,
          out_logprobs)
     B = tokens_in.numel()
@@ -304,6 +332,25 @@ def decode_advance(step_counter: torch.Tensor, sampled_tokens: torch.Tensor, sam
     if min(sampled_tokens.numel(), sampled_logprobs.numel(), positions.numel(), draw_counters.numel()) < B \
             or seq_meta.numel() < 4 * B or step_counter.numel() < 1:
         raise KernelError("decode_advance: an array is shorter than the number of requests")
+    if groups:
+        if token_seq is None or page_size < 1 or len(groups) > 4:
+            raise KernelError("decode_advance: slot mappings need token_seq, a page size and at most four groups")
+        _i32(token_seq, "decode_advance: token_seq", B)
+        n = len(groups)
+        for table, slots in groups:
+            _dev(table, slots)
+            if table.dim() != 2 or table.dtype != torch.int32 or table.stride(1) != 1:
+                raise KernelError("decode_advance: a block table must be int32 [sequences, blocks]")
+            if slots.dtype != torch.int64 or slots.numel() < B or not slots.is_contiguous():
+                raise KernelError("decode_advance: a slot mapping must be contiguous int64 with one entry per token")
+        tables = (ctypes.c_void_p * n)(*[t.data_ptr() for t, _ in groups])
+        strides = (ctypes.c_int * n)(*[t.stride(0) for t, _ in groups])
+        mappings = (ctypes.c_void_p * n)(*[m.data_ptr() for _, m in groups])
+        _lib.call("sa_decode_advance_slots", B, _ptr(step_counter), _ptr(sampled_tokens), _ptr(sampled_logprobs),
+                  _ptr(tokens_in), _ptr(positions), _ptr(seq_meta), _ptr(draw_counters), _ptr(out_tokens),
+                  _ptr(out_logprobs), out_tokens.shape[0], _ptr(token_seq), n, tables, strides, mappings, int(page_size),
+                  _stream())
+        return
     _lib.call("sa_decode_advance", B, _ptr(step_counter), _ptr(sampled_tokens), _ptr(sampled_logprobs), _ptr(tokens_in),
               _ptr(positions), _ptr(seq_meta), _ptr(draw_counters), _ptr(out_tokens), _ptr(out_logprobs),
               out_tokens.shape[0], _stream())

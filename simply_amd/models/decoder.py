@@ -112,9 +112,12 @@ class DecoderModel:
             block = self.layers[entry.layer]
             nxt = self.layers[schedule[i + 1].layer].first_norm() if i + 1 < len(schedule) else None
             h, normed = block.forward(h, ctx, cache_views[i], normed, nxt)
-        if isinstance(normed, PendingNorm):
-            h = normed.settle()      # the last block's residual sum, if it is still pending
         if logit_rows is None or logit_rows.numel() == 0:
             return None
+        if isinstance(normed, PendingNorm):
+            # the last block's residual sum is still pending: the final norm of the wanted rows comes out of the
+            # same kernel (the residual stream itself is of no use to anyone after the last block)
+            pending = PendingNorm(normed.residual, normed.y, normed.post_norm, self.final_norm, ctx.dtype)
+            return self.head.forward(pending.rows_through(logit_rows), out=logits_out)
         rows = ops.gather_rows(h, logit_rows)
         return self.head.forward(PendingNorm(rows, None, None, self.final_norm, ctx.dtype), out=logits_out)

@@ -140,6 +140,25 @@ class PendingNorm:
             self.y = None
         return self.residual
 
+    def rows_through(self, rows: torch.Tensor) -> torch.Tensor:
+        """next_norm of the rows `rows` (int32 indices) of the pending sum, for a consumer that needs those rows only
+        and nothing of the residual stream afterwards (the head at a model's end): one kernel over those rows where
+        the norms can, else the sum, a gather and the norm."""
+        from ..kernels import ops
+
+        if self.next_norm is None:
+            raise ValueError("a pending sum without a following norm has no activations")
+        pn, nn = self.post_norm, self.next_norm
+        if (self.y is not None and isinstance(self.y, torch.Tensor) and self.y.is_cuda and self.y.is_contiguous()
+                and getattr(nn, "fusable_rms", False) and (pn is None or getattr(pn, "fusable_rms", False))):
+            y, self.y = self.y, None
+            return ops.add_rmsnorm_rows(y, self.residual, rows, post_weight=pn.scale if pn is not None else None,
+                                        post_eps=pn.eps if pn is not None else 0.0,
+                                        post_plus_one=pn.scale_plus_one if pn is not None else True,
+                                        next_weight=nn.scale, next_eps=nn.eps, next_plus_one=nn.scale_plus_one,
+                                        out_dtype=self.dtype)
+        return nn.forward(ops.gather_rows(self.settle(), rows), self.dtype)
+
     def materialize(self) -> torch.Tensor:
         """The activations, computed with the separate kernels."""
         if self.next_norm is None:

@@ -1051,3 +1051,59 @@ def test_deferred_sum_of_the_projection_is_added_up_by_the_rotary_kernel(T, H, K
     assert torch.equal(q0, q1) and torch.equal(k0, k1) and torch.equal(v0, v1)
     if (T, hd) == (64, 256):
         assert cut   # this size does cut K
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,D,R", [(5, 100, 3), (16, 2304, 16), (9, 4608, 1), (40, 6000, 7), (3, 48, 3)])
+def test_add_rmsnorm_rows(dtype, T, D, R):
+    """The final norm of the rows whose logits are wanted, with the last residual sum, in one kernel: equals the sum
+    over all rows, a gather and the norm; the residual stream is left as it was."""
+    from simply_amd.kernels import ops
+    y = rand((T, D), dtype, 150, 2.0)
+    h = rand((T, D), torch.float32, 151, 5.0)
+    w1, w2 = rand((D,), dtype, 152, 0.3), rand((D,), dtype, 153, 0.3)
+    index = torch.randperm(T)[:R].to(torch.int32).cuda()
+    for with_post in (True, False):
+        h_ref = h.clone()
+        ref.add_rmsnorm(y, h_ref, post_weight=w1 if with_post else None, post_eps=1e-6)
+        want = ref.rmsnorm(h_ref[index.long()], w2, 1e-5, True, dtype)
+        before = h.clone()
+        got = ops.add_rmsnorm_rows(y, h, index, post_weight=w1 if with_post else None, post_eps=1e-6, next_weight=w2,
+                                   next_eps=1e-5, out_dtype=dtype)
+        assert torch.equal(h, before)
+        check(got.float(), want.float(), **tol(dtype))
+
+
+def test_decode_advance_with_slots():
+    """Between two decode steps on the device: tokens handed on, positions and counters moved, and the slot of the
+    next key in every cache group, in one launch: equals the separate kernels."""
+    from simply_amd.kernels import ops
+    B, P, steps = 5, 16, 4
+    g = torch.Generator().manual_seed(9)
+    positions = torch.tensor([15, 16, 0, 31, 100], dtype=torch.int32).cuda()
+    token_seq = torch.tensor([3, 0, 4, 1, 2], dtype=torch.int32).cuda()
+    tables = [torch.randint(0, 50, (6, 9), generator=g, dtype=torch.int32).cuda() for _ in range(3)]
+
+    def state():
+        return dict(counter=torch.zeros(1, dtype=torch.int32).cuda(), tokens_in=torch.zeros(B, dtype=torch.int32).cuda(),
+                    positions=positions.clone(), meta=torch.arange(4 * B, dtype=torch.int32).reshape(B, 4).cuda().contiguous(),
+                    draws=torch.arange(B, dtype=torch.int32).cuda(), out_tok=torch.zeros((steps, B), dtype=torch.int32).cuda(),
+                    out_lp=torch.zeros((steps, B)).cuda(), slots=[torch.zeros(B, dtype=torch.int64).cuda() for _ in tables])
+
+    a, b = state(), state()
+    for k in range(3):
+        toks = torch.randint(0, 1000, (B,), generator=g, dtype=torch.int32).cuda()
+        lps = torch.randn(B, generator=g).cuda()
+        ops.decode_advance(a["counter"], toks, lps, a["tokens_in"], a["positions"], a["meta"], a["draws"], a["out_tok"],
+                           a["out_lp"])
+        for t, s in zip(tables, a["slots"]):
+            ops.decode_slots(a["positions"], token_seq, t, P, s)
+        ops.decode_advance(b["counter"], toks, lps, b["tokens_in"], b["positions"], b["meta"], b["draws"], b["out_tok"],
+                           b["out_lp"], token_seq=token_seq, page_size=P, groups=list(zip(tables, b["slots"])))
+        for name in ("counter", "tokens_in", "positions", "meta", "draws", "out_tok", "out_lp"):
+            assert torch.equal(a[name], b[name]), (k, name)
+        for s1, s2, t in zip(a["slots"], b["slots"], tables):
+            assert torch.equal(s1, s2)
+            pos = b["positions"].long()
+            assert torch.equal(s2, t[token_seq.long(), pos // P].long() * P + pos % P)
+    assert int(b["counter"]) == 3 and torch.equal(b["positions"], positions + 3)
