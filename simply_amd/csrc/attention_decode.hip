@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     float* __restrict__ workspace) {
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;  // output blocks of 16 dimensions
-  __shared__ float o_s[2][16][HD + 1];   // a wave's output [row][d], while two waves are merged
+  __shared__ __align__(16) float o_s[2][16][HD + 4];   // a wave's output [row][d], while two waves are merged (rows of 16-byte pieces)
   __shared__ float m_s[2][16], l_s[2][16];
   __shared__ int2 where_s[kMaxRangeSubTiles];  // per sub-tile of this workgroup's range: its page, its block within it
 
@@ -77,12 +77,23 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   // of 16.)  The host cuts the keys so that a range fits one pass; a range that is longer all the same (a caller
   // that understates max_kv_len) takes further passes, each with its own look-up, instead of reading beyond the
   // array.
+  // (the queries are asked for first: their load is under way during the look-up)
+  // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
+  bf16x8 qf[NDC];
+  {
+    const bf16* qp = q + static_cast<size_t>(sm.q_start + (row_ok ? qi : 0)) * q_stride +
+                     static_cast<size_t>(kh * G + (row_ok ? g : 0)) * HD + grp * 8;
+#pragma unroll
+    for (int dc = 0; dc < NDC; ++dc)
+      qf[dc] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + dc * 32) : bf16x8{};
+  }
   constexpr int kPassTiles = kMaxRangeSubTiles / 2;
   int pass_b = tb;                                        // this pass covers tiles [pass_b, pass_e)
   int pass_e = te - tb > kPassTiles ? tb + kPassTiles : te;
   int sub0 = 2 * pass_b;
   auto look_up = [&]() {
-    const int nsub = 2 * (pass_e - pass_b);
+    // (at least the first entry is written, also for a range without tiles: loads that are not needed go there)
+    const int nsub = pass_e > pass_b ? 2 * (pass_e - pass_b) : 1;
     for (int i = tid; i < nsub; i += 256) {
       const int key = (sub0 + i) * 16;
       int2 w = {0, 0};
@@ -96,16 +107,6 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     __syncthreads();
   };
   look_up();
-
-  // Q as B operands: lane (row r, grp) holds Q[row r][dc * 32 + grp * 8 .. + 8]
-  bf16x8 qf[NDC];
-  {
-    const bf16* qp = q + static_cast<size_t>(sm.q_start + (row_ok ? qi : 0)) * q_stride +
-                     static_cast<size_t>(kh * G + (row_ok ? g : 0)) * HD + grp * 8;
-#pragma unroll
-    for (int dc = 0; dc < NDC; ++dc)
-      qf[dc] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + dc * 32) : bf16x8{};
-  }
 
   floatx4 acc[NDB];
 #pragma unroll
@@ -125,13 +126,16 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     SubTile st;
     const int sk0 = tile * kTile + t * 16;
     st.ok = tile < pass_e && sk0 < hi && sk0 + 16 > lo;  // wave-uniform
-    // A sub-tile outside the range is loaded all the same, from the pool's first page: every load of the loop is
-    // unconditional, the loop straight-line code, and the compiler counts the loads in flight (with a branch
-    // around a load it waits for all of them, and loads and products do not overlap).  What is loaded there is
-    // never used: its scores are masked and its values replaced by zeros.
+    // A sub-tile outside the range is loaded all the same, from where this pass's first sub-tile lies: every load of
+    // the loop is unconditional, the loop straight-line code, and the compiler counts the loads in flight (with a
+    // branch around a load it waits for all of them, and loads and products do not overlap).  What is loaded there
+    // is never used: its scores are masked and its values replaced by zeros.  (Not from one place for everybody,
+    // such as the pool's first page: with a tile or two to a wave, as for a single request, every wave of the GPU
+    // has such loads, and a thousand waves on the same sixteen KiB queue up at its few channels of L2; a
+    // workgroup's own first sub-tile is in its CU's cache.)
     const int2 w = where_s[st.ok ? 2 * tile + t - sub0 : 0];
-    const size_t head = st.ok ? static_cast<size_t>(w.x) * Kh + kh : 0;
-    const int blk = st.ok ? w.y : 0;
+    const size_t head = static_cast<size_t>(w.x) * Kh + kh;
+    const int blk = w.y;
     // keys are stored in 16-key x 32-dimension blocks of operand order: block (blk, dc) is a contiguous KiB
     st.k = k_pages + head * page_size * HD + static_cast<size_t>(blk) * (NDC * 512) + lane * 8;
     st.v = v_pages + (head * HD + r) * page_size + blk * 16 + grp * 4;
@@ -254,25 +258,29 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   // ---- merge the four waves in two rounds through LDS (waves 2, 3 into 0, 1; then 1 into 0).
   // acc[db][v] is O^T[d = db * 16 + 4 * grp + v][row r].
   l_run = sum_over_row_lanes(l_run);
+  // (acc[db] is four consecutive dimensions: one 16-byte piece of LDS; rows beyond the request's hold nothing)
   auto put = [&](int slot) {
+    if (row_ok) {
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) o_s[slot][r][db * 16 + 4 * grp + v] = acc[db][v];
-    if (grp == 0) {
-      m_s[slot][r] = m_run;
-      l_s[slot][r] = l_run;
+      for (int db = 0; db < NDB; ++db) *reinterpret_cast<floatx4*>(&o_s[slot][r][db * 16 + 4 * grp]) = acc[db];
+      if (grp == 0) {
+        m_s[slot][r] = m_run;
+        l_s[slot][r] = l_run;
+      }
     }
   };
   auto take = [&](int slot) {
+    if (!row_ok) return;
     const float m_o = m_s[slot][r], l_o = l_s[slot][r];
     const float M = fmaxf(m_run, m_o);
     const float a = m_run == -INFINITY ? 0.f : __expf(m_run - M);
     const float b = m_o == -INFINITY ? 0.f : __expf(m_o - M);
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+    for (int db = 0; db < NDB; ++db) {
+      const floatx4 o = *reinterpret_cast<const floatx4*>(&o_s[slot][r][db * 16 + 4 * grp]);
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[db][v] = acc[db][v] * a + o_s[slot][r][db * 16 + 4 * grp + v] * b;
+      for (int v = 0; v < 4; ++v) acc[db][v] = acc[db][v] * a + o[v] * b;
+    }
     l_run = l_run * a + l_o * b;
     m_run = M;
   };
