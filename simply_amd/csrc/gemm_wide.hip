@@ -13,9 +13,11 @@
 //   * Schedule of a wave: the fragments of the two halves of a slab have registers of their own; the products of
 //     the second half are held back until after the next barrier, where they cover the fragment reads of the next
 //     slab's first half, and the reads of the second half are covered by the products of the first: between two
-//     barriers the MFMA unit always has products to do.  The loads of the slab one or two ahead are spread over
-//     the products, one after each row of them: issued together after the barrier, the eight waves queue up at
-//     the memory pipeline (16 cycles a load) while the MFMA unit idles.
+//     barriers the MFMA unit always has products to do.  On the larger tiles the reads are issued one by one
+//     between those products (a wave issues in order: many reads in a row keep its products back).  The loads of
+//     the slab one or two ahead are spread over the products, one after every few: issued together after the
+//     barrier, the waves queue up at the memory pipeline (16 cycles a load) while the MFMA unit idles; with two
+//     buffers they all go out in the first half of a slab, so that the second half covers the last one's way.
 //   * The products are taken transposed (W fragment as the first operand), so that a lane holds four neighbouring
 //     columns of one row of C and stores them as one 8-byte piece.
 //
@@ -169,23 +171,46 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
     for (int j = 0; j < WN; ++j)
       fw[kc][j] = *reinterpret_cast<const bf16x8*>(stage + ((A_BLOCKS + (wn * WN + j) * 2 + kc) * 64 + lane) * 8);
   };
-  // The products of half kc; after each row of them the next PER_ROW loads of slab `slab`, from load `first` on, are
-  // asked for (if there are any left): the loads of a slab are spread over its products, so that the waves do not
-  // queue up at the memory pipeline (which takes 16 cycles for each) while the MFMA unit idles.
-  constexpr int PER_ROW = (LOADS + 2 * WM - 1) / (2 * WM);
-  auto multiply = [&](int kc, int first, int slab, int buf) __attribute__((always_inline)) {
+  // fragment n of half kc alone: W's first (the first row of products needs them all), then A's
+  auto read_one = [&](const __bf16* stage, int kc, int n) __attribute__((always_inline)) {
+    if (n < WN)
+      fw[kc][n] = *reinterpret_cast<const bf16x8*>(stage + ((A_BLOCKS + (wn * WN + n) * 2 + kc) * 64 + lane) * 8);
+    else
+      fa[kc][n - WN] = *reinterpret_cast<const bf16x8*>(stage + (wm * WM + n - WN) * 1024 + a_frag[kc]);
+  };
+  // Tiles with enough products read the fragments of the other half one by one, each after one of the first
+  // products of this half, instead of all of them before: a wave issues in order, and sixteen reads in a row keep
+  // its products from the MFMA unit for a few hundred cycles.
+  constexpr bool INTERLEAVED = WM * WN >= 2 * (WM + WN);
+  // The products of half kc (`first`: 0 for the held-back half, which comes first after the barrier; 1 for the
+  // other; -1: no loads).  After every EVERY products, counted through the slab, one load of slab `slab` is asked
+  // for: spread out, so that the waves do not queue up at the memory pipeline (which takes 16 cycles for each) while
+  // the MFMA unit idles, and early: with two buffers all of them among the first half's products, so that the
+  // second half's cover the time that the last one takes.
+  constexpr int SPAN = NSTAGE == 2 ? WM * WN : 2 * WM * WN;
+  constexpr int EVERY = SPAN / LOADS > 0 ? SPAN / LOADS : 1;
+  constexpr int PER = SPAN / LOADS > 0 ? 1 : (LOADS + SPAN - 1) / SPAN;  // (small tiles: several loads after each product)
+  auto multiply = [&](int kc, int first, int slab, int buf, const __bf16* rstage = nullptr, int rkc = -1)
+                      __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
+      for (int j = 0; j < WN; ++j) {
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kc][j], fa[kc][i], acc[i][j], 0, 0, 0);
+        if (INTERLEAVED && rkc >= 0 && i * WN + j < WM + WN) {
+          __builtin_amdgcn_sched_barrier(0);
+          read_one(rstage, rkc, i * WN + j);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        const int q = (first > 0 ? WM * WN : 0) + i * WN + j + 1;  // products of this slab so far
 #pragma unroll
-      for (int e = 0; e < PER_ROW; ++e) {
-        const int n = first + i * PER_ROW + e;
-        if (first >= 0 && n < LOADS) {
-          __builtin_amdgcn_sched_barrier(0);
-          request_one(n, slab, buf);
-          __builtin_amdgcn_sched_barrier(0);
+        for (int e = 0; e < PER; ++e) {
+          const int n = (q / EVERY - 1) * PER + e;
+          if (first >= 0 && q % EVERY == 0 && n < LOADS) {
+            __builtin_amdgcn_sched_barrier(0);
+            request_one(n, slab, buf);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
     }
@@ -212,13 +237,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
     bare_barrier();
     const int ahead = s + NSTAGE - 1 < slabs ? s + NSTAGE - 1 : slabs - 1;
     const __bf16* stage = stages + cur * STAGE;
-    read(stage, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(1, 0, ahead, target);
-    __builtin_amdgcn_sched_barrier(0);  // (reads moved up among these products would need registers of their own)
-    read(stage, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(0, WM * PER_ROW, ahead, target);
+    if (INTERLEAVED) {
+      multiply(1, 0, ahead, target, stage, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(0, 1, ahead, target, stage, 1);
+    } else {
+      read(stage, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(1, 0, ahead, target);
+      __builtin_amdgcn_sched_barrier(0);  // (reads moved up among these products would need registers of their own)
+      read(stage, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(0, 1, ahead, target);
+    }
     target = cur;
     cur = cur + 1 == NSTAGE ? 0 : cur + 1;
   }
