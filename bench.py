@@ -303,6 +303,46 @@ def run_products(which: str):
         torch.cuda.empty_cache()
 
 
+def measure_ceilings():
+    """What this GPU reaches by itself, with the library's two probe kernels: reading HBM with all CUs (2 GiB,
+    contiguously and in shuffled 8 KiB pieces, as a cache's pages lie) and retiring bfloat16 MFMA instructions
+    (operands of zeros, and of random values: the clock held under that load depends on the bits that toggle).
+    The decode step's kernels cannot read faster than the first, the prompt's products cannot multiply faster than
+    the last; the published peaks are higher than both."""
+    import torch
+    from simply_amd.kernels import ops
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(reps):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            fn()
+            end.record()
+            torch.cuda.synchronize()
+            best = min(best, start.elapsed_time(end) * 1e-3)
+        return best
+
+    nbytes = 2 << 30
+    buffer = torch.zeros(nbytes // 4, dtype=torch.float32, device="cuda:0")
+    order = torch.randperm(nbytes // 8192, device="cuda:0").to(torch.int32)
+    out = {"hbm_read_gbps": round(nbytes / timed(lambda: ops.probe_hbm_read(buffer), 5) / 1e9, 1),
+           "hbm_read_8k_pieces_gbps": round(nbytes / timed(lambda: ops.probe_hbm_read(buffer, order), 5) / 1e9, 1)}
+    del buffer, order
+    iters = 40000  # about 5 ms a launch: long enough for the clock to settle
+    for name, operands in (("zeros", torch.zeros(8192, dtype=torch.bfloat16, device="cuda:0")),
+                           ("random", (torch.rand(8192, device="cuda:0") - 0.5).to(torch.bfloat16))):
+        flops = [0.0]
+
+        def run():
+            flops[0] = ops.probe_mfma(operands, iters)
+        seconds = timed(run, 8)
+        out[f"mfma_bf16_{name}_tflops"] = round(flops[0] / seconds / 1e12, 1)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -318,9 +358,10 @@ def main():
     ap.add_argument("--batches", default="1,8,32,64", help="--only decode-grid: the batch sizes")
     ap.add_argument("--contexts", default="1024,4096,8192", help="--only decode-grid: the context lengths")
     ap.add_argument("--only", default="all", choices=["all", "decode", "decode-grid", "prefill", "prefill-chunked", "products",
-                                                      "gated-products"],
+                                                      "gated-products", "ceilings"],
                     help="measure one part alone (for profiles); the line then holds that part only.  products / "
-                         "gated-products: the sweep of the product kernels over rows and weight sizes")
+                         "gated-products: the sweep of the product kernels over rows and weight sizes; ceilings: "
+                         "what the GPU itself reaches in reading HBM and in bfloat16 MFMA instructions")
     ap.add_argument("--latency-steps", type=int, default=100,
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
@@ -340,6 +381,10 @@ def main():
     from simply_amd.kernels import lib
 
     lib.load()
+    if args.only == "ceilings":
+        print(json.dumps({"metric": "measured ceilings of this GPU", **measure_ceilings(),
+                          "published": {"hbm_gbps": HBM_GBPS, "mfma_bf16_tflops": PEAK_TFLOPS["bf16"]}}), flush=True)
+        return
     if args.only in ("products", "gated-products"):
         run_products("gated" if args.only == "gated-products" else "plain")
         return
@@ -450,6 +495,7 @@ def main():
                      "frac": round(achieved / HBM_GBPS, 4)},
         "points": points,
         "self_check": check,
+        "measured_ceilings": measure_ceilings(),
     }
     print(json.dumps(out), flush=True)
 

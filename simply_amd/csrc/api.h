@@ -214,6 +214,14 @@ int sa_score(const float* logits, int64_t row_stride, int R, int V, const float*
 
 // Host function: one block of the Philox4x32-10 generator that sa_sample uses.
 void sa_philox4x32_10(const uint32_t* counter4, const uint32_t* key2, uint32_t* out4);
+
+// Measurements of the machine (the caller times them).  All CUs read `bytes` (a multiple of 8 KiB) of `buffer` once,
+// in 8 KiB pieces in their natural order or in the order given (piece numbers, one per piece: the pages of a cache).
+// `sink` (512 floats) is never written in practice.
+int sa_probe_hbm_read(const void* buffer, int64_t bytes, const int* order, void* sink, hipStream_t stream);
+// `workgroups` workgroups of eight waves retire 16 * iters v_mfma_f32_16x16x32_bf16 per wave on operands taken from
+// the 16 KiB at `operands`: 2 * 16 * 16 * 32 * 16 * iters * 8 * workgroups floating-point operations.
+int sa_probe_mfma(const void* operands, int iters, int workgroups, void* sink, hipStream_t stream);
 }
 
 namespace sa {

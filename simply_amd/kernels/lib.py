@@ -53,6 +53,8 @@ _SIGNATURES = {
     "sa_gemm_normed_rotary": [_P, _P, _P, _P, _I, _F, _I, _P, _I, _F, _I, _P, _P, _I, _L, _I, _I, _P, _P, _F, _F, _P, _P,
                               _P, _I, _I, _I, _I, _P],
     "sa_score": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P],
+    "sa_probe_hbm_read": [_P, _L, _P, _P, _P],
+    "sa_probe_mfma": [_P, _I, _I, _P, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }
 

@@ -673,6 +673,35 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                             unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
 
 
+# --------------------------------------------------------------------------- measurements of the machine
+
+
+def probe_hbm_read(buffer: torch.Tensor, order: torch.Tensor | None = None) -> None:
+    """All CUs read `buffer` (whole 8 KiB pieces) once from memory, piece after piece or in the order given (int32
+    piece numbers): the caller times it.  What the decode step's kernels, which are bound by reading weights and
+    cache, can reach at most."""
+    _dev(buffer, order)
+    nbytes = buffer.numel() * buffer.element_size()
+    if not buffer.is_contiguous() or nbytes % 8192:
+        raise KernelError("probe_hbm_read: a contiguous buffer of whole 8 KiB pieces")
+    if order is not None:
+        _i32(order, "probe_hbm_read: order", nbytes // 8192)
+    sink = _workspace(buffer.device)
+    _lib.call("sa_probe_hbm_read", _ptr(buffer), nbytes, _ptr(order), _ptr(sink), _stream())
+
+
+def probe_mfma(operands: torch.Tensor, iters: int, workgroups: int = 256) -> float:
+    """`workgroups` workgroups of eight waves each retire 16 * iters bfloat16 MFMA instructions per wave on the
+    16 KiB of `operands`; returns the floating-point operations that this is (the caller times it).  The rate
+    depends on the operands' bits: the clock that the GPU holds under this load does."""
+    _dev(operands)
+    if operands.numel() * operands.element_size() < 16384 or not operands.is_contiguous():
+        raise KernelError("probe_mfma: 16 KiB of operands")
+    sink = _workspace(operands.device)
+    _lib.call("sa_probe_mfma", _ptr(operands), int(iters), int(workgroups), _ptr(sink), _stream())
+    return 2.0 * 16 * 16 * 32 * 16 * iters * 8 * workgroups
+
+
 # --------------------------------------------------------------------------- sampling
 
 

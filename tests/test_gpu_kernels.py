@@ -1107,3 +1107,22 @@ def test_decode_advance_with_slots():
             pos = b["positions"].long()
             assert torch.equal(s2, t[token_seq.long(), pos // P].long() * P + pos % P)
     assert int(b["counter"]) == 3 and torch.equal(b["positions"], positions + 3)
+
+
+def test_machine_probes_run_and_refuse():
+    """The two probe kernels (reading memory with all CUs, retiring MFMA instructions) run to their end, count the
+    work they are said to do, and refuse buffers that do not fit."""
+    from simply_amd.kernels import ops
+    from simply_amd.kernels.lib import KernelError
+    buffer = torch.ones(3 * 8192 // 4, dtype=torch.float32, device="cuda:0")  # three pieces: an odd count per wave
+    ops.probe_hbm_read(buffer)
+    ops.probe_hbm_read(buffer, torch.tensor([2, 0, 1], dtype=torch.int32, device="cuda:0"))
+    operands = torch.randn(8192, device="cuda:0").to(torch.bfloat16)
+    assert ops.probe_mfma(operands, 10, workgroups=4) == 2.0 * 16 * 16 * 32 * 16 * 10 * 8 * 4
+    torch.cuda.synchronize()
+    with pytest.raises(KernelError):
+        ops.probe_hbm_read(torch.ones(1000, dtype=torch.float32, device="cuda:0"))
+    with pytest.raises(KernelError):
+        ops.probe_hbm_read(buffer, torch.tensor([0, 1], dtype=torch.int32, device="cuda:0"))
+    with pytest.raises(KernelError):
+        ops.probe_mfma(operands[:100], 10)
