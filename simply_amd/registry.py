@@ -8,7 +8,29 @@ for an unknown name is an error that lists the known names.
 """
 from __future__ import annotations
 
+import importlib
+import os
 from typing import Any, Callable, Iterator
+
+#: environment variable naming modules (comma-separated, importable) that register architectures and parts of
+#: their own when they are imported: how a model that does not live in this package reaches the command line
+#: and `bin/trace_run`
+PLUGINS_ENV = "SIMPLY_AMD_PLUGINS"
+_plugins_loaded = False
+
+
+def load_plugins() -> None:
+    """Imports the modules that $SIMPLY_AMD_PLUGINS names, once.  A registry does it by itself before it calls a
+    name unknown."""
+    global _plugins_loaded
+    if _plugins_loaded:
+        return
+    _plugins_loaded = True
+    for module in filter(None, (m.strip() for m in os.environ.get(PLUGINS_ENV, "").split(","))):
+        try:
+            importlib.import_module(module)
+        except ImportError as exc:
+            raise ImportError(f"${PLUGINS_ENV} names the module {module!r}, which cannot be imported: {exc}") from exc
 
 
 class Registry:
@@ -35,6 +57,8 @@ class Registry:
         self._entries.pop(name, None)
 
     def get(self, name: str) -> Any:
+        if name not in self._entries:
+            load_plugins()
         try:
             return self._entries[name]
         except KeyError:
